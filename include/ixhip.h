@@ -1,0 +1,125 @@
+/*
+ * ixhip -- C ABI of the gfx950 (MI355X) INT8-X decode / fused decode+GEMV library.
+ *
+ * The library replaces the three Triton kernels of dfytensor/ixrun and the
+ * launch half of their Python wrappers.  Each entry point below names the
+ * reference interface it stands in for (file:line in the reference tree).
+ *
+ * Conventions
+ *   - every pointer inside IxhPacked and every buffer argument is a DEVICE
+ *     pointer owned by the caller; the library never allocates, frees, copies
+ *     to the host or synchronises, so every call may be stream-captured;
+ *   - all work is enqueued on the given stream (0 = the null stream);
+ *   - return value: IXH_OK (0) or a negative IXH_E* code; ixh_last_error()
+ *     gives the calling thread's last message.  Nothing throws or aborts;
+ *   - lengths of every stream are passed and respected: no kernel reads past
+ *     them, whatever the level counts are (empty levels are legal);
+ *   - int32 words of the reference's torch.int32 tensors are taken as raw
+ *     32-bit patterns.
+ */
+#ifndef IXHIP_H
+#define IXHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define IXH_MAX_LEVELS 8
+
+#define IXH_OK 0
+#define IXH_EINVAL (-1)       /* malformed argument (message says which) */
+#define IXH_EUNSUPPORTED (-2) /* valid request this build has no kernel for */
+#define IXH_ELAUNCH (-3)      /* the HIP runtime refused a launch */
+#define IXH_EWORKSPACE (-4)   /* workspace missing or too small */
+
+/* ixh_gemv flags */
+#define IXH_GEMV_ATOMIC 1u /* add fp32 partials into y32 with atomics (caller zeroes y32) */
+#define IXH_GEMV_FORCE_GENERIC 2u /* skip the (3,5,8) specialised kernels (testing / comparison) */
+
+typedef void *ixh_stream_t; /* a hipStream_t */
+
+/*
+ * One packed tensor: the device-resident fields of the dictionary written by
+ * the reference's int8x_quantize (ixrun/quantize.py:110-122).
+ *   level_bits  ascending code widths, last one 8 (quantize.py:55-58)
+ *   bitmaps[i]  nested bitmap i, i < n_levels-1, 1 bit per element not in a
+ *               lower level (quantize.py:91-96), LSB-first 32-bit words
+ *   streams[i]  level-i codes, level_bits[i] bits each, LSB-first across
+ *               32-bit words (bitpack.py:13-61), i < n_levels-1
+ *   last        raw bytes of the 8-bit last level (quantize.py:84-86)
+ *   scale       the bf16 per-tensor scale, read on the device
+ */
+typedef struct IxhPacked {
+    int32_t n_levels;
+    int32_t level_bits[IXH_MAX_LEVELS];
+    int64_t out_f;
+    int64_t in_f;
+    const uint32_t *bitmaps[IXH_MAX_LEVELS - 1];
+    uint64_t bitmap_words[IXH_MAX_LEVELS - 1];
+    const uint32_t *streams[IXH_MAX_LEVELS - 1];
+    uint64_t stream_words[IXH_MAX_LEVELS - 1];
+    const uint8_t *last;
+    uint64_t last_bytes;
+    const uint16_t *scale;
+} IxhPacked;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int ixh_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char *ixh_last_error(void);
+
+/*
+ * Number of int32 entries per level of a prefix table with the given chunk:
+ * ceil(n / chunk) + 1.
+ */
+int64_t ixh_prefix_entries(int64_t n, int64_t chunk);
+
+/*
+ * Rank-prefix table, built on the device.
+ *   prefix[i * entries + u] = number of level-i elements with flat index
+ *   < min(u * chunk, N), for i < n_levels-1 and u = 0 .. entries-1.
+ * chunk = in_f reproduces compute_row_prefixes(packed) (ixrun/fused.py:60-65),
+ * a divisor of in_f reproduces compute_row_prefixes(packed, chunk)
+ * (ixrun/fused.py:67-78), chunk = 1024 reproduces precompute_block_offsets
+ * (ixrun/triton_kernels.py:180-220); the extra last entry holds the totals.
+ */
+int ixh_prefix_build(const IxhPacked *packed, int64_t chunk, int32_t *prefix, ixh_stream_t stream);
+
+/*
+ * Full decode: out_i8[p] = int8 value of flat element p (nullable),
+ * out_bf16[p] = bf16(f32(v) * f32(scale)) (nullable).  Replaces
+ * _ix_decode_kernel / decode_weight_triton (ixrun/triton_kernels.py:68-177,
+ * :224-259) and StreamingLinear._decode (ixrun/engine.py:109-133), for any
+ * level scheme.  prefix/chunk: a table from ixh_prefix_build; any chunk > 0.
+ */
+int ixh_decode(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, int8_t *out_i8,
+               uint16_t *out_bf16, ixh_stream_t stream);
+
+/*
+ * Fused decode + GEMV / skinny GEMM:
+ *   y[m, r] = bf16( sum_k f32(x[m, k]) * f32(bf16(f32(v[r, k]) * f32(scale))) ),
+ * fp32 accumulation, m < M <= 16; x is bf16 [M, ldx], y is bf16 [M, ldy].
+ * Replaces _ix_gemv_kernel / _ix_gemv_split_kernel / fused_gemv
+ * (ixrun/fused.py:84-179, :209-294, :297-347) for M = 1 and the decode +
+ * F.linear path of StreamingLinear.forward (ixrun/engine.py:171-173) for
+ * 2 <= M <= 16.  chunk must divide in_f; the table must come from
+ * ixh_prefix_build(packed, chunk).  Partial sums of the in_f / chunk chunks of
+ * a row are combined in a fixed order through `workspace`
+ * (ixh_gemv_workspace_bytes) and written to y, or, with IXH_GEMV_ATOMIC, added
+ * into the caller-zeroed fp32 y32 [M, out_f] with atomics as the reference's
+ * split kernel does (fused.py:294); y may then be NULL.
+ */
+int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, const uint16_t *x,
+             int32_t m, int64_t ldx, uint16_t *y, int64_t ldy, float *y32, void *workspace,
+             size_t workspace_bytes, uint32_t flags, ixh_stream_t stream);
+
+size_t ixh_gemv_workspace_bytes(const IxhPacked *packed, int64_t chunk, int32_t m, uint32_t flags);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* IXHIP_H */

@@ -1,0 +1,193 @@
+"""ctypes binding of ``libixhip.so`` (the C ABI declared in ``include/ixhip.h``).
+
+The library is built in-tree by ``csrc/build.sh``.  There is no CPU fallback:
+if the shared object is missing, or a call is made without a GPU tensor,
+loading or the call raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libixhip.so")
+
+IXH_MAX_LEVELS = 8
+IXH_GEMV_ATOMIC = 1
+IXH_GEMV_FORCE_GENERIC = 2
+
+ERROR_NAMES = {-1: "IXH_EINVAL", -2: "IXH_EUNSUPPORTED", -3: "IXH_ELAUNCH", -4: "IXH_EWORKSPACE"}
+
+
+class IxhPacked(C.Structure):
+    _fields_ = [
+        ("n_levels", C.c_int32),
+        ("level_bits", C.c_int32 * IXH_MAX_LEVELS),
+        ("out_f", C.c_int64),
+        ("in_f", C.c_int64),
+        ("bitmaps", C.c_void_p * (IXH_MAX_LEVELS - 1)),
+        ("bitmap_words", C.c_uint64 * (IXH_MAX_LEVELS - 1)),
+        ("streams", C.c_void_p * (IXH_MAX_LEVELS - 1)),
+        ("stream_words", C.c_uint64 * (IXH_MAX_LEVELS - 1)),
+        ("last", C.c_void_p),
+        ("last_bytes", C.c_uint64),
+        ("scale", C.c_void_p),
+    ]
+
+
+class IxhError(RuntimeError):
+    """A call into libixhip returned a negative code."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"{ERROR_NAMES.get(code, code)}: {message}")
+        self.code = code
+
+
+_lib = None
+
+EXPORTS = (
+    "ixh_version", "ixh_last_error", "ixh_prefix_entries", "ixh_prefix_build", "ixh_decode",
+    "ixh_gemv", "ixh_gemv_workspace_bytes",
+)
+
+
+def lib() -> C.CDLL:
+    """Load the library once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with ixrun_amd/csrc/build.sh "
+                "(hipcc --offload-arch=gfx950); there is no fallback path"
+            )
+        L = C.CDLL(LIB_PATH)
+        L.ixh_version.restype = C.c_int
+        L.ixh_last_error.restype = C.c_char_p
+        L.ixh_prefix_entries.restype = C.c_int64
+        L.ixh_prefix_entries.argtypes = [C.c_int64, C.c_int64]
+        L.ixh_prefix_build.restype = C.c_int
+        L.ixh_prefix_build.argtypes = [C.POINTER(IxhPacked), C.c_int64, C.c_void_p, C.c_void_p]
+        L.ixh_decode.restype = C.c_int
+        L.ixh_decode.argtypes = [C.POINTER(IxhPacked), C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.ixh_gemv.restype = C.c_int
+        L.ixh_gemv.argtypes = [
+            C.POINTER(IxhPacked), C.c_void_p, C.c_int64, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p,
+            C.c_int64, C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint32, C.c_void_p,
+        ]
+        L.ixh_gemv_workspace_bytes.restype = C.c_size_t
+        L.ixh_gemv_workspace_bytes.argtypes = [C.POINTER(IxhPacked), C.c_int64, C.c_int32, C.c_uint32]
+        _lib = L
+    return _lib
+
+
+def check(code: int) -> None:
+    if code != 0:
+        raise IxhError(code, lib().ixh_last_error().decode())
+
+
+def current_stream(device) -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _require_cuda(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{what} must live on the GPU (got {t.device}); the HIP path has no CPU fallback")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{what} must be contiguous")
+
+
+class DevicePacked:
+    """An ``IxhPacked`` built over device tensors that it keeps alive."""
+
+    def __init__(self, level_bits, out_f, in_f, bitmaps, streams, scale):
+        level_bits = tuple(int(b) for b in level_bits)
+        n_levels = len(level_bits)
+        if not 2 <= n_levels <= IXH_MAX_LEVELS:
+            raise ValueError(f"{n_levels} levels: the device path takes 2..{IXH_MAX_LEVELS}")
+        if len(bitmaps) != n_levels - 1 or len(streams) != n_levels:
+            raise ValueError("need one bitmap per level but the last and one stream per level")
+        self.level_bits, self.out_f, self.in_f = level_bits, int(out_f), int(in_f)
+        self.N = self.out_f * self.in_f
+        self.tensors = list(bitmaps) + list(streams) + [scale]
+        for i, t in enumerate(self.tensors):
+            _require_cuda(t, f"packed tensor {i}")
+        if scale.dtype != torch.bfloat16 or scale.numel() != 1:
+            raise ValueError("scale must be a one-element bf16 tensor")
+        self.device = scale.device
+        s = IxhPacked()
+        s.n_levels = n_levels
+        for i, b in enumerate(level_bits):
+            s.level_bits[i] = b
+        s.out_f, s.in_f = self.out_f, self.in_f
+        for i in range(n_levels - 1):
+            bm, st = bitmaps[i], streams[i]
+            if bm.dtype != torch.int32 or st.dtype != torch.int32:
+                raise ValueError("bitmaps and packed streams must be torch.int32")
+            s.bitmaps[i] = bm.data_ptr() if bm.numel() else None
+            s.bitmap_words[i] = bm.numel()
+            s.streams[i] = st.data_ptr() if st.numel() else None
+            s.stream_words[i] = st.numel()
+        last = streams[-1]
+        if last.dtype != torch.uint8:
+            raise ValueError("the last stream must be torch.uint8")
+        s.last = last.data_ptr() if last.numel() else None
+        s.last_bytes = last.numel()
+        s.scale = scale.data_ptr()
+        self.struct = s
+
+    @classmethod
+    def from_dict(cls, packed: dict, device=None) -> "DevicePacked":
+        dev = torch.device(device if device is not None else "cuda")
+        mv = lambda t: t.to(dev).contiguous()
+        return cls(packed["level_bits"], packed["out_f"], packed["in_f"],
+                   [mv(b) for b in packed["bitmaps"]], [mv(s) for s in packed["streams"]],
+                   mv(packed["scale"].reshape(1)))
+
+    # ---- thin call wrappers -------------------------------------------------
+    def prefix_entries(self, chunk: int) -> int:
+        return int(lib().ixh_prefix_entries(self.N, int(chunk)))
+
+    def prefix_build(self, chunk: int) -> torch.Tensor:
+        """int32 [n_levels-1, entries] rank table at flat positions u*chunk (device)."""
+        entries = self.prefix_entries(chunk)
+        if entries < 1:
+            raise ValueError(f"chunk {chunk} must be positive")
+        table = torch.empty((len(self.level_bits) - 1, entries), dtype=torch.int32, device=self.device)
+        check(lib().ixh_prefix_build(C.byref(self.struct), int(chunk), table.data_ptr(), current_stream(self.device)))
+        return table
+
+    def decode(self, table: torch.Tensor, chunk: int, out_i8=None, out_bf16=None) -> None:
+        for t, dt in ((out_i8, torch.int8), (out_bf16, torch.bfloat16)):
+            if t is not None:
+                _require_cuda(t, "decode output")
+                if t.dtype != dt or t.numel() < self.N:
+                    raise ValueError(f"decode output must be {dt} with at least {self.N} elements")
+        check(lib().ixh_decode(
+            C.byref(self.struct), table.data_ptr(), int(chunk),
+            out_i8.data_ptr() if out_i8 is not None else None,
+            out_bf16.data_ptr() if out_bf16 is not None else None, current_stream(self.device)))
+
+    def gemv_workspace_bytes(self, chunk: int, m: int, flags: int = 0) -> int:
+        return int(lib().ixh_gemv_workspace_bytes(C.byref(self.struct), int(chunk), int(m), int(flags)))
+
+    def gemv(self, table, chunk, x, y=None, y32=None, workspace=None, flags=0) -> None:
+        """x bf16 [M, in_f] (row stride x.stride(0)); y bf16 [M, out_f] or y32 fp32 (atomic mode)."""
+        if not x.is_cuda:
+            raise RuntimeError(f"x must live on the GPU (got {x.device}); the HIP path has no CPU fallback")
+        if x.dtype != torch.bfloat16:
+            raise ValueError("x must be bf16")
+        x2 = x.reshape(-1, self.in_f)
+        if x2.stride(1) != 1:
+            raise ValueError("x rows must be contiguous")
+        m = x2.shape[0]
+        ldx = x2.stride(0) if m > 1 else self.in_f
+        ldy = y.stride(0) if (y is not None and y.dim() == 2 and m > 1) else self.out_f
+        check(lib().ixh_gemv(
+            C.byref(self.struct), table.data_ptr(), int(chunk), x2.data_ptr(), m, ldx,
+            y.data_ptr() if y is not None else None, ldy,
+            y32.data_ptr() if y32 is not None else None,
+            workspace.data_ptr() if workspace is not None else None,
+            workspace.numel() * workspace.element_size() if workspace is not None else 0,
+            int(flags), current_stream(self.device)))

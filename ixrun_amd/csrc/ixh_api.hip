@@ -1,0 +1,176 @@
+// C boundary of the library: argument checks, kernel selection, error text.
+// Declarations and the reference interfaces they replace: include/ixhip.h.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "ixh_dev.h"
+#include "ixh_fast358.h"
+
+namespace ixh {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+// Validate an IxhPacked and turn it into the kernel-argument form.
+static int to_dev(const IxhPacked *pk, Dev *out) {
+    if (!pk) { set_error("packed is NULL"); return IXH_EINVAL; }
+    const int L = pk->n_levels;
+    if (L < 2 || L > IXH_MAX_LEVELS) { set_error("n_levels %d not in 2..%d", L, IXH_MAX_LEVELS); return IXH_EINVAL; }
+    if (pk->level_bits[L - 1] != 8) { set_error("last level must be 8-bit, got %d", pk->level_bits[L - 1]); return IXH_EINVAL; }
+    for (int i = 0; i < L - 1; ++i) {
+        const int b = pk->level_bits[i];
+        if (b < 1 || b > 7 || (i > 0 && b < pk->level_bits[i - 1])) {
+            set_error("level_bits[%d] = %d: widths must ascend within 1..7 before the final 8", i, b);
+            return IXH_EINVAL;
+        }
+    }
+    if (pk->out_f < 0 || pk->in_f < 0) { set_error("negative shape"); return IXH_EINVAL; }
+    const uint64_t n = (uint64_t)pk->out_f * (uint64_t)pk->in_f;
+    if (n >= (1ull << 31)) { set_error("out_f * in_f = %llu does not fit the 31-bit rank tables", (unsigned long long)n); return IXH_EINVAL; }
+    if (n != 0 && !pk->scale) { set_error("scale is NULL"); return IXH_EINVAL; }
+    Dev d;
+    memset(&d, 0, sizeof(d));
+    d.n_levels = L;
+    d.out_f = (uint32_t)pk->out_f;
+    d.in_f = (uint32_t)pk->in_f;
+    d.n = (uint32_t)n;
+    for (int i = 0; i < L; ++i) d.bits[i] = pk->level_bits[i];
+    for (int i = 0; i < L - 1; ++i) {
+        if (pk->bitmap_words[i] >= (1ull << 31) || pk->stream_words[i] >= (1ull << 31)) {
+            set_error("stream %d longer than 2^31 words", i);
+            return IXH_EINVAL;
+        }
+        if ((pk->bitmap_words[i] && !pk->bitmaps[i]) || (pk->stream_words[i] && !pk->streams[i])) {
+            set_error("level %d: non-empty stream with NULL pointer", i);
+            return IXH_EINVAL;
+        }
+        d.bm[i] = pk->bitmaps[i];
+        d.bm_words[i] = (uint32_t)pk->bitmap_words[i];
+        d.st[i] = pk->streams[i];
+        d.st_words[i] = (uint32_t)pk->stream_words[i];
+    }
+    if (pk->last_bytes >= (1ull << 31)) { set_error("last stream longer than 2^31 bytes"); return IXH_EINVAL; }
+    if (pk->last_bytes && !pk->last) { set_error("last stream non-empty with NULL pointer"); return IXH_EINVAL; }
+    // bitmap 0 must cover every element; shorter would make the kernels read past it
+    if (d.bm_words[0] < (d.n + 31u) / 32u) {
+        set_error("bitmap 0 has %u words, %u elements need %u", d.bm_words[0], d.n, (d.n + 31u) / 32u);
+        return IXH_EINVAL;
+    }
+    d.last = pk->last;
+    d.last_bytes = (uint32_t)pk->last_bytes;
+    d.scale = pk->scale;
+    *out = d;
+    return IXH_OK;
+}
+
+static bool is_358(const Dev &d) { return d.n_levels == 3 && d.bits[0] == 3 && d.bits[1] == 5 && d.bits[2] == 8; }
+
+}  // namespace ixh
+
+using namespace ixh;
+
+extern "C" {
+
+int ixh_version(void) { return 100; }
+
+const char *ixh_last_error(void) { return g_error; }
+
+int64_t ixh_prefix_entries(int64_t n, int64_t chunk) {
+    if (n < 0 || chunk <= 0) return -1;
+    return (n + chunk - 1) / chunk + 1;
+}
+
+int ixh_prefix_build(const IxhPacked *packed, int64_t chunk, int32_t *prefix, ixh_stream_t stream) {
+    Dev d;
+    int rc = to_dev(packed, &d);
+    if (rc) return rc;
+    if (chunk <= 0 || chunk >= (1ll << 31)) { set_error("chunk %lld out of range", (long long)chunk); return IXH_EINVAL; }
+    if (!prefix) { set_error("prefix is NULL"); return IXH_EINVAL; }
+    rc = launch_prefix_build(d, (uint32_t)chunk, prefix, (hipStream_t)stream);
+    if (rc) set_error("prefix_build: launch failed");
+    return rc;
+}
+
+int ixh_decode(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, int8_t *out_i8,
+               uint16_t *out_bf16, ixh_stream_t stream) {
+    Dev d;
+    int rc = to_dev(packed, &d);
+    if (rc) return rc;
+    if (chunk <= 0 || chunk >= (1ll << 31)) { set_error("chunk %lld out of range", (long long)chunk); return IXH_EINVAL; }
+    if (d.n == 0) return IXH_OK;
+    if (!prefix) { set_error("prefix is NULL"); return IXH_EINVAL; }
+    if (!out_i8 && !out_bf16) { set_error("both outputs are NULL"); return IXH_EINVAL; }
+    rc = launch_decode(d, prefix, (uint32_t)chunk, out_i8, out_bf16, (hipStream_t)stream);
+    if (rc == IXH_ELAUNCH) set_error("decode: launch failed");
+    return rc;
+}
+
+static int gemv_checks(const Dev &d, int64_t chunk, int32_t m) {
+    if (m < 1 || m > 16) { set_error("m = %d not in 1..16", m); return IXH_EINVAL; }
+    if (chunk <= 0 || chunk > (int64_t)d.in_f || d.in_f % chunk != 0) {
+        set_error("chunk %lld must divide in_f %u", (long long)chunk, d.in_f);
+        return IXH_EINVAL;
+    }
+    return IXH_OK;
+}
+
+size_t ixh_gemv_workspace_bytes(const IxhPacked *packed, int64_t chunk, int32_t m, uint32_t flags) {
+    Dev d;
+    if (to_dev(packed, &d)) return 0;
+    if (d.n == 0 || gemv_checks(d, chunk, m)) return 0;
+    if (flags & IXH_GEMV_ATOMIC) return 0;
+    const size_t n_chunks = d.in_f / (uint32_t)chunk;
+    if (n_chunks == 1) return 0;
+    return n_chunks * (size_t)m * d.out_f * sizeof(float);
+}
+
+int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, const uint16_t *x, int32_t m,
+             int64_t ldx, uint16_t *y, int64_t ldy, float *y32, void *workspace, size_t workspace_bytes,
+             uint32_t flags, ixh_stream_t stream) {
+    Dev d;
+    int rc = to_dev(packed, &d);
+    if (rc) return rc;
+    if (d.n == 0) {
+        if (d.out_f != 0 && m >= 1 && m <= 16 && !(flags & IXH_GEMV_ATOMIC) && y) {
+            // no inputs: every output is an empty sum
+            for (int j = 0; j < m; ++j)
+                if (launch_fill_u16(y + (int64_t)j * ldy, d.out_f, 0, (hipStream_t)stream)) return IXH_ELAUNCH;
+        }
+        return IXH_OK;
+    }
+    rc = gemv_checks(d, chunk, m);
+    if (rc) return rc;
+    if (!prefix || !x) { set_error("prefix or x is NULL"); return IXH_EINVAL; }
+    if (ldx < (int64_t)d.in_f && m > 1) { set_error("ldx %lld < in_f %u", (long long)ldx, d.in_f); return IXH_EINVAL; }
+    const bool atomic = (flags & IXH_GEMV_ATOMIC) != 0;
+    if (atomic) {
+        if (!y32) { set_error("IXH_GEMV_ATOMIC needs y32"); return IXH_EINVAL; }
+    } else {
+        if (!y) { set_error("y is NULL"); return IXH_EINVAL; }
+        if (ldy < (int64_t)d.out_f && m > 1) { set_error("ldy %lld < out_f %u", (long long)ldy, d.out_f); return IXH_EINVAL; }
+        const size_t need = ixh_gemv_workspace_bytes(packed, chunk, m, flags);
+        if (need && (!workspace || workspace_bytes < need)) {
+            set_error("workspace of %zu bytes needed, %zu given", need, workspace ? workspace_bytes : (size_t)0);
+            return IXH_EWORKSPACE;
+        }
+    }
+    rc = IXH_EUNSUPPORTED;
+    if (!(flags & IXH_GEMV_FORCE_GENERIC) && is_358(d) && fast358_supports(d, (uint32_t)chunk, m))
+        rc = launch_gemv_358(d, prefix, (uint32_t)chunk, x, m, ldx, y, ldy, y32, (float *)workspace, atomic,
+                             (hipStream_t)stream);
+    if (rc == IXH_EUNSUPPORTED) {  // other schemes, other chunk sizes, unaligned x
+        rc = launch_gemv_generic(d, prefix, (uint32_t)chunk, x, m, ldx, y, ldy, y32, (float *)workspace, atomic,
+                                 (hipStream_t)stream);
+    }
+    if (rc == IXH_ELAUNCH) set_error("gemv: launch failed");
+    return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,99 @@
+// Device-side view of a packed tensor and the wave64 helpers shared by the
+// gfx950 kernels.  Internal to the library; the public interface is
+// include/ixhip.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/ixhip.h"
+
+namespace ixh {
+
+constexpr int kWave = 64;
+
+// Kernel-argument form of IxhPacked: 32-bit lengths (N < 2^31 is checked at
+// the C boundary) and the derived sizes the kernels need.
+struct Dev {
+    int n_levels;
+    int bits[IXH_MAX_LEVELS];
+    const uint32_t *bm[IXH_MAX_LEVELS - 1];
+    uint32_t bm_words[IXH_MAX_LEVELS - 1];
+    const uint32_t *st[IXH_MAX_LEVELS - 1];
+    uint32_t st_words[IXH_MAX_LEVELS - 1];
+    const uint8_t *last;
+    uint32_t last_bytes;
+    const uint16_t *scale;
+    uint32_t out_f, in_f, n;
+};
+
+__device__ __forceinline__ uint32_t lanes_below(uint64_t mask) {
+    return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// round-to-nearest-even bf16 bit pattern of a finite fp32
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+
+// the reference's dequantisation: bf16(f32(v) * f32(scale)), returned as fp32
+__device__ __forceinline__ float dequant(int v, float scale) {
+    return bf16_bits_to_f32(f32_to_bf16_bits((float)v * scale));
+}
+
+__device__ __forceinline__ int threshold_of(int bits) { return (1 << (bits - 1)) - 1; }
+
+// Decode the 64 consecutive flat elements p0 .. p0+63 (one per lane; lanes with
+// alive == false take no part).  cnt[i] is the number of level-i elements
+// before p0 and is advanced past the group.  Works for any level scheme: lane
+// ranks come from ballots, so there is no scan and no shared memory.
+template <int L>
+__device__ __forceinline__ int decode64(const Dev &P, uint32_t p0, bool alive, uint32_t (&cnt)[L - 1]) {
+    int v = 0;
+    uint32_t space = p0;  // rank, in the current level's index space, of the group's first element
+#pragma unroll
+    for (int i = 0; i < L - 1; ++i) {
+        const uint64_t alive_mask = __ballot(alive);
+        const uint32_t r = space + lanes_below(alive_mask);
+        uint32_t bit = 0;
+        if (alive && P.bm_words[i] != 0) {
+            const uint32_t wi = min(r >> 5, P.bm_words[i] - 1);
+            bit = (P.bm[i][wi] >> (r & 31)) & 1u;
+        }
+        const bool taken = alive && bit;
+        const uint64_t taken_mask = __ballot(taken);
+        if (taken && P.st_words[i] != 0) {
+            const int b = P.bits[i];
+            const uint64_t bitpos = (uint64_t)(cnt[i] + lanes_below(taken_mask)) * (uint32_t)b;
+            const uint32_t wi = min((uint32_t)(bitpos >> 5), P.st_words[i] - 1);
+            const uint32_t s = (uint32_t)bitpos & 31u;
+            const uint32_t lo = P.st[i][wi];
+            const uint32_t hi = (s + b > 32 && wi + 1 < P.st_words[i]) ? P.st[i][wi + 1] : 0u;
+            const uint64_t both = ((uint64_t)hi << 32) | lo;
+            v = (int)((uint32_t)(both >> s) & ((1u << b) - 1u)) - threshold_of(b);
+        }
+        alive = alive && !bit;
+        space -= cnt[i];
+        cnt[i] += (uint32_t)__popcll(taken_mask);
+    }
+    const uint64_t alive_mask = __ballot(alive);
+    if (alive && P.last_bytes != 0) {
+        const uint32_t r = min(space + lanes_below(alive_mask), P.last_bytes - 1);
+        v = (int)P.last[r] - 127;
+    }
+    return v;
+}
+
+// ---- host-side launchers (one per translation unit of kernels) ----
+int launch_prefix_build(const Dev &P, uint32_t chunk, int32_t *prefix, hipStream_t s);
+int launch_decode(const Dev &P, const int32_t *prefix, uint32_t chunk, int8_t *o8, uint16_t *o16, hipStream_t s);
+int launch_gemv_generic(const Dev &P, const int32_t *prefix, uint32_t chunk, const uint16_t *x, int m,
+                        int64_t ldx, uint16_t *y, int64_t ldy, float *y32, float *ws, bool atomic,
+                        hipStream_t s);
+int launch_fill_u16(uint16_t *dst, uint32_t n, uint16_t value, hipStream_t s);
+void set_error(const char *fmt, ...);
+
+}  // namespace ixh

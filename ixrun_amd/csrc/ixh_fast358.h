@@ -1,0 +1,17 @@
+// Specialised (3,5,8) fused decode+GEMV for gfx950 (see ixh_fast358.hip).
+#pragma once
+#include "ixh_dev.h"
+
+namespace ixh {
+
+constexpr uint32_t kFastChunk = 512;  // elements per table unit the kernel is built around
+
+// true when launch_gemv_358 can serve the request (otherwise the caller uses the general kernel)
+bool fast358_supports(const Dev &P, uint32_t chunk, int m);
+// x / ld alignment is checked at launch; returns IXH_EUNSUPPORTED if it does not fit
+int launch_gemv_358(const Dev &P, const int32_t *prefix, uint32_t chunk, const uint16_t *x, int m, int64_t ldx,
+                    uint16_t *y, int64_t ldy, float *y32, float *ws, bool atomic, hipStream_t s);
+int launch_reduce_chunks(const float *ws, uint32_t n_chunks, int m, uint32_t out_f, uint16_t *y, int64_t ldy,
+                         hipStream_t s);
+
+}  // namespace ixh

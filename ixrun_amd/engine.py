@@ -1,0 +1,361 @@
+"""Deploy modules and engine of the INT8-X streaming path.
+
+``StreamingLinear`` keeps a layer's packed streams resident on the GPU and
+serves every forward from them: up to 16 activation rows go through the fused
+decode+GEMV kernel (the bf16 weight never reaches memory), larger batches are
+decoded into a shared bf16 buffer and multiplied with ``F.linear``.
+``GraphLinear`` / ``Int8XEngine`` follow the reference's ``ixrun/engine.py``
+(``StreamingLinear`` ``:40-173``, ``GraphLinear`` ``:179-196``,
+``ResourceScheduler`` ``:202-235``, ``Int8XEngine`` ``:241-516``) and keep its
+attribute names (``_b1 .. _l3, _scale, _b1_blk, _b2_blk, _q1, _q2,
+_split_chunk, _use_fused, _w_buf``), which callers of ``fused_gemv`` read.
+"""
+from __future__ import annotations
+
+import gc
+import os
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import _lib
+from .config import TRITON_BLOCK
+from .fused import FUSED_TILE, _pick_split, pick_unit, shared_workspace
+from .linear import _set_parent_child, iter_quantizable_linears
+from .quantize import int8x_quantize
+
+__all__ = ["Int8XEngine", "StreamingLinear", "GraphLinear", "ResourceScheduler"]
+
+MAX_FUSED_ROWS = 16  # activation rows served by the fused kernel
+
+
+class StreamingLinear(nn.Module):
+    """GPU-resident packed weight, decoded inside every forward.
+
+    Construction mirrors the reference (``ixrun/engine.py:49-104``): the packed
+    tensors become buffers on the GPU and the rank tables are derived once.
+    Here the tables are counted on the device from the bitmaps
+    (``ixh_prefix_build``); ``_q1``/``_q2`` and ``_b1_blk``/``_b2_blk`` are the
+    reference-shaped views of them.  Any level scheme is accepted; bitmaps and
+    streams beyond the third level are registered as ``_b3``, ``_l4`` and so on.
+    """
+
+    def __init__(self, packed: dict, bias=None):
+        super().__init__()
+        self.out_features = packed["out_f"]
+        self.in_features = packed["in_f"]
+        self.N = packed["N"]
+        self.level_bits = tuple(packed["level_bits"])
+        self.counts = packed["counts"]
+
+        n_levels = len(self.level_bits)
+        for i in range(n_levels - 1):
+            self.register_buffer(f"_b{i + 1}", packed["bitmaps"][i].cuda())
+        for i in range(n_levels):
+            self.register_buffer(f"_l{i + 1}", packed["streams"][i].cuda())
+        self.register_buffer("_scale", packed["scale"].reshape(()).cuda())
+        self._bind()
+
+        # rank tables: the kernels' own (unit = 512 where rows allow it) and
+        # the two the reference exposes
+        self._unit = pick_unit(self.in_features)
+        self.register_buffer("_table", self._dp.prefix_build(self._unit))
+        if self.N % TRITON_BLOCK == 0 and TRITON_BLOCK % self._unit == 0:
+            blk_table = self._table[:, :: TRITON_BLOCK // self._unit][:, : self.N // TRITON_BLOCK]
+        else:
+            blk_table = self._dp.prefix_build(TRITON_BLOCK)[:, :-1]
+        self.register_buffer("_b1_blk", blk_table[0].contiguous())
+        self.register_buffer("_b2_blk", blk_table[1].contiguous() if n_levels > 2 else torch.zeros_like(blk_table[0]))
+        self._use_triton = True
+
+        self._use_fused = True
+        self._split_chunk = 0
+        per_row = self.in_features // self._unit
+        split = _pick_split(self.in_features) if self.out_features < self.in_features else 1
+        if split > 1 and self.in_features % FUSED_TILE == 0:
+            self._split_chunk = self.in_features // split
+            step = self._split_chunk // self._unit
+        else:
+            step = per_row
+        q = self._table[:, : self.out_features * per_row : step]
+        self.register_buffer("_q1", q[0].contiguous())
+        self.register_buffer("_q2", q[1].contiguous() if n_levels > 2 else torch.zeros_like(q[0]))
+        self._y32 = None
+
+        if bias is not None:
+            self.register_buffer("_bias", bias.detach().clone().cuda())
+        else:
+            self._bias = None
+        self._w_buf = None  # set by the engine
+
+    def _bind(self):
+        n_levels = len(self.level_bits)
+        self._dp = _lib.DevicePacked(
+            self.level_bits, self.out_features, self.in_features,
+            [getattr(self, f"_b{i + 1}") for i in range(n_levels - 1)],
+            [getattr(self, f"_l{i + 1}") for i in range(n_levels)],
+            self._scale.reshape(1),
+        )
+
+    def _apply(self, fn, recurse=True):
+        # .to()/.cuda() may move the buffers: point the kernel arguments at the new storage
+        out = super()._apply(fn, recurse)
+        if hasattr(self, "_scale") and self._scale.is_cuda:
+            self._bind()
+        return out
+
+    def _set_shared_buf(self, w_buf):
+        self._w_buf = w_buf
+
+    def _decode(self):
+        """Decode into the shared buffer and return it as ``[out_f, in_f]``
+        (reference ``ixrun/engine.py:109-133``)."""
+        w_flat = self._w_buf[: self.N]
+        self._dp.decode(self._table, self._unit, out_bf16=w_flat)
+        return w_flat.view(self.out_features, self.in_features)
+
+    def forward(self, x):
+        rows = x.numel() // self.in_features if self.in_features else 0
+        if (self._use_fused and x.dtype == torch.bfloat16 and x.is_cuda and 1 <= rows <= MAX_FUSED_ROWS
+                and x.shape[-1] == self.in_features):
+            x2 = x.reshape(rows, self.in_features)
+            if x2.stride(1) != 1:
+                x2 = x2.contiguous()
+            y = torch.empty((rows, self.out_features), dtype=torch.bfloat16, device=x.device)
+            ws = shared_workspace(x.device, self._dp.gemv_workspace_bytes(self._unit, rows))
+            self._dp.gemv(self._table, self._unit, x2, y=y, workspace=ws)
+            y = y.view(x.shape[:-1] + (self.out_features,))
+            if self._bias is not None:
+                y = y + self._bias.to(y.dtype)
+            return y
+        w = self._decode()
+        bias = self._bias.to(x.dtype) if self._bias is not None else None
+        return F.linear(x, w.to(x.dtype) if w.dtype != x.dtype else w, bias)
+
+
+class GraphLinear(nn.Module):
+    """GEMM-only layer whose weight buffer is refreshed by a captured graph of
+    decode launches (reference ``ixrun/engine.py:179-196``)."""
+
+    def __init__(self, packed: dict, bias=None, decode_buf=None):
+        super().__init__()
+        self.out_features = packed["out_f"]
+        self.in_features = packed["in_f"]
+        self.N = packed["N"]
+        self._w_buf = decode_buf
+        if bias is not None:
+            self.register_buffer("_bias", bias.detach().clone().cuda())
+        else:
+            self._bias = None
+
+    def forward(self, x):
+        w = self._w_buf[: self.N].view(self.out_features, self.in_features)
+        bias = self._bias.to(x.dtype) if self._bias is not None else None
+        return F.linear(x, w, bias)
+
+
+class ResourceScheduler:
+    """Memory estimates and a mode recommendation (reference ``ixrun/engine.py:202-235``)."""
+
+    @staticmethod
+    @torch.no_grad()
+    def estimate(model: nn.Module, level_bits=(3, 5, 8)) -> dict:
+        bf16_bytes = packed_bytes = n_elems = max_layer = 0
+        for _, mod in iter_quantizable_linears(model):
+            w = mod.weight.data
+            packed_bytes += int8x_quantize(w, level_bits)["total_bytes"]
+            bf16_bytes += w.numel() * 2
+            n_elems += w.numel()
+            max_layer = max(max_layer, w.numel())
+        return {
+            "bf16_weight_MB": bf16_bytes / 1e6,
+            "packed_storage_MB": packed_bytes / 1e6,
+            "compression": bf16_bytes / max(packed_bytes, 1),
+            "max_layer_elems": max_layer,
+            "shared_decode_buf_MB": max_layer * 2 / 1e6,
+            "n_elems": n_elems,
+        }
+
+    @staticmethod
+    def recommend(model: nn.Module, gpu_budget_GB: float, level_bits=(3, 5, 8)) -> str:
+        est = ResourceScheduler.estimate(model, level_bits)
+        return "cached" if est["bf16_weight_MB"] + 1500 <= gpu_budget_GB * 1000 else "streaming"
+
+
+class Int8XEngine:
+    """Load a model, deploy it on packed weights, generate.
+
+    Same construction and deploy modes as the reference's ``Int8XEngine``
+    (``ixrun/engine.py:241-516``).  The three ``_deploy_*`` helpers take any
+    ``nn.Module``; ``from_pretrained`` needs ``transformers`` and a local
+    checkpoint, as in the reference.
+    """
+
+    def __init__(self, model, tokenizer, stats=None, graph_replay=None):
+        self.model = model
+        self.tokenizer = tokenizer
+        self.stats = stats or {}
+        self._graph_replay = graph_replay
+        self.model.eval()
+
+    @classmethod
+    def from_pretrained(cls, model_path: str, mode: str = "cached", level_bits=(3, 5, 8),
+                        dtype=torch.bfloat16, verbose: bool = True, cache_path: str | None = None):
+        from transformers import AutoModelForCausalLM, AutoTokenizer
+
+        tokenizer = AutoTokenizer.from_pretrained(model_path, trust_remote_code=True)
+        if tokenizer.pad_token is None:
+            tokenizer.pad_token = tokenizer.eos_token
+        big = mode in ("streaming", "graph")
+        model = AutoModelForCausalLM.from_pretrained(model_path, dtype=dtype, low_cpu_mem_usage=True)
+        if not big:
+            model = model.cuda()
+        if mode == "streaming":
+            stats = cls._deploy_streaming(model, level_bits, verbose=verbose, cache_path=cache_path)
+        elif mode == "graph":
+            stats, replay = cls._deploy_graph(model, level_bits, verbose=verbose)
+            return cls(model, tokenizer, stats, graph_replay=replay)
+        else:
+            stats = cls._deploy_cached(model, level_bits, verbose=verbose)
+        eng = cls(model, tokenizer, stats)
+        if big:
+            eng._finalize_device()
+        return eng
+
+    # ----- deploy helpers ---------------------------------------------------
+    @staticmethod
+    def _deploy_cached(model, level_bits, verbose=True):
+        from .linear import deploy_model
+
+        return deploy_model(model, level_bits=level_bits, cache="full", verbose=verbose)
+
+    @staticmethod
+    @torch.no_grad()
+    def _deploy_streaming(model, level_bits, verbose=True, cache_path=None):
+        """Packed weights resident on the GPU plus one shared decode buffer
+        (reference ``ixrun/engine.py:343-416``).  ``cache_path`` names a file of
+        already packed layers, ``{"level_bits": ..., "layers": [(name, packed,
+        bias), ...]}``, written on the first deploy and read on later ones; a
+        cache built with other ``level_bits`` or for other layer names raises
+        ``ValueError`` as in the reference (``:360-370``)."""
+        targets = list(iter_quantizable_linears(model))
+        layer_data = None
+        if cache_path is not None and os.path.exists(cache_path):
+            if verbose:
+                print(f"[engine][cache] loading packed weights from {cache_path}", flush=True)
+            # tuples, dicts, numbers and tensors only: the safe loader reads all of it
+            blob = torch.load(cache_path, map_location="cpu", weights_only=True)
+            if tuple(blob["level_bits"]) != tuple(level_bits):
+                raise ValueError(
+                    f"cache was built with level_bits={blob['level_bits']}, "
+                    f"requested {tuple(level_bits)}; delete the cache or change level_bits")
+            layer_data = blob["layers"]
+            have = {n for n, _ in model.named_modules()}
+            missing = [n for n, _, _ in layer_data if n not in have]
+            if missing:
+                raise ValueError(f"cache/model mismatch: {len(missing)} unknown layers")
+            if verbose:
+                print(f"[engine][cache] {len(layer_data)} layers loaded", flush=True)
+        if layer_data is None:
+            layer_data = []
+            for name, mod in targets:
+                bias = mod.bias.data if mod.bias is not None else None
+                layer_data.append((name, int8x_quantize(mod.weight.data, level_bits), bias))
+            if cache_path is not None:
+                if verbose:
+                    print(f"[engine][cache] saving packed weights to {cache_path}", flush=True)
+                torch.save({"level_bits": tuple(level_bits), "layers": layer_data}, cache_path)
+
+        total_bytes = max_n = 0
+        layers = []
+        for name, packed, bias in layer_data:
+            layers.append((name, StreamingLinear(packed, bias=bias)))
+            total_bytes += packed["total_bytes"]
+            max_n = max(max_n, packed["N"])
+        shared_w = torch.empty(max_n, dtype=torch.bfloat16, device="cuda")
+        for name, sl in layers:
+            sl._set_shared_buf(shared_w)
+            _set_parent_child(model, name, sl)
+        gc.collect()
+        torch.cuda.empty_cache()
+        shared_mb = shared_w.numel() * 2 / 1e6
+        if verbose:
+            print(f"[engine][streaming] {len(layers)} layers | packed GPU-resident={total_bytes / 1e6:.0f}MB | "
+                  f"shared decode buf={shared_mb:.1f}MB", flush=True)
+        return {"mode": "streaming", "n_layers": len(layers), "total_bytes": total_bytes, "shared_gpu_MB": shared_mb}
+
+    @staticmethod
+    @torch.no_grad()
+    def _deploy_graph(model, level_bits, verbose=True):
+        """Streaming deploy with every layer's decode launch captured in one
+        graph (reference ``ixrun/engine.py:420-487``): each layer gets its own
+        decode buffer, the graph replays all decodes, forwards are GEMM-only."""
+        targets = list(iter_quantizable_linears(model))
+        total_params = sum(m.weight.numel() for _, m in targets)
+        if total_params * 2 > torch.cuda.get_device_properties(0).total_memory * 0.9:
+            raise RuntimeError(
+                f"graph mode needs {total_params * 2 / 1e9:.1f}GB of per-layer decode buffers "
+                f"- too large for this GPU; use mode='streaming'")
+        total_bytes = 0
+        specs = []
+        for name, mod in targets:
+            packed = int8x_quantize(mod.weight.data, level_bits)
+            bias = mod.bias.data if mod.bias is not None else None
+            sl = StreamingLinear(packed, bias=bias)
+            buf = torch.empty(packed["N"], dtype=torch.bfloat16, device="cuda")
+            sl._set_shared_buf(buf)
+            specs.append((name, sl, buf))
+            total_bytes += packed["total_bytes"]
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _, sl, _ in specs:
+                sl._decode()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _, sl, _ in specs:
+                sl._decode()
+        torch.cuda.synchronize()
+        if verbose:
+            print(f"[engine][graph] captured {len(specs)} decode kernels", flush=True)
+        for name, sl, buf in specs:
+            meta = {"out_f": sl.out_features, "in_f": sl.in_features, "N": sl.N}
+            _set_parent_child(model, name, GraphLinear(meta, bias=sl._bias, decode_buf=buf))
+
+        def replay(_keep_alive=specs, _graph=graph):
+            _graph.replay()
+
+        if verbose:
+            print(f"[engine][graph] {len(specs)} layers | packed={total_bytes / 1e6:.0f}MB | decode=graph.replay()",
+                  flush=True)
+        return {"mode": "graph", "n_layers": len(specs), "total_bytes": total_bytes}, replay
+
+    # ----- inference --------------------------------------------------------
+    def _finalize_device(self):
+        """Move whatever the deploy left on the CPU (reference ``ixrun/engine.py:490-504``)."""
+        for _, mod in self.model.named_modules():
+            for p in mod.parameters(recurse=False):
+                if p.data.device.type != "cuda":
+                    p.data = p.data.cuda()
+            for bname, b in mod.named_buffers(recurse=False):
+                if b.device.type != "cuda":
+                    setattr(mod, bname, b.cuda())
+        gc.collect()
+        torch.cuda.empty_cache()
+        self.model.eval()
+
+    def _pre_forward(self):
+        if self._graph_replay is not None:
+            self._graph_replay()
+
+    @torch.no_grad()
+    def generate(self, prompt, max_new_tokens: int = 64, **kw):
+        """Greedy text generation through the wrapped model's own ``generate``."""
+        self._pre_forward()
+        ids = self.tokenizer(prompt, return_tensors="pt").to("cuda")
+        out = self.model.generate(**ids, max_new_tokens=max_new_tokens, do_sample=False, **kw)
+        return self.tokenizer.decode(out[0][ids["input_ids"].shape[1]:], skip_special_tokens=True)

@@ -1,0 +1,98 @@
+"""Host-side checks of the C ABI that need no GPU: the library loads, exports
+every symbol include/ixhip.h declares, and refuses malformed requests before
+any kernel launch."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+from ixrun_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ixhip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ixh_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported():
+    lib = _lib.lib()
+    names = declared_symbols()
+    assert "ixh_gemv" in names and "ixh_decode" in names and "ixh_prefix_build" in names
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in include/ixhip.h but not exported"
+    assert set(_lib.EXPORTS) == set(names)
+    assert lib.ixh_version() >= 100
+
+
+def _packed(level_bits=(3, 5, 8), out_f=4, in_f=8, bm0_words=1):
+    s = _lib.IxhPacked()
+    s.n_levels = len(level_bits)
+    for i, b in enumerate(level_bits):
+        s.level_bits[i] = b
+    s.out_f, s.in_f = out_f, in_f
+    s.bitmaps[0] = 0x1000
+    s.bitmap_words[0] = bm0_words
+    s.scale = 0x1000
+    return s
+
+
+def test_entries_and_workspace_sizes():
+    lib = _lib.lib()
+    assert lib.ixh_prefix_entries(10, 5) == 3 and lib.ixh_prefix_entries(11, 5) == 4
+    assert lib.ixh_prefix_entries(0, 512) == 1 and lib.ixh_prefix_entries(10, 0) == -1
+    s = _packed(out_f=8, in_f=2048, bm0_words=512)
+    assert lib.ixh_gemv_workspace_bytes(C.byref(s), 512, 3, 0) == 4 * 3 * 8 * 4
+    assert lib.ixh_gemv_workspace_bytes(C.byref(s), 2048, 3, 0) == 0
+    assert lib.ixh_gemv_workspace_bytes(C.byref(s), 512, 3, _lib.IXH_GEMV_ATOMIC) == 0
+
+
+@pytest.mark.parametrize("mutate,needle", [
+    (lambda s: setattr(s, "n_levels", 1), "n_levels"),
+    (lambda s: s.level_bits.__setitem__(2, 7), "last level"),
+    (lambda s: s.level_bits.__setitem__(0, 6), "ascend"),
+    (lambda s: setattr(s, "out_f", 1 << 20) or setattr(s, "in_f", 1 << 12), "31-bit"),
+    (lambda s: s.bitmap_words.__setitem__(0, 0), "bitmap 0"),
+    (lambda s: setattr(s, "scale", None), "scale"),
+])
+def test_malformed_packed_is_refused(mutate, needle):
+    lib = _lib.lib()
+    s = _packed()
+    mutate(s)
+    rc = lib.ixh_prefix_build(C.byref(s), 8, 0x1000, None)
+    assert rc == -1 and needle in lib.ixh_last_error().decode()
+
+
+def test_malformed_gemv_arguments():
+    lib = _lib.lib()
+    s = _packed(out_f=4, in_f=1024, bm0_words=128)
+    call = lambda chunk, m, x=0x1000, y=0x1000, ws=None, wsb=0, flags=0: lib.ixh_gemv(
+        C.byref(s), 0x1000, chunk, x, m, 1024, y, 4, None, ws, wsb, flags, None)
+    assert call(512, 0) == -1 and "m = 0" in lib.ixh_last_error().decode()
+    assert call(512, 17) == -1
+    assert call(500, 1) == -1 and "divide" in lib.ixh_last_error().decode()
+    assert call(512, 1, x=None) == -1
+    assert call(512, 1, y=None) == -1
+    assert call(512, 1) == -4 and "workspace" in lib.ixh_last_error().decode()  # two chunks need partial sums
+    assert call(512, 1, flags=_lib.IXH_GEMV_ATOMIC) == -1 and "y32" in lib.ixh_last_error().decode()
+    with pytest.raises(_lib.IxhError):
+        _lib.check(-1)
+
+
+def test_device_packed_refuses_cpu_tensors():
+    from ixrun_amd.quantize import int8x_quantize
+
+    p = int8x_quantize((torch.randn(8, 64) * 0.02).bfloat16())
+    with pytest.raises(RuntimeError, match="GPU"):
+        _lib.DevicePacked(p["level_bits"], 8, 64, p["bitmaps"], p["streams"], p["scale"].reshape(1))
+
+
+def test_missing_library_is_loud(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libixhip.so")
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _lib.lib()

@@ -1,0 +1,268 @@
+"""Parity of the gfx950 kernels with the CPU oracle, through the C ABI.
+
+Integer results (rank tables, decoded int8, decoded bf16 bit patterns) must be
+bit-exact.  Fused decode+GEMV outputs are compared with the fp64 oracle on the
+same seeded inputs: relative L2 error <= 1e-3 (the build's tolerance) and the
+reference's own acceptance metric max|dy| / max|y| < 5e-3
+(tests/test_fused.py:34-37, tests/test_splitk.py:34-35).
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import (activations, bf16_bits, calibrated_weight, int8_mix, outlier_weight, packed_from_int8, rel_l2,
+                     student_t_weight)
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_TOL = 1e-3
+REF_MAX_TOL = 5e-3
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from ixrun_amd import _lib
+
+    assert _lib.lib().ixh_version() >= 100  # the HIP library itself, not a fallback
+    return torch.device("cuda:0")
+
+
+def quantize(w, level_bits=(3, 5, 8)):
+    from ixrun_amd.quantize import int8x_quantize
+
+    return int8x_quantize(w, level_bits)
+
+
+def device_packed(p, dev):
+    from ixrun_amd import _lib
+
+    return _lib.DevicePacked.from_dict(p, dev)
+
+
+def check_outputs(y_bits, y64, what=""):
+    y = (y_bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    err = rel_l2(y, y64)
+    ref_metric = np.abs(y - y64).max() / max(np.abs(y64).max(), 1e-300)
+    assert err <= REL_L2_TOL, f"{what}: rel-L2 {err:.3e}"
+    assert ref_metric < REF_MAX_TOL, f"{what}: max-rel {ref_metric:.3e}"
+    return err
+
+
+def make_packed(kind, out_f, in_f, level_bits=(3, 5, 8)):
+    """Packed dictionaries with the level mixes the kernels must survive."""
+    if kind == "outlier":
+        return quantize(outlier_weight(out_f, in_f, seed=0), level_bits)
+    if kind == "student_t":
+        return quantize(student_t_weight(out_f, in_f, seed=0), level_bits)
+    if kind == "calibrated_pow2":
+        return quantize(calibrated_weight(out_f, in_f, seed=0)[0], level_bits)
+    if kind == "calibrated_odd_scale":  # scale bf16(0.0123): v*scale is rounded when dequantised
+        return quantize(calibrated_weight(out_f, in_f, seed=0, scale=0.0123046875)[0], level_bits)
+    return packed_from_int8(int8_mix(kind, out_f * in_f, seed=1), out_f, in_f, level_bits=level_bits)
+
+
+KINDS = ["outlier", "student_t", "calibrated_pow2", "calibrated_odd_scale", "only_l1", "no_l3", "no_l2", "only_l3",
+         "rare_other"]
+
+
+# ---------------------------------------------------------------- rank tables
+@pytest.mark.parametrize("shape,level_bits,chunk", [
+    ((64, 1024), (3, 5, 8), 512), ((96, 1024), (3, 5, 8), 1024), ((33, 96), (3, 4, 5, 6, 8), 32),
+    ((5, 7), (3, 5, 8), 7), ((17, 100), (3, 5, 8), 1024), ((300, 1536), (3, 5, 8), 512), ((7, 33), (2, 8), 5)])
+def test_prefix_build(oracle, dev, shape, level_bits, chunk):
+    p = quantize(outlier_weight(*shape, seed=7), level_bits)
+    dp = device_packed(p, dev)
+    table = dp.prefix_build(chunk).cpu().numpy()
+    pn = oracle.packed_to_numpy(p)
+    want = oracle.prefix(p["N"], len(level_bits), pn["bitmaps"], chunk)
+    assert table.shape == want.shape and np.array_equal(table, want)
+
+
+def test_reference_shaped_tables(oracle, dev):
+    from ixrun_amd.fused import compute_row_prefixes
+    from ixrun_amd.triton_kernels import precompute_block_offsets
+
+    p = quantize(outlier_weight(48, 2048, seed=3))
+    b1_blk, b2_blk = precompute_block_offsets(p, device=dev)
+    pn = oracle.packed_to_numpy(p)
+    want = oracle.prefix(p["N"], 3, pn["bitmaps"], 1024)
+    assert b1_blk.dtype == torch.int32 and b1_blk.is_cuda and b1_blk.numel() == p["N"] // 1024
+    assert np.array_equal(b1_blk.cpu().numpy(), want[0, :-1]) and np.array_equal(b2_blk.cpu().numpy(), want[1, :-1])
+    q1, q2 = compute_row_prefixes(p, 1024)
+    assert np.array_equal(q1.numpy(), want[0, :-1]) and np.array_equal(q2.numpy(), want[1, :-1])
+
+
+# ---------------------------------------------------------------- decode, bit-exact
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("shape", [(1, 1), (3, 11), (7, 33), (128, 256), (33, 1000), (64, 1536), (300, 1031)])
+def test_decode_bit_exact(oracle, dev, kind, shape):
+    p = make_packed(kind, *shape)
+    dp = device_packed(p, dev)
+    q_want = oracle.decode_packed_i8(p)
+    w_want = oracle.decode_packed_bf16(p)
+    for chunk in (1024, 512, 96):
+        table = dp.prefix_build(chunk)
+        o8 = torch.full((p["N"],), 99, dtype=torch.int8, device=dev)
+        o16 = torch.zeros(p["N"], dtype=torch.bfloat16, device=dev)
+        dp.decode(table, chunk, out_i8=o8, out_bf16=o16)
+        assert np.array_equal(o8.cpu().numpy(), q_want), (kind, shape, chunk)
+        assert np.array_equal(bf16_bits(o16).reshape(shape), w_want), (kind, shape, chunk)
+
+
+@pytest.mark.parametrize("level_bits", [(3, 4, 5, 6, 8), (2, 8), (4, 8), (1, 2, 3, 4, 5, 6, 7, 8), (3, 3, 8)])
+def test_decode_other_level_schemes(oracle, dev, level_bits):
+    from ixrun_amd.triton_kernels import decode_weight_triton, decode_int8
+
+    p = quantize(outlier_weight(96, 200, seed=9), level_bits)
+    assert np.array_equal(decode_int8(p, dev).cpu().numpy().reshape(-1), oracle.decode_packed_i8(p))
+    w = decode_weight_triton(p, device=dev)
+    assert w.dtype == torch.bfloat16 and w.shape == (96, 200)
+    assert np.array_equal(bf16_bits(w), oracle.decode_packed_bf16(p))
+
+
+def test_decode_config1_2048(oracle, dev):
+    """BASELINE config 1: 2048x2048 Student-t, int8 round trip bit-exact, level fractions reported."""
+    from ixrun_amd.triton_kernels import decode_weight_triton, decode_int8
+
+    w = student_t_weight(2048, 2048, seed=0)
+    p = quantize(w)
+    scale_bits, q = oracle.quantize_bf16(bf16_bits(w))
+    assert np.array_equal(decode_int8(p, dev).cpu().numpy().reshape(-1), q)
+    assert np.array_equal(bf16_bits(decode_weight_triton(p, device=dev)).reshape(-1), oracle.dequant_bf16(q, scale_bits))
+    frac = [c / p["N"] for c in p["counts"]]
+    print(f"config1 fractions L1/L2/L3 = {frac[0]:.4f}/{frac[1]:.4f}/{frac[2]:.5f}, bpw {p['bits_per_weight']:.3f}")
+    assert p["total_bytes"] == 2_336_569  # the size SURVEY measured for this recipe
+
+
+# ---------------------------------------------------------------- fused decode + GEMV
+def run_gemv(dp, chunk, x, m, dev, flags=0, atomic=False):
+    from ixrun_amd import _lib
+
+    table = dp.prefix_build(chunk)
+    xd = x.to(dev)
+    if atomic:
+        y32 = torch.zeros((m, dp.out_f), dtype=torch.float32, device=dev)
+        dp.gemv(table, chunk, xd, y32=y32, flags=flags | _lib.IXH_GEMV_ATOMIC)
+        return bf16_bits(y32.to(torch.bfloat16))
+    y = torch.zeros((m, dp.out_f), dtype=torch.bfloat16, device=dev)
+    nbytes = dp.gemv_workspace_bytes(chunk, m, flags)
+    ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=dev)
+    dp.gemv(table, chunk, xd, y=y, workspace=ws, flags=flags)
+    return bf16_bits(y)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("shape", [(64, 512), (37, 1024), (130, 1536), (256, 4608)])
+@pytest.mark.parametrize("m", [1, 2, 3, 8, 16])
+def test_gemv_fast_and_general(oracle, dev, kind, shape, m):
+    from ixrun_amd import _lib
+
+    out_f, in_f = shape
+    p = make_packed(kind, out_f, in_f)
+    dp = device_packed(p, dev)
+    x = activations(m, in_f, seed=1)
+    y64 = oracle.gemm_f64(oracle.decode_packed_bf16(p), bf16_bits(x))
+    for flags, chunk, atomic in [(0, 512, False), (0, 512, True), (_lib.IXH_GEMV_FORCE_GENERIC, 512, False),
+                                 (0, in_f, False), (0, 256, True)]:
+        y = run_gemv(dp, chunk, x, m, dev, flags=flags, atomic=atomic)
+        check_outputs(y, y64, f"{kind} {shape} m={m} flags={flags} chunk={chunk} atomic={atomic}")
+
+
+@pytest.mark.parametrize("shape,level_bits,chunk", [((40, 96), (3, 4, 5, 6, 8), 32), ((33, 100), (3, 5, 8), 50),
+                                                    ((64, 1024), (3, 4, 5, 6, 8), 512), ((9, 7), (2, 8), 7)])
+def test_gemv_general_shapes_and_schemes(oracle, dev, shape, level_bits, chunk):
+    p = quantize(outlier_weight(*shape, seed=4), level_bits)
+    dp = device_packed(p, dev)
+    for m in (1, 5):
+        x = activations(m, shape[1], seed=2)
+        y64 = oracle.gemm_f64(oracle.decode_packed_bf16(p), bf16_bits(x))
+        check_outputs(run_gemv(dp, chunk, x, m, dev), y64, f"{shape} {level_bits} m={m}")
+
+
+@pytest.mark.parametrize("kind", ["student_t", "calibrated_odd_scale", "rare_other"])
+def test_gemv_one_hot_is_exact(oracle, dev, kind):
+    """x = e_k makes y the decoded column k, exactly: products with 1.0 and zeros add without rounding."""
+    out_f, in_f = 96, 1024
+    p = make_packed(kind, out_f, in_f)
+    dp = device_packed(p, dev)
+    w_want = oracle.decode_packed_bf16(p)
+    for k in (0, 31, 32, 511, 512, 1023):
+        x = torch.zeros(1, in_f, dtype=torch.bfloat16)
+        x[0, k] = 1.0
+        for chunk in (512, in_f):
+            assert np.array_equal(run_gemv(dp, chunk, x, 1, dev)[0], w_want[:, k]), (kind, k, chunk)
+
+
+def test_gemv_is_reproducible(oracle, dev):
+    p = make_packed("calibrated_odd_scale", 256, 2048)
+    dp = device_packed(p, dev)
+    x = activations(4, 2048, seed=5)
+    first = run_gemv(dp, 512, x, 4, dev)
+    for _ in range(5):
+        assert np.array_equal(run_gemv(dp, 512, x, 4, dev), first)
+
+
+@pytest.mark.parametrize("shape", [(1536, 1536), (4608, 1536), (1536, 4608)])
+def test_reference_call_surface(oracle, dev, shape):
+    """fused_gemv / StreamingLinear called the way the reference's tests call them
+    (tests/test_fused.py:24-33, tests/test_splitk.py:25-33), on the reference's weight recipe."""
+    from ixrun_amd.engine import StreamingLinear
+    from ixrun_amd.fused import compute_row_prefixes, fused_gemv, _pick_split
+
+    out_f, in_f = shape
+    p = quantize(outlier_weight(out_f, in_f, seed=0))
+    x = activations(1, in_f, seed=1).reshape(in_f)
+    y64 = oracle.gemm_f64(oracle.decode_packed_bf16(p), bf16_bits(x).reshape(1, -1))
+    b1, b2 = (t.to(dev) for t in p["bitmaps"])
+    l1, l2, l3 = (t.to(dev) for t in p["streams"])
+    q1, q2 = compute_row_prefixes(p)
+    y = fused_gemv(x.to(dev), b1, b2, l1, l2, l3, q1.to(dev), q2.to(dev), p["scale"].to(dev), out_f, in_f)
+    assert y.dtype == torch.bfloat16 and y.shape == (out_f,)
+    check_outputs(bf16_bits(y).reshape(1, -1), y64, f"fused_gemv {shape}")
+    split = _pick_split(in_f) if out_f < in_f else 1
+    if split > 1:
+        chunk = in_f // split
+        q1c, q2c = compute_row_prefixes(p, chunk)
+        y32 = torch.zeros(out_f, dtype=torch.float32, device=dev)
+        ret = fused_gemv(x.to(dev), b1, b2, l1, l2, l3, q1c.to(dev), q2c.to(dev), p["scale"].to(dev), out_f, in_f,
+                         chunk=chunk, y32=y32)
+        assert ret is y32
+        check_outputs(bf16_bits(y32.to(torch.bfloat16)).reshape(1, -1), y64, f"fused_gemv split {shape}")
+
+    bias = torch.randn(out_f, generator=torch.Generator().manual_seed(3)).bfloat16()
+    sl = StreamingLinear(p, bias=bias)
+    shared = torch.empty(p["N"], dtype=torch.bfloat16, device=dev)
+    sl._set_shared_buf(shared)
+    assert np.array_equal(sl._q1.cpu().numpy(), (compute_row_prefixes(p, sl._split_chunk) if sl._split_chunk
+                                                   else compute_row_prefixes(p))[0].numpy())
+    w_ref = torch.from_numpy(oracle.decode_packed_bf16(p).view(np.int16)).view(torch.bfloat16)
+    assert torch.equal(sl._decode().cpu(), w_ref)
+    for xin in (x.to(dev).reshape(1, 1, in_f), activations(3, in_f, seed=2).to(dev), activations(40, in_f, seed=3).to(dev)):
+        out = sl(xin)
+        assert out.shape == xin.shape[:-1] + (out_f,) and out.dtype == torch.bfloat16
+        want = torch.nn.functional.linear(xin.float().cpu(), w_ref.float()).double().numpy()
+        got = (out.float().cpu() - bias.float()).double().numpy()
+        assert rel_l2(got, want) < 6e-3  # bias add and output are bf16-rounded
+
+
+@pytest.mark.parametrize("shape,m", [((5120, 5120), 1), ((5120, 17408), 1), ((17408, 5120), 4)])
+def test_full_size_layers(oracle, dev, shape, m):
+    """BASELINE configs 2, 3 and 4 at full size: decoded int8 bit-exact, outputs within tolerance."""
+    from ixrun_amd.engine import StreamingLinear
+
+    out_f, in_f = shape
+    w = student_t_weight(out_f, in_f, seed=0)
+    p = quantize(w)
+    q_want = oracle.decode_packed_i8(p)
+    sl = StreamingLinear(p)
+    o8 = torch.empty(p["N"], dtype=torch.int8, device=dev)
+    sl._dp.decode(sl._table, sl._unit, out_i8=o8)
+    assert np.array_equal(o8.cpu().numpy(), q_want)
+    x = activations(m, in_f, seed=1)
+    y = sl(x.to(dev))
+    w_bits = oracle.dequant_bf16(q_want, oracle.packed_to_numpy(p)["scale_bits"]).reshape(out_f, in_f)
+    y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
+    err = check_outputs(bf16_bits(y), y64, f"full {shape} m={m}")
+    print(f"{shape} m={m}: rel-L2 {err:.2e}, fractions {[round(c / p['N'], 5) for c in p['counts']]}, "
+          f"packed {p['total_bytes']} B")
