@@ -1,0 +1,203 @@
+#!/usr/bin/env python3
+"""Headline benchmark: fused (3,5,8) decode + GEMV on the 5120x17408 batch-1 layer.
+
+One step = one fused decode+GEMV over one packed layer.  The timed region walks
+round-robin over COPIES distinct packed copies of the layer (together larger
+than the 256 MB last-level cache) so that every launch streams its packed bytes
+from HBM.  Inputs are resident on the GPU before the clock starts.
+
+Prints one JSON line (see README / DESIGN.md for the fields).  Extra workloads
+(--workload) time the other shapes of the hot path with the same harness.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK = 8.0e12  # B/s, MI355X published
+
+WORKLOADS = {
+    # name: (out_f, in_f, m, weight recipe)
+    "down_proj_5120x17408_m1_student_t": (5120, 17408, 1, "student_t"),
+    "down_proj_5120x17408_m1_calibrated": (5120, 17408, 1, "calibrated"),
+    "attn_proj_5120x5120_m1_student_t": (5120, 5120, 1, "student_t"),
+    "gate_up_17408x5120_m2_student_t": (17408, 5120, 2, "student_t"),
+    "gate_up_17408x5120_m4_student_t": (17408, 5120, 4, "student_t"),
+    "gate_up_17408x5120_m8_student_t": (17408, 5120, 8, "student_t"),
+    "gate_up_17408x5120_m16_student_t": (17408, 5120, 16, "student_t"),
+}
+
+
+def make_weight(out_f, in_f, recipe):
+    from helpers import calibrated_weight, student_t_weight
+
+    if recipe == "student_t":
+        return student_t_weight(out_f, in_f, seed=0)
+    return calibrated_weight(out_f, in_f, seed=0)[0]
+
+
+def cpu_baseline(weight, x, level_bits=(3, 5, 8), rows=640):
+    """The reference's CPU path on the host cores: torch scatter decode of the packed
+    layer to bf16 (ixrun/quantize.py:154-183 restated in ixrun_amd.quantize) followed
+    by F.linear, on the first `rows` rows of the same weight so that it stays bounded;
+    next to it the oracle's single-core C walk (decode + fp32 dot) over the same rows."""
+    import torch.nn.functional as F
+
+    from ixrun_amd.quantize import decode_to_weight, int8x_quantize
+    from oracle import ix_oracle as oracle
+
+    sub = int8x_quantize(weight[:rows].contiguous(), level_bits)
+    n = sub["N"]
+    xs = x[:1]
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        w = decode_to_weight(sub, device="cpu")
+        t1 = time.perf_counter()
+        F.linear(xs, w)
+        t2 = time.perf_counter()
+        times.append((t2 - t0, t1 - t0, t2 - t1))
+    total, dec, mm = sorted(times)[1]
+    pn = oracle.packed_to_numpy(sub)
+    xb = xs[0].contiguous().view(torch.int16).numpy().view(np.uint16)
+    reps, t0 = 0, time.perf_counter()
+    while reps < 3 or time.perf_counter() - t0 < 3.0:
+        oracle.fused_gemv_f32(rows, pn["in_f"], pn["level_bits"], pn["bitmaps"], pn["streams"], pn["last"],
+                              pn["scale_bits"], xb)
+        reps += 1
+    t_c = (time.perf_counter() - t0) / reps
+    return {
+        "value": n / total / 1e9, "unit": "G weights/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"first {rows} rows ({n} weights) of the same layer: torch CPU scatter decode {dec:.2f} s + "
+                  f"F.linear {mm * 1e3:.1f} ms, median of 3; host has {os.cpu_count()} logical cores",
+        "oracle_c_single_core_G_weights_per_s": n / t_c / 1e9,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=480)
+    ap.add_argument("--warmup", type=int, default=48)
+    ap.add_argument("--workload", default="down_proj_5120x17408_m1_student_t", choices=list(WORKLOADS))
+    ap.add_argument("--copies", type=int, default=0, help="distinct packed copies to rotate over (0 = enough for 600 MB)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--eager", action="store_true", help="time eager launches instead of hipGraph replays")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (one MI355X holds the whole layer); "
+                 "run with --gpus 1")
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    dev = torch.device("cuda:0")
+
+    from ixrun_amd.engine import StreamingLinear
+
+    out_f, in_f, m, recipe = WORKLOADS[args.workload]
+    t0 = time.perf_counter()
+    from ixrun_amd.quantize import int8x_quantize
+
+    weight = make_weight(out_f, in_f, recipe)
+    packed = int8x_quantize(weight)
+    prep_s = time.perf_counter() - t0
+    copies = args.copies or max(2, -(-600_000_000 // packed["total_bytes"]))
+    layers = [StreamingLinear(packed) for _ in range(copies)]
+    g = torch.Generator("cpu").manual_seed(1)
+    x_host = torch.randn(m, in_f, generator=g).bfloat16()
+    x = x_host.to(dev)
+    table_bytes = layers[0]._table.numel() * 4
+    # algorithmic bytes of one step: the packed layer, the activations in, the outputs out
+    alg_bytes = packed["total_bytes"] + m * in_f * 2 + m * out_f * 2
+
+    def step(i):
+        return layers[i % copies](x)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+
+    # One pass over all copies is captured as a hipGraph (the per-layer launches
+    # of a decode step are replayed the same way); the timed region replays it.
+    rounds = max(1, -(-args.steps // copies))
+    steps = rounds * copies if not args.eager else args.steps
+    graph = None
+    if not args.eager:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for i in range(copies):
+                step(i)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            outs = [step(i) for i in range(copies)]
+        graph.replay()
+        torch.cuda.synchronize()
+
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t_wall = time.perf_counter()
+    start.record()
+    if graph is not None:
+        for _ in range(rounds):
+            graph.replay()
+    else:
+        for i in range(steps):
+            step(i)
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t_wall) * 1e3
+    ms_per_step = start.elapsed_time(stop) / steps
+
+    # eager launches with an event pair around every call, for the spread and the host cost
+    n_ev = min(steps, 240)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_ev)]
+    for i, (a, b) in enumerate(evs):
+        a.record()
+        step(i)
+        b.record()
+    torch.cuda.synchronize()
+    per_call = np.array([a.elapsed_time(b) for a, b in evs]) * 1e3  # us
+
+    us = ms_per_step * 1e3
+    weights_per_s = out_f * in_f / (ms_per_step * 1e-3)
+    achieved = alg_bytes / (ms_per_step * 1e-3)
+    out = {
+        "metric": "fused decode+GEMV G weights/s & % HBM peak (5120x17408, batch 1); us/layer",
+        "value": weights_per_s / 1e9, "unit": "G weights/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "us_per_layer": us, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16 activations x int8 codes, fp32 accumulate", "data": "synthetic",
+        "config": {
+            "workload": args.workload, "out_f": out_f, "in_f": in_f, "batch": m, "level_bits": [3, 5, 8],
+            "weights": recipe, "level_fractions": [c / packed["N"] for c in packed["counts"]],
+            "bits_per_weight": packed["bits_per_weight"], "packed_bytes": packed["total_bytes"],
+            "rank_table_bytes": table_bytes, "distinct_copies": copies,
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK, "traffic": None,
+            "note": "algorithmic bytes = packed layer + x + y per launch; time = HIP-event time of the timed region / steps",
+        },
+        "launch": "eager" if graph is None else f"hipGraph of {copies} layer launches, replayed {rounds}x",
+        "eager_per_call_us": {"median": float(np.median(per_call)), "min": float(per_call.min()),
+                        "p90": float(np.percentile(per_call, 90))},
+        "host_wall_ms_per_step": wall_ms / steps,
+        "prep_s": prep_s,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(weight, x_host)
+        out["cpu_baseline"]["speedup_vs_cpu"] = out["value"] / out["cpu_baseline"]["value"]
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

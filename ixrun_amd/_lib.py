@@ -12,11 +12,13 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "csrc", "libixhip.so")
+# IXH_LIB names another build of the library (development); the default is the in-tree one
+LIB_PATH = os.environ.get("IXH_LIB") or os.path.join(_HERE, "csrc", "libixhip.so")
 
 IXH_MAX_LEVELS = 8
 IXH_GEMV_ATOMIC = 1
 IXH_GEMV_FORCE_GENERIC = 2
+IXH_GEMV_COLUMN_KERNEL = 4
 
 ERROR_NAMES = {-1: "IXH_EINVAL", -2: "IXH_EUNSUPPORTED", -3: "IXH_ELAUNCH", -4: "IXH_EWORKSPACE"}
 

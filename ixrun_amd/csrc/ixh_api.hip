@@ -162,7 +162,10 @@ int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, cons
         }
     }
     rc = IXH_EUNSUPPORTED;
-    if (!(flags & IXH_GEMV_FORCE_GENERIC) && is_358(d) && fast358_supports(d, (uint32_t)chunk, m))
+    const bool fast = !(flags & IXH_GEMV_FORCE_GENERIC) && is_358(d) && fast358_supports(d, (uint32_t)chunk, m);
+    if (fast && !atomic && !(flags & IXH_GEMV_COLUMN_KERNEL))
+        rc = launch_gemv_358_rows(d, prefix, x, m, ldx, y, ldy, (hipStream_t)stream);
+    if (fast && rc == IXH_EUNSUPPORTED)
         rc = launch_gemv_358(d, prefix, (uint32_t)chunk, x, m, ldx, y, ldy, y32, (float *)workspace, atomic,
                              (hipStream_t)stream);
     if (rc == IXH_EUNSUPPORTED) {  // other schemes, other chunk sizes, unaligned x

@@ -11,6 +11,9 @@ bool fast358_supports(const Dev &P, uint32_t chunk, int m);
 // x / ld alignment is checked at launch; returns IXH_EUNSUPPORTED if it does not fit
 int launch_gemv_358(const Dev &P, const int32_t *prefix, uint32_t chunk, const uint16_t *x, int m, int64_t ldx,
                     uint16_t *y, int64_t ldy, float *y32, float *ws, bool atomic, hipStream_t s);
+// single-launch row-block kernel (ixh_rows358.hip); IXH_EUNSUPPORTED if the shape does not fit it
+int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
+                         int64_t ldy, hipStream_t s);
 int launch_reduce_chunks(const float *ws, uint32_t n_chunks, int m, uint32_t out_f, uint16_t *y, int64_t ldy,
                          hipStream_t s);
 

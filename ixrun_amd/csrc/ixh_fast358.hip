@@ -88,7 +88,8 @@ __device__ __forceinline__ void resolve_queue(const Dev &P, const uint4 *queue, 
             const uint32_t r = rec.x, r0u = rec.y, q2u = rec.z;
             const uint32_t slot = rec.w >> 16, koff = rec.w & 0xFFFFu;
             // level-2 elements among bitmap-1 bits [r0u, r), and the bit at r
-            const uint32_t wf = r0u >> 5, wl = r >> 5;
+            // (a unit has 512 elements, so a well-formed record spans at most 17 words)
+            const uint32_t wf = r0u >> 5, wl = min(r >> 5, wf + 17u);
             const uint32_t first_mask = ~0u << (r0u & 31);
             uint32_t cnt = 0;
             for (uint32_t w = wf; w < wl; ++w) {

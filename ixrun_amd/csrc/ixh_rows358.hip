@@ -1,0 +1,626 @@
+// (3,5,8) fused decode + GEMV for gfx950, row-block variant: one workgroup owns
+// whole rows, so the result leaves as bf16 from a single launch with no
+// workspace, no atomics in global memory and a fixed summation order.
+//
+// Work split.  The matrix is cut into 512-wide column blocks ("units" of one
+// row) and into row quads.  Wave w of a workgroup owns C neighbouring column
+// blocks and keeps its x slices in registers; the workgroup walks down its row
+// quads, each 16-lane DPP row of a wave taking one matrix row and each lane 32
+// consecutive elements (one word of bitmap 0).
+//
+// Memory pipeline.  Nothing the kernel streams depends on what it decodes: the
+// 3-bit stream range of a unit follows from the rank table alone.  The
+// workgroup first copies its slice of the table into LDS; after that
+// every wave keeps kRStages unit-quads in flight with LDS-DMA buffer loads (one
+// dword per lane of bitmap 0, and 13 x 16 bytes per row of the 3-bit stream),
+// which need no registers and are bounds-checked by the buffer descriptor.
+//
+// Decode.  Per unit a lane reads its bitmap word, ranks it with a 4-step DPP
+// scan over its row, reads its own 96-bit code window from the staged stream
+// and aligns it with three v_alignbit.  Elements that are not level 1 are
+// spliced out of the window (their field becomes the code of 0) and handed, one
+// record per lane, to a per-wave LDS queue that is resolved 64 records at a
+// time.  When the workgroup's share of bitmap 1 and of the 5-bit and 8-bit
+// streams is small (the usual case: few elements are above level 1) it is
+// staged in LDS up front and the resolution touches no global memory.  Two
+// neighbouring codes index a bank-conflict-free table of dequantised weight
+// pairs in LDS (64 entries x 32 lane copies); the packed bf16 pair meets the x
+// pair in v_dot2_f32_bf16.  The window of unit i+1 is opened while the pairs of
+// unit i are processed.
+//
+// Reduction.  Lanes sum over the wave's C blocks, rows over their 16 lanes
+// (DPP), waves through LDS after one barrier, in wave order.
+#include <stdlib.h>
+
+#include "ixh_fast358.h"
+
+namespace ixh {
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+
+constexpr int kRStages = 3;              // unit-quads in flight per wave
+constexpr uint32_t kRStageBytes = 1280;  // 1024 stream + 256 bitmap
+constexpr uint32_t kRQueue = 128;        // records per wave
+constexpr uint32_t kRSlots = 64;         // rows per workgroup at most
+constexpr int kRMaxWaves = 12;           // waves per workgroup at most: 3 per SIMD, up to 168 VGPRs each
+constexpr uint32_t kRLutBytes = 64 * 32 * 4;
+constexpr uint32_t kRSpliceBytes = 33 * 32;
+// staged share of the other streams: bitmap 1 (1 KB), 5-bit stream (2 KB), 8-bit stream (1 KB)
+constexpr uint32_t kRSideB2 = 0, kRSideL2 = 1024, kRSideL3 = 3072, kRSideBytes = 4096;
+
+constexpr uint32_t kFlagStageSide = 2u;  // the 8-bit stream is dword aligned, the side streams may be staged
+
+constexpr uint32_t kZeroCodes0 = 0xDB6DB6DBu, kZeroCodes1 = 0xB6DB6DB6u, kZeroCodes2 = 0x6DB6DB6Du;
+
+__host__ __device__ constexpr uint32_t wave_lds_bytes(int mt) {
+    return kRStages * kRStageBytes + kRQueue * 16 + kRSlots * mt * 4;
+}
+
+// byte offsets of the regions of a workgroup's LDS; the pair table is at 0, the splice masks follow
+struct RowsLds {
+    uint32_t tq1, tq2, side, waves, total;
+};
+
+__host__ __device__ inline RowsLds rows_layout(uint32_t rows_cap, uint32_t n_chunks, uint32_t n_waves, int mt) {
+    RowsLds L;
+    const uint32_t tbl = ((rows_cap * n_chunks + 1u + 3u) & ~3u) * 4u;  // one entry past the slice: its end ranks
+    L.tq1 = kRLutBytes + kRSpliceBytes;
+    L.tq2 = L.tq1 + tbl;
+    L.side = L.tq2 + tbl;
+    L.waves = L.side + kRSideBytes;
+    L.total = L.waves + n_waves * wave_lds_bytes(mt);
+    return L;
+}
+
+__device__ __forceinline__ uint32_t dpp_shr(uint32_t v, int n) {
+    switch (n) {
+        case 1: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, true);
+        case 2: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, true);
+        case 4: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, true);
+        default: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, true);
+    }
+}
+
+__device__ __forceinline__ uint32_t row_scan(uint32_t v) {
+    v += dpp_shr(v, 1);
+    v += dpp_shr(v, 2);
+    v += dpp_shr(v, 4);
+    v += dpp_shr(v, 8);
+    return v;
+}
+
+__device__ __forceinline__ float row_sum(float v) {
+    v += __uint_as_float(dpp_shr(__float_as_uint(v), 1));
+    v += __uint_as_float(dpp_shr(__float_as_uint(v), 2));
+    v += __uint_as_float(dpp_shr(__float_as_uint(v), 4));
+    v += __uint_as_float(dpp_shr(__float_as_uint(v), 8));
+    return v;
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmem() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ uint32_t lds_u32(uint32_t addr) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) uint32_t *>((uintptr_t)addr);
+}
+__device__ __forceinline__ uint32_t lds_u16(uint32_t addr) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>((uintptr_t)addr);
+}
+__device__ __forceinline__ uint32_t lds_u8(uint32_t addr) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) uint8_t *>((uintptr_t)addr);
+}
+__device__ __forceinline__ u32x4 lds_u128(uint32_t addr) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) u32x4 *>((uintptr_t)addr);
+}
+
+// where the elements above level 1 of this workgroup's rows live
+struct SideView {
+    bool staged;             // true: in LDS at `base`; false: read from global memory
+    uint32_t base;           // LDS address of the staged region
+    uint32_t b2w0, l2w0, l3w0;  // first staged word of bitmap 1 / 5-bit stream / 8-bit stream
+};
+
+// Resolve queued lanes: every record is one bitmap word with elements above
+// level 1; the lane that takes it walks those elements and adds x*w to the row sums.
+template <int MT>
+__device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, uint32_t tq1_addr, uint32_t tq2_addr,
+                                             uint32_t unit0, const uint4 *queue, uint32_t count, float *rowacc,
+                                             const uint16_t *__restrict__ x, int m,
+                                             int64_t ldx, float scale, uint32_t lane) {
+    const uint32_t *__restrict__ b2 = P.bm[1];
+    const uint32_t b2_words = P.bm_words[1];
+    for (uint32_t base = 0; base < count; base += kWave) {
+        const uint32_t idx = base + lane;
+        if (idx < count) {
+            const uint4 rec = queue[idx];
+            uint32_t zeros = rec.x;
+            const uint32_t r0_lane = rec.y, unit = rec.z;
+            const uint32_t slot = rec.w >> 16, k0 = rec.w & 0xFFFFu;
+            const uint32_t r0u = unit * kFastChunk - lds_u32(tq1_addr + (unit - unit0) * 4);
+            const uint32_t q2u = lds_u32(tq2_addr + (unit - unit0) * 4);
+            const uint32_t wf = r0u >> 5;
+            const uint32_t first_mask = ~0u << (r0u & 31);
+            uint32_t nth = 0;
+            while (zeros != 0) {
+                const uint32_t e = __builtin_ctz(zeros);
+                zeros &= zeros - 1;
+                const uint32_t r = r0_lane + nth++;
+                // level-2 elements among bitmap-1 bits [r0u, r) (a unit spans at most 17 words), and the bit at r
+                const uint32_t wl = min(r >> 5, wf + 17u);
+                uint32_t cnt = 0;
+                for (uint32_t w = wf; w < wl; ++w) {
+                    uint32_t bits = sv.staged ? lds_u32(sv.base + kRSideB2 + (w - sv.b2w0) * 4)
+                                              : (w < b2_words ? b2[w] : 0u);
+                    if (w == wf) bits &= first_mask;
+                    cnt += __popc(bits);
+                }
+                const uint32_t bits = sv.staged ? lds_u32(sv.base + kRSideB2 + (wl - sv.b2w0) * 4)
+                                                : (wl < b2_words ? b2[wl] : 0u);
+                uint32_t low = (1u << (r & 31)) - 1u;
+                if (wl == wf) low &= first_mask;
+                cnt += __popc(bits & low);
+                int v = 0;
+                if ((bits >> (r & 31)) & 1u) {
+                    const uint64_t bitpos = (uint64_t)(q2u + cnt) * 5u;
+                    const uint32_t wi = (uint32_t)(bitpos >> 5), s = (uint32_t)bitpos & 31u;
+                    uint32_t lo, hi;
+                    if (sv.staged) {
+                        lo = lds_u32(sv.base + kRSideL2 + (wi - sv.l2w0) * 4);
+                        hi = lds_u32(sv.base + kRSideL2 + (wi - sv.l2w0) * 4 + 4);
+                    } else {
+                        lo = wi < P.st_words[1] ? P.st[1][wi] : 0u;
+                        hi = (s > 27 && wi + 1 < P.st_words[1]) ? P.st[1][wi + 1] : 0u;
+                    }
+                    v = (int)((uint32_t)((((uint64_t)hi << 32) | lo) >> s) & 31u) - 15;
+                } else {
+                    const uint32_t i3 = r - (q2u + cnt);
+                    // (the staged copy is made of whole dwords: the stream's last 1..3 bytes come from memory)
+                    if (sv.staged && i3 < (P.last_bytes & ~3u)) v = (int)lds_u8(sv.base + kRSideL3 + (i3 - sv.l3w0 * 4)) - 127;
+                    else v = i3 < P.last_bytes ? (int)P.last[i3] - 127 : 0;
+                }
+                const float w = dequant(v, scale);
+#pragma unroll
+                for (int j = 0; j < MT; ++j) {
+                    if (j < m) {
+                        atomicAdd(&rowacc[slot * MT + j], bf16_bits_to_f32(x[(int64_t)j * ldx + k0 + e]) * w);
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int MT, int C>
+__global__ void __launch_bounds__(kRMaxWaves * kWave)
+k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t quads_per_wg_arg, uint32_t flags,
+               const uint16_t *__restrict__ x, int m, int64_t ldx, uint16_t *__restrict__ y, int64_t ldy
+#ifdef IXH_VARIANTS
+               , unsigned long long *trace
+#endif
+               ) {
+#ifdef IXH_VARIANTS  // timing experiments only: stamps, and bits 16.. of the argument switch parts off
+#define IXH_STAMP(k) do { if (trace && threadIdx.x == 0) trace[blockIdx.x * 8 + (k)] = wall_clock64(); } while (0)
+    const uint32_t dbg = quads_per_wg_arg >> 16, quads_per_wg = quads_per_wg_arg & 0xFFFFu;
+#else
+#define IXH_STAMP(k) do { } while (0)
+    constexpr uint32_t dbg = 0;
+    const uint32_t quads_per_wg = quads_per_wg_arg;
+#endif
+    IXH_STAMP(0);
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t n_waves = blockDim.x >> 6;
+    const uint32_t quarter = lane >> 4, li = lane & 15;
+
+    const uint32_t n_quads = (P.out_f + 3) >> 2;
+    const uint32_t quad0 = blockIdx.x * quads_per_wg;
+    const uint32_t n_steps = min(quads_per_wg, n_quads - quad0);
+    const uint32_t row0 = quad0 * 4;
+    const uint32_t rows_here = min(n_steps * 4, P.out_f - row0);
+    const RowsLds L = rows_layout(min(quads_per_wg * 4, P.out_f), n_chunks, n_waves, MT);
+
+    // The pair table is addressed with (index bits | lane bits), which needs it at
+    // LDS address 0; that holds because the kernel has no other LDS.  Should it
+    // ever not hold, say so in the output instead of computing garbage.
+    if ((uint32_t)(uintptr_t)(lds_ptr_t)smem != 0) {
+        for (uint32_t t = tid; t < rows_here * MT; t += blockDim.x)
+            if ((int)(t % MT) < m) y[(int64_t)(t % MT) * ldy + row0 + t / MT] = 0x7FC0;  // NaN
+        return;
+    }
+    uint32_t *const lut = reinterpret_cast<uint32_t *>(smem);            // [64][32]
+    uint4 *const splice = reinterpret_cast<uint4 *>(smem + kRLutBytes);  // [33][2]
+    uint32_t *const tq1 = reinterpret_cast<uint32_t *>(smem + L.tq1);
+    uint32_t *const tq2 = reinterpret_cast<uint32_t *>(smem + L.tq2);
+    uint8_t *const wave_base = smem + L.waves + wave * wave_lds_bytes(MT);
+    uint8_t *const ring = wave_base;
+    uint4 *const queue = reinterpret_cast<uint4 *>(wave_base + kRStages * kRStageBytes);
+    float *const rowacc = reinterpret_cast<float *>(wave_base + kRStages * kRStageBytes + kRQueue * 16);
+
+    // ---- workgroup set-up: table slices and x first (they wait on memory), then the tables built here ----
+    const uint32_t unit0 = row0 * n_chunks;
+    const uint32_t entries = P.out_f * n_chunks + 1;
+    if (!(dbg & 16))
+        for (uint32_t i = tid; i <= rows_here * n_chunks; i += blockDim.x) {
+            tq1[i] = (uint32_t)prefix[unit0 + i];
+            tq2[i] = (uint32_t)prefix[entries + unit0 + i];
+        }
+    const float scale = bf16_bits_to_f32(*P.scale);
+    if (!(dbg & 8))
+        for (uint32_t i = tid; i < 64 * 32; i += blockDim.x) {
+            const int c0 = (i >> 5) & 7, c1 = i >> 8;
+            const uint32_t w0 = c0 < 7 ? f32_to_bf16_bits((float)(c0 - 3) * scale) : 0u;
+            const uint32_t w1 = c1 < 7 ? f32_to_bf16_bits((float)(c1 - 3) * scale) : 0u;
+            lut[i] = w0 | (w1 << 16);
+        }
+    if (tid <= 32) {
+        // entry e < 32: masks for a zero at element e (code bits 3e..3e+2): the bits below it, and its field;
+        // entry 32: the identity (nothing to splice)
+        const uint32_t pos = 3 * tid;
+        uint32_t lm[3], f[3];
+#pragma unroll
+        for (int d = 0; d < 3; ++d) {
+            const uint32_t base = 32u * d;
+            lm[d] = pos <= base ? 0u : (pos >= base + 32 ? ~0u : (1u << (pos - base)) - 1u);
+            f[d] = (pos + 3 <= base || pos >= base + 32) ? 0u : (pos >= base ? 7u << (pos - base) : 7u >> (base - pos));
+        }
+        splice[2 * tid] = make_uint4(lm[0], lm[1], lm[2], 0u);
+        splice[2 * tid + 1] = make_uint4(f[0], f[1], f[2], 0u);
+    }
+    for (uint32_t j = lane; j < kRSlots * MT; j += kWave) rowacc[j] = 0.0f;
+    __syncthreads();
+    IXH_STAMP(1);
+
+    const uint32_t col0 = wave * C;
+
+    // this lane's activations: C blocks x MT rows x 16 packed bf16 pairs
+    uint32_t xr[C][MT][16];
+#pragma unroll
+    for (int cc = 0; cc < C; ++cc) {
+        const uint32_t col = min(col0 + cc, n_chunks - 1);
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            if (j < m && !(dbg & 32)) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const uint4 v = reinterpret_cast<const uint4 *>(x + (int64_t)j * ldx + col * kFastChunk + li * 32)[t];
+                    xr[cc][j][4 * t] = v.x; xr[cc][j][4 * t + 1] = v.y;
+                    xr[cc][j][4 * t + 2] = v.z; xr[cc][j][4 * t + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 16; ++t) xr[cc][j][t] = 0u;
+            }
+        }
+    }
+
+    const __amdgpu_buffer_rsrc_t b1_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[0], 0, (int)(P.bm_words[0] * 4u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t l1_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[0], 0, (int)(P.st_words[0] * 4u), 0x00020000);
+
+    // ---- this workgroup's share of bitmap 1 and of the 5-bit / 8-bit streams ----
+    // Its extent follows from the ranks at the first and one past the last row.  If it fits, every wave
+    // DMAs all of it (same bytes to the same place, so no barrier is needed: a wave's own loads
+    // complete in order, before the first unit it waits for).
+    SideView sv;
+    {
+        const uint32_t n_local = rows_here * n_chunks;
+        const uint32_t q1b = tq1[0], q2b = tq2[0], q1e = tq1[n_local], q2e = tq2[n_local];
+        const uint32_t nl1b = row0 * P.in_f - q1b, nl1e = (row0 + rows_here) * P.in_f - q1e;
+        sv.base = L.side;
+        sv.b2w0 = nl1b >> 5;
+        sv.l2w0 = (uint32_t)(((uint64_t)q2b * 5u) >> 5);
+        sv.l3w0 = (nl1b - q2b) >> 2;
+        const uint32_t n_b2 = ((nl1e + 31) >> 5) - sv.b2w0;
+        const uint32_t n_l2 = (uint32_t)((((uint64_t)q2e * 5u) + 31) >> 5) - sv.l2w0;
+        const uint32_t n_l3 = ((nl1e - q2e + 3) >> 2) - sv.l3w0;
+        // one word of slack each: the resolver reads the word after a code's first word unconditionally
+        sv.staged = (flags & kFlagStageSide) && n_b2 < 256 && n_l2 < 511 && n_l3 <= 256;
+        if (sv.staged) {
+            const __amdgpu_buffer_rsrc_t b2_rsrc =
+                __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[1], 0, (int)(P.bm_words[1] * 4u), 0x00020000);
+            const __amdgpu_buffer_rsrc_t l2_rsrc =
+                __builtin_amdgcn_make_buffer_rsrc((void *)P.st[1], 0, (int)(P.st_words[1] * 4u), 0x00020000);
+            const __amdgpu_buffer_rsrc_t l3_rsrc =
+                __builtin_amdgcn_make_buffer_rsrc((void *)P.last, 0, (int)P.last_bytes, 0x00020000);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(b2_rsrc, (lds_ptr_t)(smem + L.side + kRSideB2), 16,
+                                                     (int)(sv.b2w0 * 4 + lane * 16), 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(l2_rsrc, (lds_ptr_t)(smem + L.side + kRSideL2), 16,
+                                                     (int)(sv.l2w0 * 4 + lane * 16), 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(l2_rsrc, (lds_ptr_t)(smem + L.side + kRSideL2 + 1024), 16,
+                                                     (int)(sv.l2w0 * 4 + 1024 + lane * 16), 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(l3_rsrc, (lds_ptr_t)(smem + L.side + kRSideL3), 16,
+                                                     (int)(sv.l3w0 * 4 + lane * 16), 0, 0, 0);
+        }
+    }
+
+    const uint32_t lut_lane = (lane & 31u) << 2;
+    const uint32_t splice_addr = kRLutBytes;
+    const uint32_t tq1_addr = L.tq1, tq2_addr = L.tq2;
+    const uint32_t ring_addr = (uint32_t)(uintptr_t)(lds_ptr_t)ring;
+
+    // Unit-quads of this wave in walk order: index i -> (step i / C, block i % C).
+    const uint32_t n_units = n_steps * C;
+
+    // ---- producer: LDS-DMA of unit-quad i into ring stage i % kRStages ----
+    uint32_t i_step = 0, i_cc = 0;                            // (step, block) of the next unit to issue
+    uint32_t i_lrn = min(quarter, rows_here - 1) * n_chunks;  // its local row * n_chunks, per lane
+    auto issue = [&](uint32_t i) {
+        const uint32_t col = min(col0 + i_cc, n_chunks - 1);
+        const uint32_t q1u = lds_u32(tq1_addr + (i_lrn + col) * 4);
+        const uint32_t unit = unit0 + i_lrn + col;
+        uint8_t *stage = ring + (i % kRStages) * kRStageBytes;
+        asm volatile("" ::: "memory");
+        if (li < 13)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(l1_rsrc, (lds_ptr_t)stage, 16,
+                                                     (int)(((q1u * 3u) >> 5) * 4u + li * 16u), 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(b1_rsrc, (lds_ptr_t)(stage + 1024), 4,
+                                                 (int)((unit * 16u + li) * 4u), 0, 0, 0);
+        if (++i_cc == C) {
+            i_cc = 0;
+            ++i_step;
+            i_lrn = min(4 * i_step + quarter, rows_here - 1) * n_chunks;
+        }
+    };
+
+    uint32_t qcount = 0;  // wave-uniform
+
+    // one splice of the 96-bit window at the lowest zero bit left in zrem (identity when none is left)
+    auto splice_once = [&](uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &zrem) {
+        const uint32_t e = zrem != 0 ? (uint32_t)__builtin_ctz(zrem) : 32u;
+        zrem &= zrem - 1;
+        const u32x4 lm = lds_u128(splice_addr + e * 32), fm = lds_u128(splice_addr + e * 32 + 16);
+        const uint32_t s0 = w0 << 3;
+        const uint32_t s1 = __builtin_amdgcn_alignbit(w1, w0, 29);
+        const uint32_t s2 = __builtin_amdgcn_alignbit(w2, w1, 29);
+        w0 = (w0 & lm.x) | (s0 & ~lm.x);
+        w1 = (w1 & lm.y) | (s1 & ~lm.y);
+        w2 = (w2 & lm.z) | (s2 & ~lm.z);
+        w0 = (w0 & ~fm.x) | (kZeroCodes0 & fm.x);
+        w1 = (w1 & ~fm.y) | (kZeroCodes1 & fm.y);
+        w2 = (w2 & ~fm.z) | (kZeroCodes2 & fm.z);
+    };
+
+    // ---- consumer, first half: code window of unit-quad i (its data is in the ring), spliced once ----
+    auto open_window = [&](uint32_t i, uint32_t slot, uint32_t lrn, bool valid, uint32_t cc, uint32_t &w0,
+                           uint32_t &w1, uint32_t &w2, uint32_t &zrem) {
+        valid = valid && (col0 + cc < n_chunks);
+        const uint32_t col = min(col0 + cc, n_chunks - 1);
+        const uint32_t stage = ring_addr + (i % kRStages) * kRStageBytes;
+        const uint32_t word = lds_u32(stage + 1024 + lane * 4);
+        const uint32_t q1u = lds_u32(tq1_addr + (lrn + col) * 4);
+        const uint32_t c = __popc(word);
+        const uint32_t excl = row_scan(c) - c;
+        const uint32_t off = excl * 3u + ((q1u * 3u) & 31u);  // bit offset inside the staged stream piece
+        const uint32_t wa = stage + quarter * 256 + (off >> 5) * 4;
+        const uint32_t d0 = lds_u32(wa), d1 = lds_u32(wa + 4), d2 = lds_u32(wa + 8), d3 = lds_u32(wa + 12);
+        w0 = __builtin_amdgcn_alignbit(d1, d0, off);
+        w1 = __builtin_amdgcn_alignbit(d2, d1, off);
+        w2 = __builtin_amdgcn_alignbit(d3, d2, off);
+        uint32_t zeros = ~word;
+        if (!valid) {
+            zeros = 0u;
+            w0 = kZeroCodes0; w1 = kZeroCodes1; w2 = kZeroCodes2;
+        }
+        // lanes with elements above level 1 leave a record (the loop head keeps 64 slots free)
+        const uint64_t any = __ballot(zeros != 0);
+        if (zeros != 0) {
+            const uint32_t unit = unit0 + lrn + col;
+            const uint32_t r0_lane = unit * kFastChunk + li * 32u - (q1u + excl);
+            queue[qcount + lanes_below(any)] =
+                make_uint4(zeros, r0_lane, unit, (slot << 16) | (col * kFastChunk + li * 32u));
+        }
+        qcount += (uint32_t)__popcll(any);
+        zrem = zeros;
+        splice_once(w0, w1, w2, zrem);
+    };
+
+    auto resolve = [&]() {
+        resolve_rows<MT>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc, x, m, ldx, scale,
+                         lane);
+        qcount = 0;
+    };
+
+    // ---- start-up: fill the ring, open the first window ----
+    const uint32_t n_pre = min((uint32_t)kRStages, n_units);
+    for (uint32_t i = 0; i < n_pre; ++i) issue(i);
+    if (n_units >= (uint32_t)kRStages) wait_vmem<2 * (kRStages - 1)>();
+    else wait_vmem<0>();
+    IXH_STAMP(2);
+
+    uint32_t lrn_step = min(quarter, rows_here - 1) * n_chunks;  // local row * n_chunks of the current step
+    bool valid_step = quarter < rows_here;
+    uint32_t cw0, cw1, cw2, czrem;
+    open_window(0, quarter, lrn_step, valid_step, 0, cw0, cw1, cw2, czrem);
+    while (__ballot(czrem != 0) != 0) splice_once(cw0, cw1, cw2, czrem);
+
+    constexpr int NA = MT == 1 ? 4 : (MT == 2 ? 2 : 1);  // independent accumulators per x row
+
+    for (uint32_t step = 0; step < n_steps; ++step) {
+        float acc[MT][NA];
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+#pragma unroll
+            for (int a = 0; a < NA; ++a) acc[j][a] = 0.0f;
+        const uint32_t lrn_next = min(4 * (step + 1) + quarter, rows_here - 1) * n_chunks;
+        const bool valid_next = 4 * (step + 1) + quarter < rows_here;
+
+#pragma unroll
+        for (int cc = 0; cc < C; ++cc) {
+            const uint32_t i = step * C + cc;
+            if (qcount > kRQueue - kWave) resolve();  // keep room for a full wave of records
+            // refill the stage whose window was read last time; make unit i+1 readable
+            if (!(dbg & 4)) {
+                if (i + kRStages < n_units) {
+                    issue(i + kRStages);
+                    wait_vmem<2 * (kRStages - 1)>();
+                } else {
+                    wait_vmem<0>();
+                }
+            }
+
+            // window of unit i+1 (or, past the end, a void one) ...
+            uint32_t nw0 = cw0 + 1, nw1 = cw1 + 1, nw2 = cw2, nzrem = 0;
+            if (!(dbg & 2)) {
+                const bool last_cc = cc == C - 1;
+                const uint32_t n_i = min(i + 1, n_units - 1);
+                open_window(n_i, 4 * (last_cc ? step + 1 : step) + quarter, last_cc ? lrn_next : lrn_step,
+                            (last_cc ? valid_next : valid_step) && (i + 1 < n_units), last_cc ? 0 : cc + 1, nw0, nw1,
+                            nw2, nzrem);
+            }
+
+            // ... while the 16 code pairs of unit i go through the pair table and meet the x pairs
+            if (!(dbg & 1))
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const int bit = 6 * t, ob = bit & 31, d = bit >> 5;
+                const uint32_t lo = d == 0 ? cw0 : (d == 1 ? cw1 : cw2);
+                const uint32_t hi = d == 0 ? cw1 : cw2;
+                uint32_t a;  // pair index at bits 12..7
+                if (ob > 26) a = __builtin_amdgcn_alignbit(hi, lo, ob - 7);
+                else if (ob >= 7) a = lo >> (ob - 7);
+                else a = lo << (7 - ob);
+                const uint32_t wp = lds_u32((a & 0x1F80u) | lut_lane);
+#pragma unroll
+                for (int j = 0; j < MT; ++j)
+                    acc[j][t % NA] = __builtin_amdgcn_fdot2_f32_bf16(
+                        __builtin_bit_cast(bf16x2, wp), __builtin_bit_cast(bf16x2, xr[cc][j][t]), acc[j][t % NA], false);
+            }
+
+            // lanes with more than one element above level 1 (rare): splice on
+            while (__ballot(nzrem != 0) != 0) splice_once(nw0, nw1, nw2, nzrem);
+            cw0 = nw0; cw1 = nw1; cw2 = nw2;
+        }
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            float sum = acc[j][0];
+#pragma unroll
+            for (int a = 1; a < NA; ++a) sum += acc[j][a];
+            const float total = row_sum(sum);
+            if (li == 15) rowacc[(4 * step + quarter) * MT + j] += total;
+        }
+        lrn_step = lrn_next;
+        valid_step = valid_next;
+    }
+
+    IXH_STAMP(3);
+#ifdef IXH_VARIANTS
+    if (trace && lane == 0) trace[4096 + blockIdx.x * 32 + wave * 2] = wall_clock64();
+#endif
+    resolve();
+#ifdef IXH_VARIANTS
+    if (trace && lane == 0) trace[4096 + blockIdx.x * 32 + wave * 2 + 1] = wall_clock64();
+#endif
+    IXH_STAMP(4);
+    __syncthreads();
+    IXH_STAMP(5);
+
+    // ---- add the waves' row sums in wave order, write bf16 ----
+    if (dbg & 64) return;
+    const uint32_t first_acc = L.waves + kRStages * kRStageBytes + kRQueue * 16;
+    for (uint32_t t = tid; t < rows_here * MT; t += blockDim.x) {
+        const uint32_t slot = t / MT, j = t - slot * MT;
+        if ((int)j >= m) continue;
+        float sum = 0.0f;
+        for (uint32_t w = 0; w < n_waves; ++w)
+            sum += *reinterpret_cast<const float *>(smem + first_acc + w * wave_lds_bytes(MT) + t * 4);
+        y[(int64_t)j * ldy + row0 + slot] = (uint16_t)f32_to_bf16_bits(sum);
+    }
+    IXH_STAMP(6);
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+#ifdef IXH_VARIANTS
+static unsigned long long *g_trace = nullptr;
+extern "C" int ixh_debug_trace(unsigned long long *host_out, int n) {
+    if (!g_trace) return -1;
+    return hipMemcpy(host_out, g_trace, (size_t)n * 8, hipMemcpyDeviceToHost) == hipSuccess ? 0 : -2;
+}
+#endif
+
+static int env_int(const char *name) {
+    const char *e = getenv(name);
+    return e ? atoi(e) : 0;
+}
+
+constexpr size_t kLdsLimit = 160 * 1024;
+
+template <int MT, int C>
+static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, const uint16_t *x, int m,
+                       int64_t ldx, uint16_t *y, int64_t ldy, hipStream_t s) {
+    static const int forced_quads = env_int("IXH_QUADS_PER_WG");
+    const uint32_t waves = (n_chunks + C - 1) / C;
+    const uint32_t n_quads = (P.out_f + 3) / 4;
+    // how many workgroups a CU holds, by registers and LDS (asked once per workgroup size)
+    static int per_cu_cache[17] = {0};
+    int per_cu = per_cu_cache[waves];
+    if (per_cu == 0) {
+        const size_t probe = rows_layout(min(16u, P.out_f), n_chunks, waves, MT).total;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rows<MT, C>, (int)(waves * kWave), probe) !=
+                hipSuccess || per_cu < 1)
+            per_cu = -1;
+        per_cu_cache[waves] = per_cu;
+    }
+    if (per_cu < 1) return IXH_EUNSUPPORTED;
+    static const int n_cu = [] {
+        int dev = 0, v = 256;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
+        return v;
+    }();
+    // one resident set of workgroups, each with a contiguous run of row quads
+    const uint32_t resident = (uint32_t)n_cu * (uint32_t)per_cu;
+    uint32_t quads = forced_quads > 0 ? (uint32_t)forced_quads : (n_quads + resident - 1) / resident;
+    quads = max(1u, min(quads, kRSlots / 4));
+    const uint32_t groups = (n_quads + quads - 1) / quads;
+    const uint32_t rows_cap = min(quads * 4, P.out_f);
+    uint32_t flags = 0;
+    if (((uintptr_t)P.last & 3u) == 0) flags |= kFlagStageSide;
+    const size_t lds = rows_layout(rows_cap, n_chunks, waves, MT).total;
+    if (lds > kLdsLimit) return IXH_EUNSUPPORTED;
+    if (lds > 64 * 1024) {
+        static bool raised = false;  // per instantiation
+        if (!raised) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_rows<MT, C>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit) != hipSuccess)
+                return IXH_EUNSUPPORTED;
+            raised = true;
+        }
+    }
+#ifdef IXH_VARIANTS
+    static const int dbg = env_int("IXH_DBG");
+    if (!g_trace) (void)hipMalloc(&g_trace, 4096 * 8 * 8);
+    hipLaunchKernelGGL((k_gemv358_rows<MT, C>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks,
+                       quads | ((uint32_t)dbg << 16), flags, x, m, ldx, y, ldy, g_trace);
+#else
+    hipLaunchKernelGGL((k_gemv358_rows<MT, C>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks, quads,
+                       flags, x, m, ldx, y, ldy);
+#endif
+    return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
+}
+
+// Row-block kernel for the shapes whose x slices fit the register budget of a
+// full workgroup; IXH_EUNSUPPORTED sends the caller to the column kernel.
+int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
+                         int64_t ldy, hipStream_t s) {
+    if (((uintptr_t)x & 15u) != 0 || (m > 1 && (ldx & 7) != 0)) return IXH_EUNSUPPORTED;
+    const uint32_t n_chunks = P.in_f / kFastChunk;
+    const uint32_t c = (n_chunks + kRMaxWaves - 1) / kRMaxWaves;  // blocks per wave: a workgroup has at most kRMaxWaves waves
+    const int mt = m == 1 ? 1 : (m == 2 ? 2 : (m <= 4 ? 4 : 0));
+#define IXH_ROWS(MTV, CV) \
+    if (mt == MTV && c == CV) return launch_rows<MTV, CV>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
+    IXH_ROWS(1, 1) IXH_ROWS(1, 2) IXH_ROWS(1, 3) IXH_ROWS(1, 4)
+    IXH_ROWS(2, 1) IXH_ROWS(2, 2)
+    IXH_ROWS(4, 1)
+#undef IXH_ROWS
+    return IXH_EUNSUPPORTED;
+}
+
+}  // namespace ixh
