@@ -93,6 +93,8 @@ def main():
     ap.add_argument("--copies", type=int, default=0, help="distinct packed copies to rotate over (0 = enough for 600 MB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of hipGraph replays")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three 256 MiB device copies (known traffic) so that counter runs can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (one MI355X holds the whole layer); "
@@ -124,6 +126,13 @@ def main():
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
+    if args.calibrate_copy:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # One pass over all copies is captured as a hipGraph (the per-layer launches
     # of a decode step are replayed the same way); the timed region replays it.
