@@ -35,6 +35,8 @@ WORKLOADS = {
     "gate_up_17408x5120_m4_student_t": (17408, 5120, 4, "student_t"),
     "gate_up_17408x5120_m8_student_t": (17408, 5120, 8, "student_t"),
     "gate_up_17408x5120_m16_student_t": (17408, 5120, 16, "student_t"),
+    # 64 distinct 5120x5120 layers chained (each output feeds the next layer), one hipGraph: us per layer
+    "graph64_5120x5120_m1_student_t": (5120, 5120, 1, "student_t"),
 }
 
 
@@ -111,7 +113,8 @@ def main():
     weight = make_weight(out_f, in_f, recipe)
     packed = int8x_quantize(weight)
     prep_s = time.perf_counter() - t0
-    copies = args.copies or max(2, -(-600_000_000 // packed["total_bytes"]))
+    chained = args.workload.startswith("graph64")
+    copies = args.copies or (64 if chained else max(2, -(-600_000_000 // packed["total_bytes"])))
     layers = [StreamingLinear(packed) for _ in range(copies)]
     g = torch.Generator("cpu").manual_seed(1)
     x_host = torch.randn(m, in_f, generator=g).bfloat16()
@@ -120,8 +123,15 @@ def main():
     # algorithmic bytes of one step: the packed layer, the activations in, the outputs out
     alg_bytes = packed["total_bytes"] + m * in_f * 2 + m * out_f * 2
 
+    state = {"h": x}
+
     def step(i):
-        return layers[i % copies](x)
+        if not chained:
+            return layers[i % copies](x)
+        if i % copies == 0:
+            state["h"] = x
+        state["h"] = layers[i % copies](state["h"])  # the layer's output is the next layer's input
+        return state["h"]
 
     for i in range(args.warmup):
         step(i)

@@ -19,6 +19,7 @@ IXH_MAX_LEVELS = 8
 IXH_GEMV_ATOMIC = 1
 IXH_GEMV_FORCE_GENERIC = 2
 IXH_GEMV_COLUMN_KERNEL = 4
+IXH_GEMV_FORCE_358 = 8
 
 ERROR_NAMES = {-1: "IXH_EINVAL", -2: "IXH_EUNSUPPORTED", -3: "IXH_ELAUNCH", -4: "IXH_EWORKSPACE"}
 

@@ -162,7 +162,11 @@ int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, cons
         }
     }
     rc = IXH_EUNSUPPORTED;
-    const bool fast = !(flags & IXH_GEMV_FORCE_GENERIC) && is_358(d) && fast358_supports(d, (uint32_t)chunk, m);
+    // The (3,5,8) kernels are built for tensors that are almost all level 1 (every other element costs
+    // them a queue record); denser mixes go to the general kernel unless the caller insists.
+    const bool mostly_l1 = (uint64_t)d.st_words[0] * 32u / 3u >= (uint64_t)d.n / 100u * 97u;
+    const bool fast = !(flags & IXH_GEMV_FORCE_GENERIC) && is_358(d) && fast358_supports(d, (uint32_t)chunk, m) &&
+                      (mostly_l1 || (flags & (IXH_GEMV_COLUMN_KERNEL | IXH_GEMV_FORCE_358)));
     if (fast && !atomic && !(flags & IXH_GEMV_COLUMN_KERNEL))
         rc = launch_gemv_358_rows(d, prefix, x, m, ldx, y, ldy, (hipStream_t)stream);
     if (fast && rc == IXH_EUNSUPPORTED)

@@ -575,9 +575,11 @@ static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, c
         if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
         return v;
     }();
-    // one resident set of workgroups, each with a contiguous run of row quads
+    // whole rounds of resident workgroups, each workgroup with a contiguous run of at most 16 row quads:
+    // a last round with a few workgroups in it would cost as much as a full one
     const uint32_t resident = (uint32_t)n_cu * (uint32_t)per_cu;
-    uint32_t quads = forced_quads > 0 ? (uint32_t)forced_quads : (n_quads + resident - 1) / resident;
+    const uint32_t rounds = (n_quads + resident * (kRSlots / 4) - 1) / (resident * (kRSlots / 4));
+    uint32_t quads = forced_quads > 0 ? (uint32_t)forced_quads : (n_quads + rounds * resident - 1) / (rounds * resident);
     quads = max(1u, min(quads, kRSlots / 4));
     const uint32_t groups = (n_quads + quads - 1) / quads;
     const uint32_t rows_cap = min(quads * 4, P.out_f);
