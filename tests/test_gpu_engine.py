@@ -1,0 +1,97 @@
+"""Deploy modes of the engine over a toy model (the reference needs a HF checkpoint here;
+the deploy helpers take any nn.Module): cached, streaming with the packed-weight cache
+file, graph.  Outputs are compared with the same model run on plain int8-dequantised
+weights, the reference's own equivalence claim (tests/test_int8_equivalence.py:29-33)."""
+import copy
+
+import pytest
+import torch
+import torch.nn as nn
+
+from helpers import outlier_weight
+
+pytestmark = pytest.mark.gpu
+
+
+def toy_model():
+    torch.manual_seed(0)
+    model = nn.Sequential()
+    model.add_module("proj_in", nn.Linear(512, 1024, bias=True))
+    model.add_module("act", nn.GELU())
+    model.add_module("proj_out", nn.Linear(1024, 512, bias=False))
+    model.add_module("lm_head", nn.Linear(512, 64, bias=False))  # skipped by name
+    model.add_module("tiny", nn.Linear(64, 8))                   # skipped by size
+    with torch.no_grad():
+        model.proj_in.weight.copy_(outlier_weight(1024, 512, seed=1).float())
+        model.proj_out.weight.copy_(outlier_weight(512, 1024, seed=2).float())
+    return model.bfloat16()
+
+
+def int8_reference(model):
+    ref = copy.deepcopy(model)
+    with torch.no_grad():
+        for name in ("proj_in", "proj_out"):
+            w = getattr(ref, name).weight
+            scale = w.abs().max().clamp(min=1e-8) / 127.0
+            i8 = (w.float() / scale).round().clamp(-127, 127)
+            w.copy_((i8 * scale.bfloat16().float()).to(torch.bfloat16))
+    return ref.cuda()
+
+
+def close(a, b):
+    return (a.float() - b.float()).abs().max() <= 2e-2 * b.float().abs().max()
+
+
+@pytest.mark.parametrize("rows", [1, 3, 40])
+def test_deploy_modes(tmp_path, rows):
+    from ixrun_amd.engine import GraphLinear, Int8XEngine, StreamingLinear
+    from ixrun_amd.linear import Int8XLinear
+
+    x = torch.randn(rows, 512, generator=torch.Generator().manual_seed(5)).bfloat16().cuda()
+    base = toy_model()
+    want = int8_reference(base)(x)
+
+    cached = copy.deepcopy(base).cuda()
+    stats = Int8XEngine._deploy_cached(cached, (3, 5, 8), verbose=False)
+    assert stats["n_layers"] == 2 and isinstance(cached.proj_in, Int8XLinear) and isinstance(cached.lm_head, nn.Linear)
+    assert torch.equal(cached.proj_out._w.cpu(), int8_reference(base).proj_out.weight.cpu())  # bit-exact weights
+    assert close(cached(x), want)
+
+    cache = str(tmp_path / "packed.pt")
+    streaming = copy.deepcopy(base)
+    stats = Int8XEngine._deploy_streaming(streaming, (3, 5, 8), verbose=False, cache_path=cache)
+    assert stats["mode"] == "streaming" and stats["n_layers"] == 2 and isinstance(streaming.proj_in, StreamingLinear)
+    streaming = streaming.cuda()
+    assert close(streaming(x), want)
+    again = copy.deepcopy(base)
+    Int8XEngine._deploy_streaming(again, (3, 5, 8), verbose=False, cache_path=cache)  # now read from the file
+    assert torch.equal(again.cuda()(x), streaming(x))
+    with pytest.raises(ValueError, match="level_bits"):
+        Int8XEngine._deploy_streaming(copy.deepcopy(base), (3, 4, 5, 6, 8), verbose=False, cache_path=cache)
+    other = nn.Sequential(nn.Linear(512, 1024))
+    with pytest.raises(ValueError, match="mismatch"):
+        Int8XEngine._deploy_streaming(other.bfloat16(), (3, 5, 8), verbose=False, cache_path=cache)
+
+    graph_model = copy.deepcopy(base)
+    stats, replay = Int8XEngine._deploy_graph(graph_model, (3, 5, 8), verbose=False)
+    assert stats["mode"] == "graph" and isinstance(graph_model.proj_in, GraphLinear)
+    graph_model = graph_model.cuda()
+    for _ in range(3):
+        replay()
+        torch.cuda.synchronize()
+        assert close(graph_model(x), want)
+
+
+def test_five_level_streaming_linear():
+    from ixrun_amd.engine import StreamingLinear
+    from ixrun_amd.quantize import int8x_quantize, decode_to_weight
+
+    w = outlier_weight(256, 768, seed=7)
+    p = int8x_quantize(w, (3, 4, 5, 6, 8))
+    sl = StreamingLinear(p)
+    sl._set_shared_buf(torch.empty(p["N"], dtype=torch.bfloat16, device="cuda"))
+    assert torch.equal(sl._decode().cpu(), decode_to_weight(p))
+    for rows in (1, 5, 64):
+        x = torch.randn(rows, 768, generator=torch.Generator().manual_seed(rows)).bfloat16().cuda()
+        want = torch.nn.functional.linear(x.float().cpu(), decode_to_weight(p).float())
+        assert close(sl(x).cpu(), want)
