@@ -121,6 +121,25 @@ int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, cons
 
 size_t ixh_gemv_workspace_bytes(const IxhPacked *packed, int64_t chunk, int32_t m, uint32_t flags);
 
+/*
+ * Fused decode + GEMM for many activation rows (prefill, m > 16 in the reference's
+ * dispatch): y[j, r] = bf16( sum_k f32(x[j, k]) * f32(w[r, k]) ) with
+ * w = bf16(f32(v) * f32(scale)) decoded into on-chip memory tile by tile and multiplied
+ * on the matrix cores (bf16 x bf16, fp32 accumulate).  Replaces the decode-to-bf16 +
+ * F.linear pair of StreamingLinear.forward (ixrun/engine.py:171-173) and of
+ * GraphLinear.forward (ixrun/engine.py:214-233), which materialise the whole bf16
+ * weight in device memory first.  Any m >= 1; x is bf16 [m, ldx], y is bf16 [m, ldy].
+ * The table must come from ixh_prefix_build(packed, 512).  Needs in_f a multiple of
+ * 512 with in_f >= 4096, x 16-byte aligned with ldx a multiple of 8, and the last-level
+ * stream 4-byte aligned; otherwise IXH_EUNSUPPORTED (the caller then decodes with
+ * ixh_decode and multiplies itself).  K is cut into 8 slices whose fp32 partial sums are
+ * combined in slice order through `workspace` (ixh_gemm_workspace_bytes).
+ */
+int ixh_gemm(const IxhPacked *packed, const int32_t *prefix, const uint16_t *x, int32_t m, int64_t ldx,
+             uint16_t *y, int64_t ldy, void *workspace, size_t workspace_bytes, ixh_stream_t stream);
+
+size_t ixh_gemm_workspace_bytes(const IxhPacked *packed, int32_t m);
+
 #ifdef __cplusplus
 }
 #endif

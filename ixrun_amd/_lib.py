@@ -21,6 +21,7 @@ IXH_GEMV_FORCE_GENERIC = 2
 IXH_GEMV_COLUMN_KERNEL = 4
 IXH_GEMV_FORCE_358 = 8
 
+IXH_EUNSUPPORTED = -2
 ERROR_NAMES = {-1: "IXH_EINVAL", -2: "IXH_EUNSUPPORTED", -3: "IXH_ELAUNCH", -4: "IXH_EWORKSPACE"}
 
 
@@ -52,7 +53,7 @@ _lib = None
 
 EXPORTS = (
     "ixh_version", "ixh_last_error", "ixh_prefix_entries", "ixh_prefix_build", "ixh_decode",
-    "ixh_gemv", "ixh_gemv_workspace_bytes",
+    "ixh_gemv", "ixh_gemv_workspace_bytes", "ixh_gemm", "ixh_gemm_workspace_bytes",
 )
 
 
@@ -81,6 +82,13 @@ def lib() -> C.CDLL:
         ]
         L.ixh_gemv_workspace_bytes.restype = C.c_size_t
         L.ixh_gemv_workspace_bytes.argtypes = [C.POINTER(IxhPacked), C.c_int64, C.c_int32, C.c_uint32]
+        L.ixh_gemm.restype = C.c_int
+        L.ixh_gemm.argtypes = [
+            C.POINTER(IxhPacked), C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p, C.c_int64,
+            C.c_void_p, C.c_size_t, C.c_void_p,
+        ]
+        L.ixh_gemm_workspace_bytes.restype = C.c_size_t
+        L.ixh_gemm_workspace_bytes.argtypes = [C.POINTER(IxhPacked), C.c_int32]
         _lib = L
     return _lib
 
@@ -194,3 +202,25 @@ class DevicePacked:
             workspace.data_ptr() if workspace is not None else None,
             workspace.numel() * workspace.element_size() if workspace is not None else 0,
             int(flags), current_stream(self.device)))
+
+    def gemm_workspace_bytes(self, m: int) -> int:
+        return int(lib().ixh_gemm_workspace_bytes(C.byref(self.struct), int(m)))
+
+    def gemm(self, table512, x, y, workspace) -> None:
+        """Fused decode + matrix-core GEMM: x bf16 [M, in_f], y bf16 [M, out_f], any M; table512 is the
+        rank table at unit 512.  Raises IxhError(IXH_EUNSUPPORTED) for shapes the kernel does not take."""
+        if not x.is_cuda:
+            raise RuntimeError(f"x must live on the GPU (got {x.device}); the HIP path has no CPU fallback")
+        if x.dtype != torch.bfloat16 or y.dtype != torch.bfloat16:
+            raise ValueError("x and y must be bf16")
+        x2 = x.reshape(-1, self.in_f)
+        if x2.stride(1) != 1 or y.stride(-1) != 1:
+            raise ValueError("x and y rows must be contiguous")
+        m = x2.shape[0]
+        y2 = y.reshape(m, self.out_f)
+        check(lib().ixh_gemm(
+            C.byref(self.struct), table512.data_ptr(), x2.data_ptr(), m,
+            x2.stride(0) if m > 1 else self.in_f, y2.data_ptr(), y2.stride(0) if m > 1 else self.out_f,
+            workspace.data_ptr() if workspace is not None else None,
+            workspace.numel() * workspace.element_size() if workspace is not None else 0,
+            current_stream(self.device)))

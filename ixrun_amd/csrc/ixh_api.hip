@@ -180,4 +180,39 @@ int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, cons
     return rc;
 }
 
+size_t ixh_gemm_workspace_bytes(const IxhPacked *packed, int32_t m) {
+    Dev d;
+    if (to_dev(packed, &d) || d.n == 0 || m < 1) return 0;
+    return prefill_workspace_bytes(d, (uint32_t)m);
+}
+
+int ixh_gemm(const IxhPacked *packed, const int32_t *prefix, const uint16_t *x, int32_t m, int64_t ldx, uint16_t *y,
+             int64_t ldy, void *workspace, size_t workspace_bytes, ixh_stream_t stream) {
+    Dev d;
+    int rc = to_dev(packed, &d);
+    if (rc) return rc;
+    if (m < 1) { set_error("m = %d < 1", m); return IXH_EINVAL; }
+    if (!y) { set_error("y is NULL"); return IXH_EINVAL; }
+    if (ldy < (int64_t)d.out_f && m > 1) { set_error("ldy %lld < out_f %u", (long long)ldy, d.out_f); return IXH_EINVAL; }
+    if (d.n == 0) {
+        for (int j = 0; j < m && d.out_f; ++j)
+            if (launch_fill_u16(y + (int64_t)j * ldy, d.out_f, 0, (hipStream_t)stream)) return IXH_ELAUNCH;
+        return IXH_OK;
+    }
+    if (!prefix || !x) { set_error("prefix or x is NULL"); return IXH_EINVAL; }
+    if (ldx < (int64_t)d.in_f && m > 1) { set_error("ldx %lld < in_f %u", (long long)ldx, d.in_f); return IXH_EINVAL; }
+    if (!prefill_supports(d, x, ldx)) {
+        set_error("gemm: needs in_f %% 512 == 0, in_f >= 4096, x 16-byte aligned, ldx %% 8 == 0, last stream 4-byte aligned");
+        return IXH_EUNSUPPORTED;
+    }
+    const size_t need = prefill_workspace_bytes(d, (uint32_t)m);
+    if (!workspace || workspace_bytes < need) {
+        set_error("workspace of %zu bytes needed, %zu given", need, workspace ? workspace_bytes : (size_t)0);
+        return IXH_EWORKSPACE;
+    }
+    rc = launch_prefill(d, prefix, x, (uint32_t)m, ldx, y, ldy, (float *)workspace, (hipStream_t)stream);
+    if (rc == IXH_ELAUNCH) set_error("gemm: launch failed");
+    return rc;
+}
+
 }  // extern "C"

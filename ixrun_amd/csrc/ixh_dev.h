@@ -93,6 +93,10 @@ int launch_decode(const Dev &P, const int32_t *prefix, uint32_t chunk, int8_t *o
 int launch_gemv_generic(const Dev &P, const int32_t *prefix, uint32_t chunk, const uint16_t *x, int m,
                         int64_t ldx, uint16_t *y, int64_t ldy, float *y32, float *ws, bool atomic,
                         hipStream_t s);
+size_t prefill_workspace_bytes(const Dev &P, uint32_t m_rows);
+bool prefill_supports(const Dev &P, const uint16_t *x, int64_t ldx);
+int launch_prefill(const Dev &P, const int32_t *prefix, const uint16_t *x, uint32_t m_rows, int64_t ldx, uint16_t *y,
+                   int64_t ldy, float *ws, hipStream_t s);
 int launch_fill_u16(uint16_t *dst, uint32_t n, uint16_t value, hipStream_t s);
 void set_error(const char *fmt, ...);
 

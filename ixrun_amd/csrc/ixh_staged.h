@@ -1,0 +1,164 @@
+// Level-scheme-agnostic decode from LDS: the streams of one table unit (a run of
+// `chunk` <= 512 flat elements) are first copied into an LDS slot with LDS-DMA
+// buffer loads, then ranked and decoded 64 elements at a time with wave ballots,
+// reading only LDS.  Used where the gather latency of the global-memory decoder
+// (decode64 in ixh_dev.h) cannot be hidden: the prefill GEMM and dense tensors.
+#pragma once
+
+#include "ixh_dev.h"
+
+namespace ixh {
+
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+
+constexpr uint32_t kStagedChunk = 512;  // largest unit the slot is sized for
+
+// LDS words a unit of 512 elements can need: every bitmap up to 17 words, all code
+// streams together at most 512*8/32 words plus two words of slack per stream.
+__host__ __device__ constexpr uint32_t staged_slot_words(int n_levels) {
+    return (uint32_t)(n_levels - 1) * 18u + 128u + 3u * (uint32_t)n_levels + 2u;
+}
+
+__device__ __forceinline__ uint32_t slds_u32(uint32_t addr) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) uint32_t *>((uintptr_t)addr);
+}
+__device__ __forceinline__ uint32_t slds_u8(uint32_t addr) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) uint8_t *>((uintptr_t)addr);
+}
+
+// Where the staged spans of one unit sit, folded so that a lane only adds its own
+// index: 5 * (L - 1) + 1 wave-uniform words per unit.
+template <int L>
+struct StagedUnit {
+    uint32_t bm_addr[L - 1];  // LDS address of the bitmap word holding the unit's first bit
+    uint32_t bm_off[L - 1];   // add to a level-i space index to get the bit index inside the staged span
+    uint32_t st_addr[L - 1];  // LDS address of the stream word holding the unit's first code
+    uint32_t st_off[L - 1];   // add to rank * bits to get the bit index inside the staged span
+    uint32_t cnt0[L - 1];     // level counts before the unit (the table entry)
+    uint32_t last_off;        // add to a last-level rank to get the LDS byte address
+};
+
+template <int L>
+__host__ __device__ constexpr uint32_t staged_record_words() { return 5u * (uint32_t)(L - 1) + 1u; }
+
+// A unit's record parked in LDS between the wave that staged it and the decode (which may
+// be a row later): lane 0 writes, every lane reads the same words back into registers.
+template <int L>
+__device__ __forceinline__ void put_unit(uint32_t rec, uint32_t lane, const StagedUnit<L> &S) {
+    if (lane == 0) {
+        __attribute__((address_space(3))) uint32_t *r = (__attribute__((address_space(3))) uint32_t *)(uintptr_t)rec;
+#pragma unroll
+        for (int i = 0; i < L - 1; ++i) {
+            r[5 * i + 0] = S.bm_addr[i];
+            r[5 * i + 1] = S.bm_off[i];
+            r[5 * i + 2] = S.st_addr[i];
+            r[5 * i + 3] = S.st_off[i];
+            r[5 * i + 4] = S.cnt0[i];
+        }
+        r[5 * (L - 1)] = S.last_off;
+    }
+}
+template <int L>
+__device__ __forceinline__ void get_unit(uint32_t rec, StagedUnit<L> &S) {
+    const __attribute__((address_space(3))) uint32_t *r = (const __attribute__((address_space(3))) uint32_t *)(uintptr_t)rec;
+#pragma unroll
+    for (int i = 0; i < L - 1; ++i) {
+        S.bm_addr[i] = r[5 * i + 0];
+        S.bm_off[i] = r[5 * i + 1];
+        S.st_addr[i] = r[5 * i + 2];
+        S.st_off[i] = r[5 * i + 3];
+        S.cnt0[i] = r[5 * i + 4];
+    }
+    S.last_off = r[5 * (L - 1)];
+}
+
+// Start the LDS-DMA of unit u's spans into the slot at LDS byte address `slot`
+// (16-byte aligned, staged_slot_words(L) words).  Wave-uniform arguments; the
+// copies are complete after s_waitcnt vmcnt(0).  `q_lo`/`q_hi` are the table
+// entries of unit u and u+1 (level counts before the unit and before the next).
+// The last-level stream must be 4-byte aligned.
+template <int L>
+__device__ __forceinline__ void stage_unit(const Dev &P, uint32_t u, uint32_t chunk, const uint32_t (&q_lo)[L - 1],
+                                           const uint32_t (&q_hi)[L - 1], uint32_t slot, uint32_t lane,
+                                           StagedUnit<L> &S) {
+    const uint64_t e0 = (uint64_t)u * chunk;
+    uint32_t space0 = (uint32_t)e0, space1 = (uint32_t)min(e0 + chunk, (uint64_t)P.n);
+    uint32_t off = 0;  // words used so far
+#pragma unroll
+    for (int i = 0; i < L - 1; ++i) {
+        {   // bitmap i: bits [space0, space1)
+            const __amdgpu_buffer_rsrc_t rs =
+                __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[i], 0, (int)(P.bm_words[i] * 4u), 0x00020000);
+            const uint32_t w0 = space0 >> 5, n = ((space1 + 31) >> 5) - w0;
+            if (lane < n)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)(uintptr_t)(slot + off * 4), 4,
+                                                         (int)((w0 + lane) * 4u), 0, 0, 0);
+            S.bm_addr[i] = slot + off * 4;
+            S.bm_off[i] = (space0 & 31) - space0;
+            off += n;
+        }
+        {   // stream i: codes [q_lo, q_hi), b bits each; one extra word so that a straddling read stays inside
+            const __amdgpu_buffer_rsrc_t rs =
+                __builtin_amdgcn_make_buffer_rsrc((void *)P.st[i], 0, (int)(P.st_words[i] * 4u), 0x00020000);
+            const uint32_t b = (uint32_t)P.bits[i];
+            const uint64_t bit0 = (uint64_t)q_lo[i] * b, bit1 = (uint64_t)q_hi[i] * b;
+            const uint32_t w0 = (uint32_t)(bit0 >> 5), n = (uint32_t)((bit1 + 31) >> 5) - w0 + 1;
+            for (uint32_t base = 0; base < n; base += kWave)
+                if (base + lane < n)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)(uintptr_t)(slot + (off + base) * 4), 4,
+                                                             (int)((w0 + base + lane) * 4u), 0, 0, 0);
+            S.st_addr[i] = slot + off * 4;
+            S.st_off[i] = ((uint32_t)bit0 & 31) - q_lo[i] * b;
+            S.cnt0[i] = q_lo[i];
+            off += n;
+        }
+        space0 -= q_lo[i];
+        space1 -= q_hi[i];
+    }
+    {   // last level: bytes [space0, space1), staged as whole dwords.  The buffer check is per dword, so the
+        // descriptor reaches the end of the last dword (device allocations are 256-byte granular).
+        const __amdgpu_buffer_rsrc_t rs =
+            __builtin_amdgcn_make_buffer_rsrc((void *)P.last, 0, (int)((P.last_bytes + 3u) & ~3u), 0x00020000);
+        const uint32_t w0 = space0 >> 2, n = ((space1 + 3) >> 2) - w0;
+        for (uint32_t base = 0; base < n; base += kWave)
+            if (base + lane < n)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)(uintptr_t)(slot + (off + base) * 4), 4,
+                                                         (int)((w0 + base + lane) * 4u), 0, 0, 0);
+        S.last_off = slot + off * 4 + (space0 & 3) - space0;
+    }
+}
+
+// Decode the 64 consecutive flat elements p0 .. p0+63 of a staged unit (one per
+// lane; lanes with alive == false take no part).  cnt[i] is the number of level-i
+// elements before p0 (global) and is advanced past the group.  Same ranking as
+// decode64, every read from LDS.
+template <int L>
+__device__ __forceinline__ int decode64_lds(const Dev &P, const StagedUnit<L> &S, uint32_t p0, bool alive,
+                                            uint32_t (&cnt)[L - 1]) {
+    int v = 0;
+    uint32_t space = p0;
+#pragma unroll
+    for (int i = 0; i < L - 1; ++i) {
+        const uint64_t alive_mask = __ballot(alive);
+        const uint32_t rel = space + S.bm_off[i] + lanes_below(alive_mask);  // bit inside the staged span
+        uint32_t bit = 0;
+        if (alive) bit = (slds_u32(S.bm_addr[i] + (rel >> 5) * 4) >> (rel & 31)) & 1u;
+        const bool taken = alive && bit;
+        const uint64_t taken_mask = __ballot(taken);
+        if (taken) {
+            const uint32_t b = (uint32_t)P.bits[i];
+            const uint32_t bitrel = (cnt[i] + lanes_below(taken_mask)) * b + S.st_off[i];
+            const uint32_t a = S.st_addr[i] + (bitrel >> 5) * 4;
+            const uint32_t lo = slds_u32(a), hi = slds_u32(a + 4);
+            v = (int)(__builtin_amdgcn_alignbit(hi, lo, bitrel) & ((1u << b) - 1u)) - threshold_of((int)b);
+        }
+        alive = alive && !bit;
+        space -= cnt[i];
+        cnt[i] += (uint32_t)__popcll(taken_mask);
+    }
+    const uint64_t alive_mask = __ballot(alive);
+    if (alive) v = (int)slds_u8(S.last_off + space + lanes_below(alive_mask)) - 127;
+    return v;
+}
+
+}  // namespace ixh

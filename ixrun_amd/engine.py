@@ -70,6 +70,7 @@ class StreamingLinear(nn.Module):
         self._use_triton = True
 
         self._use_fused = True
+        self._gemm_ok = True
         self._split_chunk = 0
         per_row = self.in_features // self._unit
         split = _pick_split(self.in_features) if self.out_features < self.in_features else 1
@@ -129,6 +130,25 @@ class StreamingLinear(nn.Module):
             if self._bias is not None:
                 y = y + self._bias.to(y.dtype)
             return y
+        if (self._use_fused and self._gemm_ok and x.dtype == torch.bfloat16 and x.is_cuda and rows > MAX_FUSED_ROWS
+                and x.shape[-1] == self.in_features and self._unit == 512):
+            # many rows: decode tiles on chip straight into the matrix-core GEMM, no bf16 weight in HBM
+            x2 = x.reshape(rows, self.in_features)
+            if x2.stride(1) != 1:
+                x2 = x2.contiguous()
+            y = torch.empty((rows, self.out_features), dtype=torch.bfloat16, device=x.device)
+            ws = shared_workspace(x.device, self._dp.gemm_workspace_bytes(rows))
+            try:
+                self._dp.gemm(self._table, x2, y, ws)
+            except _lib.IxhError as e:
+                if e.code != _lib.IXH_EUNSUPPORTED:
+                    raise
+                self._gemm_ok = False  # shape the fused GEMM does not take: decode + GEMM from here on
+            else:
+                y = y.view(x.shape[:-1] + (self.out_features,))
+                if self._bias is not None:
+                    y = y + self._bias.to(y.dtype)
+                return y
         w = self._decode()
         bias = self._bias.to(x.dtype) if self._bias is not None else None
         return F.linear(x, w.to(x.dtype) if w.dtype != x.dtype else w, bias)
