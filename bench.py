@@ -6,8 +6,9 @@ round-robin over COPIES distinct packed copies of the layer (together larger
 than the 256 MB last-level cache) so that every launch streams its packed bytes
 from HBM.  Inputs are resident on the GPU before the clock starts.
 
-Prints one JSON line (see README / DESIGN.md for the fields).  Extra workloads
-(--workload) time the other shapes of the hot path with the same harness.
+Prints one JSON line.  Extra workloads (--workload) time the other shapes of the
+hot path with the same harness; the many-row (prefill) workload runs the fused
+decode + matrix-core GEMM and is priced against the bf16 MFMA peak.
 """
 from __future__ import annotations
 
@@ -25,6 +26,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK = 8.0e12  # B/s, MI355X published
+MFMA_BF16_PEAK = 2.5e15  # FLOP/s dense bf16, MI355X published
 
 WORKLOADS = {
     # name: (out_f, in_f, m, weight recipe)
@@ -37,6 +39,11 @@ WORKLOADS = {
     "gate_up_17408x5120_m16_student_t": (17408, 5120, 16, "student_t"),
     # 64 distinct 5120x5120 layers chained (each output feeds the next layer), one hipGraph: us per layer
     "graph64_5120x5120_m1_student_t": (5120, 5120, 1, "student_t"),
+    # many activation rows: decode into LDS tiles + bf16 MFMA, five-level scheme
+    "prefill_5120x5120_m512_five_level": (5120, 5120, 512, "student_t", (3, 4, 5, 6, 8)),
+    "prefill_5120x5120_m512_358": (5120, 5120, 512, "student_t"),
+    "prefill_5120x17408_m512_358": (5120, 17408, 512, "student_t"),
+    "prefill_5120x5120_m64_five_level": (5120, 5120, 64, "student_t", (3, 4, 5, 6, 8)),
 }
 
 
@@ -95,6 +102,8 @@ def main():
     ap.add_argument("--copies", type=int, default=0, help="distinct packed copies to rotate over (0 = enough for 600 MB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of hipGraph replays")
+    ap.add_argument("--unfused", action="store_true",
+                    help="many-row workloads: decode the bf16 weight to HBM and call the library GEMM instead")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 256 MiB device copies (known traffic) so that counter runs can be scaled")
     args = ap.parse_args()
@@ -106,16 +115,22 @@ def main():
 
     from ixrun_amd.engine import StreamingLinear
 
-    out_f, in_f, m, recipe = WORKLOADS[args.workload]
+    out_f, in_f, m, recipe, *rest = WORKLOADS[args.workload]
+    level_bits = rest[0] if rest else (3, 5, 8)
     t0 = time.perf_counter()
     from ixrun_amd.quantize import int8x_quantize
 
     weight = make_weight(out_f, in_f, recipe)
-    packed = int8x_quantize(weight)
+    packed = int8x_quantize(weight, level_bits)
     prep_s = time.perf_counter() - t0
     chained = args.workload.startswith("graph64")
     copies = args.copies or (64 if chained else max(2, -(-600_000_000 // packed["total_bytes"])))
     layers = [StreamingLinear(packed) for _ in range(copies)]
+    if args.unfused:
+        shared = torch.empty(packed["N"], dtype=torch.bfloat16, device=dev)
+        for sl in layers:
+            sl._gemm_ok = False
+            sl._set_shared_buf(shared)
     g = torch.Generator("cpu").manual_seed(1)
     x_host = torch.randn(m, in_f, generator=g).bfloat16()
     x = x_host.to(dev)
@@ -196,7 +211,7 @@ def main():
         "ms_per_step": ms_per_step, "us_per_layer": us, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16 activations x int8 codes, fp32 accumulate", "data": "synthetic",
         "config": {
-            "workload": args.workload, "out_f": out_f, "in_f": in_f, "batch": m, "level_bits": [3, 5, 8],
+            "workload": args.workload, "out_f": out_f, "in_f": in_f, "batch": m, "level_bits": list(level_bits),
             "weights": recipe, "level_fractions": [c / packed["N"] for c in packed["counts"]],
             "bits_per_weight": packed["bits_per_weight"], "packed_bytes": packed["total_bytes"],
             "rank_table_bytes": table_bytes, "distinct_copies": copies,
@@ -212,8 +227,17 @@ def main():
         "host_wall_ms_per_step": wall_ms / steps,
         "prep_s": prep_s,
     }
+    if m > 16:
+        flops = 2.0 * m * out_f * in_f
+        out["roofline"] = {
+            "bound": "mfma", "achieved": flops / (ms_per_step * 1e-3) / 1e12, "peak": MFMA_BF16_PEAK / 1e12,
+            "unit": "TFLOP/s", "frac": flops / (ms_per_step * 1e-3) / MFMA_BF16_PEAK, "traffic": None,
+            "note": "2*M*N*K flops per launch pair (GEMM + slice reduce); the kernel is bound by the VALU decode "
+                    "that feeds the matrix cores, not by MFMA issue",
+        }
+        out["path"] = "decode to HBM + library GEMM" if args.unfused else "fused decode + MFMA (ixh_gemm)"
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(weight, x_host)
+        out["cpu_baseline"] = cpu_baseline(weight, x_host, level_bits)
         out["cpu_baseline"]["speedup_vs_cpu"] = out["value"] / out["cpu_baseline"]["value"]
     print(json.dumps(out))
 

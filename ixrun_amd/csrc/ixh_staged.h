@@ -13,11 +13,16 @@ typedef __attribute__((address_space(3))) void *lds_ptr_t;
 
 constexpr uint32_t kStagedChunk = 512;  // largest unit the slot is sized for
 
-// LDS words a unit of 512 elements can need: every bitmap up to 17 words, all code
-// streams together at most 512*8/32 words plus two words of slack per stream.
+// LDS words a unit of 512 elements can need.  Every span is copied 16 bytes per lane and
+// padded to a multiple of 16 bytes: a bitmap span is at most 17 words (20 padded), all code
+// streams together at most 512*8/32 words plus, per stream, the partial first word, one
+// word for a straddling read and the padding.
 __host__ __device__ constexpr uint32_t staged_slot_words(int n_levels) {
-    return (uint32_t)(n_levels - 1) * 18u + 128u + 3u * (uint32_t)n_levels + 2u;
+    return (uint32_t)(n_levels - 1) * 20u + 128u + 8u * (uint32_t)n_levels;
 }
+// buffer loads into LDS that one call of stage_unit issues, always: the count a caller needs to wait for
+// one unit's copies while later ones are still in flight (s_waitcnt vmcnt)
+__host__ __device__ constexpr int staged_dma_count(int n_levels) { return 2 * n_levels - 1; }
 
 __device__ __forceinline__ uint32_t slds_u32(uint32_t addr) {
     return *reinterpret_cast<const __attribute__((address_space(3))) uint32_t *>((uintptr_t)addr);
@@ -73,72 +78,65 @@ __device__ __forceinline__ void get_unit(uint32_t rec, StagedUnit<L> &S) {
 }
 
 // Start the LDS-DMA of unit u's spans into the slot at LDS byte address `slot`
-// (16-byte aligned, staged_slot_words(L) words).  Wave-uniform arguments; the
-// copies are complete after s_waitcnt vmcnt(0).  `q_lo`/`q_hi` are the table
-// entries of unit u and u+1 (level counts before the unit and before the next).
-// The last-level stream must be 4-byte aligned.
+// (16-byte aligned, staged_slot_words(L) words).  Wave-uniform arguments.  Exactly
+// staged_dma_count(L) buffer loads are issued, each with lane 0 active.  `q_lo`/`q_hi` are
+// the table entries of unit u and u+1 (level counts before the unit and before the next).
+// chunk <= 512; the last-level stream must be 4-byte aligned.
 template <int L>
 __device__ __forceinline__ void stage_unit(const Dev &P, uint32_t u, uint32_t chunk, const uint32_t (&q_lo)[L - 1],
                                            const uint32_t (&q_hi)[L - 1], uint32_t slot, uint32_t lane,
                                            StagedUnit<L> &S) {
     const uint64_t e0 = (uint64_t)u * chunk;
     uint32_t space0 = (uint32_t)e0, space1 = (uint32_t)min(e0 + chunk, (uint64_t)P.n);
-    uint32_t off = 0;  // words used so far
+    uint32_t off = 0;  // bytes used so far, a multiple of 16
+    auto copy = [&](__amdgpu_buffer_rsrc_t rs, uint32_t first_word, uint32_t n_words) {
+        const uint32_t n4 = max((n_words + 3u) >> 2, 1u);  // 16-byte pieces, one per lane (at most 33)
+#ifndef IXH_PF_NO_STAGE
+        if (lane < n4)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)(uintptr_t)(slot + off), 16,
+                                                     (int)(first_word * 4u + lane * 16u), 0, 0, 0);
+#endif
+        off += n4 * 16u;
+    };
 #pragma unroll
     for (int i = 0; i < L - 1; ++i) {
         {   // bitmap i: bits [space0, space1)
-            const __amdgpu_buffer_rsrc_t rs =
-                __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[i], 0, (int)(P.bm_words[i] * 4u), 0x00020000);
             const uint32_t w0 = space0 >> 5, n = ((space1 + 31) >> 5) - w0;
-            if (lane < n)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)(uintptr_t)(slot + off * 4), 4,
-                                                         (int)((w0 + lane) * 4u), 0, 0, 0);
-            S.bm_addr[i] = slot + off * 4;
+            S.bm_addr[i] = slot + off;
             S.bm_off[i] = (space0 & 31) - space0;
-            off += n;
+            copy(__builtin_amdgcn_make_buffer_rsrc((void *)P.bm[i], 0, (int)(P.bm_words[i] * 4u), 0x00020000), w0, n);
         }
         {   // stream i: codes [q_lo, q_hi), b bits each; one extra word so that a straddling read stays inside
-            const __amdgpu_buffer_rsrc_t rs =
-                __builtin_amdgcn_make_buffer_rsrc((void *)P.st[i], 0, (int)(P.st_words[i] * 4u), 0x00020000);
             const uint32_t b = (uint32_t)P.bits[i];
             const uint64_t bit0 = (uint64_t)q_lo[i] * b, bit1 = (uint64_t)q_hi[i] * b;
             const uint32_t w0 = (uint32_t)(bit0 >> 5), n = (uint32_t)((bit1 + 31) >> 5) - w0 + 1;
-            for (uint32_t base = 0; base < n; base += kWave)
-                if (base + lane < n)
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)(uintptr_t)(slot + (off + base) * 4), 4,
-                                                             (int)((w0 + base + lane) * 4u), 0, 0, 0);
-            S.st_addr[i] = slot + off * 4;
+            S.st_addr[i] = slot + off;
             S.st_off[i] = ((uint32_t)bit0 & 31) - q_lo[i] * b;
             S.cnt0[i] = q_lo[i];
-            off += n;
+            copy(__builtin_amdgcn_make_buffer_rsrc((void *)P.st[i], 0, (int)(P.st_words[i] * 4u), 0x00020000), w0, n);
         }
         space0 -= q_lo[i];
         space1 -= q_hi[i];
     }
     {   // last level: bytes [space0, space1), staged as whole dwords.  The buffer check is per dword, so the
         // descriptor reaches the end of the last dword (device allocations are 256-byte granular).
-        const __amdgpu_buffer_rsrc_t rs =
-            __builtin_amdgcn_make_buffer_rsrc((void *)P.last, 0, (int)((P.last_bytes + 3u) & ~3u), 0x00020000);
         const uint32_t w0 = space0 >> 2, n = ((space1 + 3) >> 2) - w0;
-        for (uint32_t base = 0; base < n; base += kWave)
-            if (base + lane < n)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)(uintptr_t)(slot + (off + base) * 4), 4,
-                                                         (int)((w0 + base + lane) * 4u), 0, 0, 0);
-        S.last_off = slot + off * 4 + (space0 & 3) - space0;
+        S.last_off = slot + off + (space0 & 3) - space0;
+        copy(__builtin_amdgcn_make_buffer_rsrc((void *)P.last, 0, (int)((P.last_bytes + 3u) & ~3u), 0x00020000), w0, n);
     }
 }
 
-// Decode the 64 consecutive flat elements p0 .. p0+63 of a staged unit (one per
-// lane; lanes with alive == false take no part).  cnt[i] is the number of level-i
-// elements before p0 (global) and is advanced past the group.  Same ranking as
-// decode64, every read from LDS.
-template <int L>
-__device__ __forceinline__ int decode64_lds(const Dev &P, const StagedUnit<L> &S, uint32_t p0, bool alive,
-                                            uint32_t (&cnt)[L - 1]) {
+// Levels START .. L-1 of up to 64 elements of a staged unit, one per lane (lanes with
+// alive == false take no part).  `space` is the index, in the space of level START, of the
+// first alive lane's element; the alive lanes hold consecutive elements of that space.
+// cnt[i] (i >= START) is the number of level-i elements before that element (global) and is
+// advanced past the group.  Same ranking as decode64, every read from LDS.
+template <int L, int START>
+__device__ __forceinline__ int decode_from_lds(const Dev &P, const StagedUnit<L> &S, uint32_t space, bool alive,
+                                               uint32_t (&cnt)[L - 1]) {
     int v = 0;
-    uint32_t space = p0;
 #pragma unroll
-    for (int i = 0; i < L - 1; ++i) {
+    for (int i = START; i < L - 1; ++i) {
         const uint64_t alive_mask = __ballot(alive);
         const uint32_t rel = space + S.bm_off[i] + lanes_below(alive_mask);  // bit inside the staged span
         uint32_t bit = 0;
@@ -159,6 +157,66 @@ __device__ __forceinline__ int decode64_lds(const Dev &P, const StagedUnit<L> &S
     const uint64_t alive_mask = __ballot(alive);
     if (alive) v = (int)slds_u8(S.last_off + space + lanes_below(alive_mask)) - 127;
     return v;
+}
+
+// The 64 consecutive flat elements p0 .. p0+63 of a staged unit, all levels.
+template <int L>
+__device__ __forceinline__ int decode64_lds(const Dev &P, const StagedUnit<L> &S, uint32_t p0, bool alive,
+                                            uint32_t (&cnt)[L - 1]) {
+    return decode_from_lds<L, 0>(P, S, p0, alive, cnt);
+}
+
+// A whole staged unit of `n_el` <= 512 elements starting at flat element p_begin, dequantised to bf16 into
+// dst[0 .. n_el) (LDS).  Level 1 is ranked for all eight groups of 64 at once, without branches, so that the
+// LDS reads of the groups overlap; the elements it does not hold (few, in the tensors this format is built
+// for) are queued and taken through the deeper levels together, 64 per pass, instead of a lane or two per
+// group.  `queue`: LDS, kStagedQueue uint16 (the entries past 512 absorb the writes of lanes with nothing to
+// queue).
+constexpr uint32_t kStagedQueue = kStagedChunk + kWave;
+
+template <int L>
+__device__ __forceinline__ void decode_unit_lds(const Dev &P, const StagedUnit<L> &S, uint32_t p_begin, uint32_t n_el,
+                                                float scale, uint16_t *dst, uint16_t *queue, uint32_t lane) {
+    constexpr int G = kStagedChunk / kWave;
+    uint32_t cnt[L - 1];
+#pragma unroll
+    for (int i = 0; i < L - 1; ++i) cnt[i] = S.cnt0[i];
+    const uint32_t b = (uint32_t)P.bits[0];
+    const int thr = threshold_of((int)b);
+    uint32_t bit[G];
+    uint64_t taken_mask[G], other_mask[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {  // reads past the unit's bits stay inside the slot
+        const uint32_t p = g * kWave + lane;
+        const uint32_t rel = p_begin + p + S.bm_off[0];
+        bit[g] = p < n_el ? (slds_u32(S.bm_addr[0] + (rel >> 5) * 4) >> (rel & 31)) & 1u : 0u;
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        taken_mask[g] = __ballot(bit[g] != 0);
+        other_mask[g] = __ballot(g * kWave + lane < n_el && !bit[g]);
+    }
+    uint32_t n_taken = cnt[0], n_queued = 0;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const uint32_t p = g * kWave + lane;
+        // lanes without a level-1 code read a code all the same (a few words past their neighbours' at most)
+        const uint32_t bitrel = (n_taken + lanes_below(taken_mask[g])) * b + S.st_off[0];
+        const uint32_t a = S.st_addr[0] + (bitrel >> 5) * 4;
+        const uint32_t lo = slds_u32(a), hi = slds_u32(a + 4);
+        const int v = (int)(__builtin_amdgcn_alignbit(hi, lo, bitrel) & ((1u << b) - 1u)) - thr;
+        if (p < n_el) dst[p] = bit[g] ? (uint16_t)f32_to_bf16_bits((float)v * scale) : (uint16_t)0;
+        queue[bit[g] || p >= n_el ? kStagedChunk + lane : n_queued + lanes_below(other_mask[g])] = (uint16_t)p;
+        n_taken += (uint32_t)__popcll(taken_mask[g]);
+        n_queued += (uint32_t)__popcll(other_mask[g]);
+    }
+    const uint32_t space1 = p_begin - S.cnt0[0];  // the unit's first element in the space of level 2
+    for (uint32_t base = 0; base < n_queued; base += kWave) {
+        const bool alive = base + lane < n_queued;
+        const uint32_t p = alive ? queue[base + lane] : 0u;
+        const int v = decode_from_lds<L, 1>(P, S, space1 + base, alive, cnt);
+        if (alive) dst[p] = (uint16_t)f32_to_bf16_bits((float)v * scale);
+    }
 }
 
 }  // namespace ixh

@@ -25,7 +25,7 @@ def run_gemm(dp, x, dev):
 
 
 @pytest.mark.parametrize("kind", ["student_t", "calibrated_odd_scale", "rare_other", "only_l1", "only_l3", "no_l2"])
-@pytest.mark.parametrize("shape", [(64, 4096), (100, 4608), (130, 8192)])
+@pytest.mark.parametrize("shape", [(64, 512), (100, 4608), (130, 8192)])
 @pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8)])
 def test_gemm_matches_oracle(oracle, dev, kind, shape, level_bits):
     out_f, in_f = shape
@@ -86,9 +86,9 @@ def test_gemm_strided_rows_and_repeatability(oracle, dev):
 def test_gemm_rejects_what_it_cannot_take(oracle, dev):
     from ixrun_amd import _lib
 
-    p = make_packed("student_t", 64, 1024)
+    p = make_packed("student_t", 64, 1000)  # rows that are not whole 512-element units
     dp = device_packed(p, dev)
-    x = activations(32, 1024, seed=1)
+    x = activations(32, 1000, seed=1)
     with pytest.raises(_lib.IxhError) as e:
         run_gemm(dp, x, dev)
     assert e.value.code == _lib.IXH_EUNSUPPORTED
