@@ -166,50 +166,100 @@ __device__ __forceinline__ int decode64_lds(const Dev &P, const StagedUnit<L> &S
     return decode_from_lds<L, 0>(P, S, p0, alive, cnt);
 }
 
+// inclusive sum over the lanes at or below this one (DPP: shifts inside the 16-lane rows, then the two
+// row broadcasts that carry the totals across rows)
+__device__ __forceinline__ uint32_t wave_scan_inclusive(uint32_t v) {
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, true);   // row_shr:1
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, true);   // row_shr:2
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, true);   // row_shr:4
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, true);   // row_shr:8
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1, 3
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2, 3
+    return v;
+}
+
+typedef float staged_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 staged_bf16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t staged_u32x4 __attribute__((ext_vector_type(4)));
+
+// two fp32 -> packed bf16 (round to nearest even: v_cvt_pk_bf16_f32), first value in the low half
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    const staged_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, staged_bf16x2));
+}
+
 // A whole staged unit of `n_el` <= 512 elements starting at flat element p_begin, dequantised to bf16 into
-// dst[0 .. n_el) (LDS).  Level 1 is ranked for all eight groups of 64 at once, without branches, so that the
-// LDS reads of the groups overlap; the elements it does not hold (few, in the tensors this format is built
-// for) are queued and taken through the deeper levels together, 64 per pass, instead of a lane or two per
-// group.  `queue`: LDS, kStagedQueue uint16 (the entries past 512 absorb the writes of lanes with nothing to
-// queue).
-constexpr uint32_t kStagedQueue = kStagedChunk + kWave;
+// dst[0 .. 512) (LDS, 16-byte aligned; entries past n_el are written as zero).  Level 1 is decoded eight
+// consecutive elements per lane: the lane takes its byte of the bitmap, a wave prefix sum of the bytes'
+// popcounts gives the rank of its first code, and its codes are peeled off a 64-bit window of the stream.
+// The elements level 1 does not hold (few, in the tensors this format is built for) are queued (`queue`:
+// LDS, kStagedQueue uint16) and taken through the deeper levels together, 64 per pass, by ballot ranking.
+constexpr uint32_t kStagedQueue = kStagedChunk;
 
 template <int L>
 __device__ __forceinline__ void decode_unit_lds(const Dev &P, const StagedUnit<L> &S, uint32_t p_begin, uint32_t n_el,
                                                 float scale, uint16_t *dst, uint16_t *queue, uint32_t lane) {
-    constexpr int G = kStagedChunk / kWave;
     uint32_t cnt[L - 1];
 #pragma unroll
     for (int i = 0; i < L - 1; ++i) cnt[i] = S.cnt0[i];
     const uint32_t b = (uint32_t)P.bits[0];
     const int thr = threshold_of((int)b);
-    uint32_t bit[G];
-    uint64_t taken_mask[G], other_mask[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {  // reads past the unit's bits stay inside the slot
-        const uint32_t p = g * kWave + lane;
-        const uint32_t rel = p_begin + p + S.bm_off[0];
-        bit[g] = p < n_el ? (slds_u32(S.bm_addr[0] + (rel >> 5) * 4) >> (rel & 31)) & 1u : 0u;
+    const uint32_t e0 = 8 * lane;
+    const uint32_t n_here = e0 < n_el ? min(8u, n_el - e0) : 0u;  // elements of this lane inside the unit
+    const uint32_t here = (1u << n_here) - 1u;
+    uint32_t m;  // bit t: element e0 + t is level 1
+    {
+        const uint32_t rel = p_begin + e0 + S.bm_off[0];
+        const uint32_t a = S.bm_addr[0] + (rel >> 5) * 4;
+        m = __builtin_amdgcn_alignbit(slds_u32(a + 4), slds_u32(a), rel) & here;
     }
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        taken_mask[g] = __ballot(bit[g] != 0);
-        other_mask[g] = __ballot(g * kWave + lane < n_el && !bit[g]);
+    const uint32_t n_mine = (uint32_t)__popc(m);
+    const uint32_t incl = wave_scan_inclusive(n_mine);
+    const uint32_t n_taken = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+    uint32_t clo, chi;  // 64 bits of the stream from this lane's first code on
+    {
+        const uint32_t bitpos = (cnt[0] + incl - n_mine) * b + S.st_off[0];
+        const uint32_t a = S.st_addr[0] + (bitpos >> 5) * 4;
+        const uint32_t w0 = slds_u32(a), w1 = slds_u32(a + 4), w2 = slds_u32(a + 8);
+        clo = __builtin_amdgcn_alignbit(w1, w0, bitpos);
+        chi = __builtin_amdgcn_alignbit(w2, w1, bitpos);
     }
-    uint32_t n_taken = cnt[0], n_queued = 0;
+    float f[8];
+    uint32_t off = 0;
+    if (b <= 4) {  // eight codes fit 32 bits
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        const uint32_t p = g * kWave + lane;
-        // lanes without a level-1 code read a code all the same (a few words past their neighbours' at most)
-        const uint32_t bitrel = (n_taken + lanes_below(taken_mask[g])) * b + S.st_off[0];
-        const uint32_t a = S.st_addr[0] + (bitrel >> 5) * 4;
-        const uint32_t lo = slds_u32(a), hi = slds_u32(a + 4);
-        const int v = (int)(__builtin_amdgcn_alignbit(hi, lo, bitrel) & ((1u << b) - 1u)) - thr;
-        if (p < n_el) dst[p] = bit[g] ? (uint16_t)f32_to_bf16_bits((float)v * scale) : (uint16_t)0;
-        queue[bit[g] || p >= n_el ? kStagedChunk + lane : n_queued + lanes_below(other_mask[g])] = (uint16_t)p;
-        n_taken += (uint32_t)__popcll(taken_mask[g]);
-        n_queued += (uint32_t)__popcll(other_mask[g]);
+        for (int t = 0; t < 8; ++t) {
+            const uint32_t bit = (m >> t) & 1u;
+            const int v = ((int)__builtin_amdgcn_ubfe(clo, off, b) - thr) * (int)bit;
+            f[t] = (float)v * scale;
+            off += bit * b;
+        }
+    } else {
+        const uint32_t code_mask = (1u << b) - 1u;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const uint32_t bit = (m >> t) & 1u;
+            const uint32_t w = off < 32 ? __builtin_amdgcn_alignbit(chi, clo, off) : chi >> (off - 32);
+            const int v = ((int)(w & code_mask) - thr) * (int)bit;
+            f[t] = (float)v * scale;
+            off += bit * b;
+        }
     }
+    const staged_u32x4 packed = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                                 pack_bf16x2(f[6], f[7])};
+    *reinterpret_cast<staged_u32x4 *>(dst + e0) = packed;
+
+    // positions of the elements above level 1, in order
+    {
+        uint32_t z = ~m & here;
+        uint32_t q = min(e0, n_el) - (incl - n_mine);
+        while (z) {
+            queue[q++] = (uint16_t)(e0 + (uint32_t)__builtin_ctz(z));
+            z &= z - 1;
+        }
+    }
+    cnt[0] += n_taken;
+    const uint32_t n_queued = n_el - n_taken;
     const uint32_t space1 = p_begin - S.cnt0[0];  // the unit's first element in the space of level 2
     for (uint32_t base = 0; base < n_queued; base += kWave) {
         const bool alive = base + lane < n_queued;
