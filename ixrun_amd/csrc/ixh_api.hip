@@ -4,6 +4,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <cstdlib>
+
 #include "ixh_dev.h"
 #include "ixh_fast358.h"
 
@@ -107,7 +109,11 @@ int ixh_decode(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, in
     if (d.n == 0) return IXH_OK;
     if (!prefix) { set_error("prefix is NULL"); return IXH_EINVAL; }
     if (!out_i8 && !out_bf16) { set_error("both outputs are NULL"); return IXH_EINVAL; }
-    rc = launch_decode(d, prefix, (uint32_t)chunk, out_i8, out_bf16, (hipStream_t)stream);
+    static const bool no_staged = getenv("IXH_DECODE_GENERIC") != nullptr;  // measurement switch
+    if (!no_staged && decode_staged_supports(d, (uint32_t)chunk, out_i8, out_bf16))
+        rc = launch_decode_staged(d, prefix, out_bf16, (hipStream_t)stream);
+    else
+        rc = launch_decode(d, prefix, (uint32_t)chunk, out_i8, out_bf16, (hipStream_t)stream);
     if (rc == IXH_ELAUNCH) set_error("decode: launch failed");
     return rc;
 }

@@ -127,6 +127,21 @@ def test_decode_bit_exact(oracle, dev, kind, shape):
         assert np.array_equal(bf16_bits(o16).reshape(shape), w_want), (kind, shape, chunk)
 
 
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("shape", [(1, 512), (3, 171), (33, 1000), (64, 1536), (300, 1031), (256, 4608)])
+@pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8), (2, 8), (5, 6, 7, 8)])
+def test_decode_bf16_only(oracle, dev, kind, shape, level_bits):
+    """bf16-only decode at the 512-element table unit: the kernel that stages the streams in LDS
+    (ragged last unit, rows that are not whole units, level-1 codes wider than 4 bits)."""
+    p = make_packed(kind, *shape, level_bits)
+    dp = device_packed(p, dev)
+    table = dp.prefix_build(512)
+    o16 = torch.full((p["N"] + 8,), 7.0, dtype=torch.bfloat16, device=dev)
+    dp.decode(table, 512, out_bf16=o16[: p["N"]])
+    assert np.array_equal(bf16_bits(o16[: p["N"]]).reshape(shape), oracle.decode_packed_bf16(p)), (kind, shape, level_bits)
+    assert torch.all(o16[p["N"]:] == 7.0)  # nothing written past the end
+
+
 @pytest.mark.parametrize("level_bits", [(3, 4, 5, 6, 8), (2, 8), (4, 8), (1, 2, 3, 4, 5, 6, 7, 8), (3, 3, 8)])
 def test_decode_other_level_schemes(oracle, dev, level_bits):
     from ixrun_amd.triton_kernels import decode_weight_triton, decode_int8
