@@ -192,8 +192,9 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 // dst[0 .. 512) (LDS, 16-byte aligned; entries past n_el are written as zero).  Level 1 is decoded eight
 // consecutive elements per lane: the lane takes its byte of the bitmap, a wave prefix sum of the bytes'
 // popcounts gives the rank of its first code, and its codes are peeled off a 64-bit window of the stream.
-// The elements level 1 does not hold (few, in the tensors this format is built for) are queued (`queue`:
-// LDS, kStagedQueue uint16) and taken through the deeper levels together, 64 per pass, by ballot ranking.
+// When level 1 leaves at most 64 elements (the tensors this format is built for), those are queued (`queue`:
+// LDS, kStagedQueue uint16) and taken through the deeper levels together by ballot ranking; when it leaves
+// more (dense mixes), the lanes keep their eight elements and repeat the level-1 scheme level by level.
 constexpr uint32_t kStagedQueue = kStagedChunk;
 
 template <int L>
@@ -245,6 +246,65 @@ __device__ __forceinline__ void decode_unit_lds(const Dev &P, const StagedUnit<L
             off += bit * b;
         }
     }
+    const uint32_t n_queued = n_el - n_taken;
+    if (n_queued > kWave) {
+        // Many elements above level 1 (a dense mix): the lane keeps its eight elements through every level.
+        // `alive`: its elements no level has claimed yet; `before`: such elements in the lanes below; the
+        // lane's bits of the next bitmap are consecutive from there, its codes follow from one more prefix sum.
+        uint32_t alive = ~m & here;
+        uint32_t before = min(e0, n_el) - (incl - n_mine);
+        uint32_t space = p_begin - S.cnt0[0];  // the unit's first element in the space of the level at hand
+#pragma unroll
+        for (int i = 1; i < L - 1; ++i) {
+            const uint32_t bi = (uint32_t)P.bits[i], code_mask = (1u << bi) - 1u;
+            const int thr_i = threshold_of((int)bi);
+            const uint32_t rel = space + before + S.bm_off[i];
+            const uint32_t ba = S.bm_addr[i] + (rel >> 5) * 4;
+            const uint32_t bits = __builtin_amdgcn_alignbit(slds_u32(ba + 4), slds_u32(ba), rel) &
+                                  ((1u << __popc(alive)) - 1u);
+            const uint32_t n_t = (uint32_t)__popc(bits);
+            const uint32_t inc = wave_scan_inclusive(n_t);
+            const uint32_t bitpos = (S.cnt0[i] + inc - n_t) * bi + S.st_off[i];
+            const uint32_t wa = S.st_addr[i] + (bitpos >> 5) * 4;
+            const uint32_t w0 = slds_u32(wa), w1 = slds_u32(wa + 4), w2 = slds_u32(wa + 8);
+            const uint32_t lo = __builtin_amdgcn_alignbit(w1, w0, bitpos), hi = __builtin_amdgcn_alignbit(w2, w1, bitpos);
+            uint32_t pos = 0, idx = 0, still = 0;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const uint32_t a_t = (alive >> t) & 1u;
+                const uint32_t bit = (bits >> idx) & a_t;
+                const uint32_t w = pos < 32 ? __builtin_amdgcn_alignbit(hi, lo, pos) : hi >> (pos - 32);
+                const float val = (float)((int)(w & code_mask) - thr_i) * scale;
+                f[t] = bit ? val : f[t];
+                pos += bit * bi;
+                idx += a_t;
+                still |= (a_t ^ bit) << t;
+            }
+            alive = still;
+            before -= inc - n_t;
+            space -= S.cnt0[i];
+        }
+        {   // last level: one byte per element still alive
+            const uint32_t addr = S.last_off + space + before;
+            const uint32_t wa = addr & ~3u, sh = (addr & 3u) * 8u;
+            const uint32_t w0 = slds_u32(wa), w1 = slds_u32(wa + 4), w2 = slds_u32(wa + 8);
+            const uint32_t lo = __builtin_amdgcn_alignbit(w1, w0, sh), hi = __builtin_amdgcn_alignbit(w2, w1, sh);
+            uint32_t pos = 0;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const uint32_t a_t = (alive >> t) & 1u;
+                const uint32_t w = pos < 32 ? __builtin_amdgcn_alignbit(hi, lo, pos) : hi >> (pos - 32);
+                const float val = (float)((int)(w & 0xFFu) - 127) * scale;
+                f[t] = a_t ? val : f[t];
+                pos += a_t * 8u;
+            }
+        }
+        const staged_u32x4 packed = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                                     pack_bf16x2(f[6], f[7])};
+        *reinterpret_cast<staged_u32x4 *>(dst + e0) = packed;
+        return;
+    }
+
     const staged_u32x4 packed = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
                                  pack_bf16x2(f[6], f[7])};
     *reinterpret_cast<staged_u32x4 *>(dst + e0) = packed;
@@ -259,7 +319,6 @@ __device__ __forceinline__ void decode_unit_lds(const Dev &P, const StagedUnit<L
         }
     }
     cnt[0] += n_taken;
-    const uint32_t n_queued = n_el - n_taken;
     const uint32_t space1 = p_begin - S.cnt0[0];  // the unit's first element in the space of level 2
     for (uint32_t base = 0; base < n_queued; base += kWave) {
         const bool alive = base + lane < n_queued;

@@ -28,10 +28,10 @@ from .quantize import int8x_quantize
 __all__ = ["Int8XEngine", "StreamingLinear", "GraphLinear", "ResourceScheduler"]
 
 MAX_FUSED_ROWS = 16  # activation rows served by the fused decode+GEMV kernel
-# Up to this many rows the fused decode+GEMM is the faster path on MI355X (measured on 5120 x 5120: level with
-# decode + library GEMM at 128 rows, 60 % slower at 512, where the library GEMM's larger tiles pay off); beyond
-# it the layer decodes into the shared buffer and calls the library GEMM, unless no buffer was provided.
-MAX_FUSED_GEMM_ROWS = 128
+# More rows than that: with a shared decode buffer the layer decodes into it and calls the library GEMM
+# (5120 x 5120 five-level on MI355X: 60 us at 32 rows, 84 us at 512); without one it runs the fused
+# decode+GEMM, which keeps the bf16 weight out of HBM altogether but is slower (84 us and 194 us): its
+# decode shares the CU with the matrix-core tiles at two waves per SIMD, the stand-alone decode runs at six.
 
 
 class StreamingLinear(nn.Module):
@@ -135,8 +135,7 @@ class StreamingLinear(nn.Module):
                 y = y + self._bias.to(y.dtype)
             return y
         if (self._use_fused and self._gemm_ok and x.dtype == torch.bfloat16 and x.is_cuda and rows > MAX_FUSED_ROWS
-                and x.shape[-1] == self.in_features and self._unit == 512
-                and (rows <= MAX_FUSED_GEMM_ROWS or self._w_buf is None)):
+                and x.shape[-1] == self.in_features and self._unit == 512 and self._w_buf is None):
             # many rows: decode tiles on chip straight into the matrix-core GEMM, no bf16 weight in HBM
             x2 = x.reshape(rows, self.in_features)
             if x2.stride(1) != 1:
