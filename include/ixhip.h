@@ -37,9 +37,10 @@ extern "C" {
 
 /* ixh_gemv flags */
 #define IXH_GEMV_ATOMIC 1u /* add fp32 partials into y32 with atomics (caller zeroes y32) */
-#define IXH_GEMV_FORCE_GENERIC 2u /* skip the (3,5,8) specialised kernels (testing / comparison) */
+#define IXH_GEMV_FORCE_GENERIC 2u /* only the wave-per-unit kernel that gathers from global memory (testing / comparison) */
 #define IXH_GEMV_COLUMN_KERNEL 4u /* of the (3,5,8) kernels, take the column-block one with the workspace */
 #define IXH_GEMV_FORCE_358 8u /* use the (3,5,8) kernels even when less than 97 % of the elements are level 1 */
+#define IXH_GEMV_STAGED 16u /* skip the (3,5,8) kernels: the any-scheme kernel that stages the streams in LDS */
 
 typedef void *ixh_stream_t; /* a hipStream_t */
 

@@ -93,6 +93,9 @@ int launch_decode(const Dev &P, const int32_t *prefix, uint32_t chunk, int8_t *o
 int launch_gemv_generic(const Dev &P, const int32_t *prefix, uint32_t chunk, const uint16_t *x, int m,
                         int64_t ldx, uint16_t *y, int64_t ldy, float *y32, float *ws, bool atomic,
                         hipStream_t s);
+bool gemv_staged_supports(const Dev &P, uint32_t chunk, const uint16_t *x, int64_t ldx);
+int launch_gemv_staged(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
+                       int64_t ldy, float *y32, float *ws, bool atomic, hipStream_t s);
 bool decode_staged_supports(const Dev &P, uint32_t chunk, const int8_t *o8, const uint16_t *o16);
 int launch_decode_staged(const Dev &P, const int32_t *prefix, uint16_t *o16, hipStream_t s);
 size_t prefill_workspace_bytes(const Dev &P, uint32_t m_rows);

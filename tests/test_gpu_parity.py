@@ -221,6 +221,26 @@ def test_gemv_wide_rows(oracle, dev, kind, shape):
             check_outputs(run_gemv(dp, 512, x, m, dev, flags=flags), y64, f"{kind} {shape} m={m} flags={flags}")
 
 
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("shape", [(64, 512), (37, 1024), (130, 2048), (24, 8704), (5, 25600)])
+@pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8), (5, 8)])
+def test_gemv_staged(oracle, dev, kind, shape, level_bits):
+    """The any-scheme kernel that stages the streams in LDS: sparse and dense mixes, rows cut into pieces
+    (workspace and atomic combination), level-1 codes wider than 4 bits."""
+    from ixrun_amd import _lib
+
+    out_f, in_f = shape
+    p = make_packed(kind, out_f, in_f, level_bits)
+    dp = device_packed(p, dev)
+    w_bits = oracle.decode_packed_bf16(p)
+    for m in (1, 3, 16):
+        x = activations(m, in_f, seed=m)
+        y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
+        for atomic in (False, True):
+            y = run_gemv(dp, 512, x, m, dev, flags=_lib.IXH_GEMV_STAGED, atomic=atomic)
+            check_outputs(y, y64, f"{kind} {shape} {level_bits} m={m} atomic={atomic}")
+
+
 @pytest.mark.parametrize("shape,level_bits,chunk", [((40, 96), (3, 4, 5, 6, 8), 32), ((33, 100), (3, 5, 8), 50),
                                                     ((64, 1024), (3, 4, 5, 6, 8), 512), ((9, 7), (2, 8), 7)])
 def test_gemv_general_shapes_and_schemes(oracle, dev, shape, level_bits, chunk):
