@@ -28,6 +28,14 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK = 8.0e12  # B/s, MI355X published
 MFMA_BF16_PEAK = 2.5e15  # FLOP/s dense bf16, MI355X published
 
+# HBM bytes per launch of the dominant kernel, from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then
+# WRITE_SIZE, KiB per dispatch, scaled by what the same counters read for the 256 MiB copy of --calibrate-copy:
+# x 2.0 and x 1.0); the counter summaries are kept under profiles/.  Workloads without a counter run report null.
+MEASURED_TRAFFIC_BYTES = {
+    "down_proj_5120x17408_m1_student_t": 23144.3 * 2.0 * 1024 + 16.0 * 1024,
+    "prefill_5120x5120_m512_five_level": 45585.2 * 2.0 * 1024 + 30720.0 * 1024,
+}
+
 WORKLOADS = {
     # name: (out_f, in_f, m, weight recipe)
     "down_proj_5120x17408_m1_student_t": (5120, 17408, 1, "student_t"),
@@ -221,8 +229,9 @@ def main():
         },
         "roofline": {
             "bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK, "traffic": None,
-            "note": "algorithmic bytes = packed layer + x + y per launch; time = HIP-event time of the timed region / steps",
+            "frac": achieved / HBM_PEAK, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "note": "algorithmic bytes = packed layer + x + y per launch; time = HIP-event time of the timed region / "
+                    "steps; traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script",
         },
         "launch": "eager" if graph is None else f"hipGraph of {copies} layer launches, replayed {rounds}x",
         "eager_per_call_us": {"median": float(np.median(per_call)), "min": float(per_call.min()),
@@ -234,7 +243,8 @@ def main():
         flops = 2.0 * m * out_f * in_f
         out["roofline"] = {
             "bound": "mfma", "achieved": flops / (ms_per_step * 1e-3) / 1e12, "peak": MFMA_BF16_PEAK / 1e12,
-            "unit": "TFLOP/s", "frac": flops / (ms_per_step * 1e-3) / MFMA_BF16_PEAK, "traffic": None,
+            "unit": "TFLOP/s", "frac": flops / (ms_per_step * 1e-3) / MFMA_BF16_PEAK,
+            "traffic": None if args.unfused else MEASURED_TRAFFIC_BYTES.get(args.workload),
             "note": "2*M*N*K flops per launch pair (GEMM + slice reduce); the kernel is bound by the VALU decode "
                     "that feeds the matrix cores, not by MFMA issue",
         }

@@ -51,6 +51,9 @@ class IxhError(RuntimeError):
 
 
 _lib = None
+# measurement switch: extra ixh_gemv flags for every call (e.g. 16 = IXH_GEMV_STAGED), to time one kernel
+# against another through the same harness
+_ENV_GEMV_FLAGS = int(os.environ.get("IXH_GEMV_FLAGS", "0"))
 
 EXPORTS = (
     "ixh_version", "ixh_last_error", "ixh_prefix_entries", "ixh_prefix_build", "ixh_decode",
@@ -196,6 +199,7 @@ class DevicePacked:
         m = x2.shape[0]
         ldx = x2.stride(0) if m > 1 else self.in_f
         ldy = y.stride(0) if (y is not None and y.dim() == 2 and m > 1) else self.out_f
+        flags = int(flags) | _ENV_GEMV_FLAGS
         check(lib().ixh_gemv(
             C.byref(self.struct), table.data_ptr(), int(chunk), x2.data_ptr(), m, ldx,
             y.data_ptr() if y is not None else None, ldy,
