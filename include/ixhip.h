@@ -98,6 +98,8 @@ int ixh_prefix_build(const IxhPacked *packed, int64_t chunk, int32_t *prefix, ix
  * _ix_decode_kernel / decode_weight_triton (ixrun/triton_kernels.py:68-177,
  * :224-259) and StreamingLinear._decode (ixrun/engine.py:109-133), for any
  * level scheme.  prefix/chunk: a table from ixh_prefix_build; any chunk > 0.
+ * Fastest with chunk = 512, bf16 output only and a 16-byte aligned out_bf16
+ * (the streams are then staged through on-chip memory).
  */
 int ixh_decode(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, int8_t *out_i8,
                uint16_t *out_bf16, ixh_stream_t stream);
@@ -110,7 +112,8 @@ int ixh_decode(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, in
  * (ixrun/fused.py:84-179, :209-294, :297-347) for M = 1 and the decode +
  * F.linear path of StreamingLinear.forward (ixrun/engine.py:171-173) for
  * 2 <= M <= 16.  chunk must divide in_f; the table must come from
- * ixh_prefix_build(packed, chunk).  Partial sums of the in_f / chunk chunks of
+ * ixh_prefix_build(packed, chunk); chunk = 512 with in_f a multiple of 512 and a
+ * 16-byte aligned x is what the fast kernels take.  Partial sums of the pieces of
  * a row are combined in a fixed order through `workspace`
  * (ixh_gemv_workspace_bytes) and written to y, or, with IXH_GEMV_ATOMIC, added
  * into the caller-zeroed fp32 y32 [M, out_f] with atomics as the reference's
@@ -128,13 +131,13 @@ size_t ixh_gemv_workspace_bytes(const IxhPacked *packed, int64_t chunk, int32_t 
  * w = bf16(f32(v) * f32(scale)) decoded into on-chip memory tile by tile and multiplied
  * on the matrix cores (bf16 x bf16, fp32 accumulate).  Replaces the decode-to-bf16 +
  * F.linear pair of StreamingLinear.forward (ixrun/engine.py:171-173) and of
- * GraphLinear.forward (ixrun/engine.py:214-233), which materialise the whole bf16
+ * GraphLinear.forward (ixrun/engine.py:193-196), which materialise the whole bf16
  * weight in device memory first.  Any m >= 1; x is bf16 [m, ldx], y is bf16 [m, ldy].
  * The table must come from ixh_prefix_build(packed, 512).  Needs in_f a multiple of
- * 512 with in_f >= 4096, x 16-byte aligned with ldx a multiple of 8, and the last-level
+ * 512, x 16-byte aligned with ldx a multiple of 8 and below 2^20, and the last-level
  * stream 4-byte aligned; otherwise IXH_EUNSUPPORTED (the caller then decodes with
- * ixh_decode and multiplies itself).  K is cut into 8 slices whose fp32 partial sums are
- * combined in slice order through `workspace` (ixh_gemm_workspace_bytes).
+ * ixh_decode and multiplies itself).  K is cut into up to 16 slices whose fp32 partial
+ * sums are combined in slice order through `workspace` (ixh_gemm_workspace_bytes).
  */
 int ixh_gemm(const IxhPacked *packed, const int32_t *prefix, const uint16_t *x, int32_t m, int64_t ldx,
              uint16_t *y, int64_t ldy, void *workspace, size_t workspace_bytes, ixh_stream_t stream);

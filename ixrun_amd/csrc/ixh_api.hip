@@ -212,7 +212,7 @@ int ixh_gemm(const IxhPacked *packed, const int32_t *prefix, const uint16_t *x, 
     if (!prefix || !x) { set_error("prefix or x is NULL"); return IXH_EINVAL; }
     if (ldx < (int64_t)d.in_f && m > 1) { set_error("ldx %lld < in_f %u", (long long)ldx, d.in_f); return IXH_EINVAL; }
     if (!prefill_supports(d, x, ldx)) {
-        set_error("gemm: needs in_f %% 512 == 0, in_f >= 4096, x 16-byte aligned, ldx %% 8 == 0, last stream 4-byte aligned");
+        set_error("gemm: needs in_f %% 512 == 0, x 16-byte aligned, ldx %% 8 == 0, last stream 4-byte aligned");
         return IXH_EUNSUPPORTED;
     }
     const size_t need = prefill_workspace_bytes(d, (uint32_t)m);
