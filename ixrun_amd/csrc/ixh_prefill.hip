@@ -3,19 +3,19 @@
 // (v_mfma_f32_32x32x16_bf16, fp32 accumulate); the bf16 weight never reaches HBM.
 // Any level scheme (2..8 levels).
 //
-// A workgroup of 4 waves owns 32 weight rows x up to 512 activation rows x one K slice (a
-// run of 512-element table units); two workgroups share a CU, so that one decodes (VALU)
-// while the other multiplies (MFMA, memory).  Per 512-wide unit column: every wave decodes
-// 8 of the 32 rows into a 32 x 512 bf16 tile in LDS.  The streams of a row unit reach LDS
-// by DMA a few row units ahead of their decode (a ring of slots per wave, ixh_staged.h),
-// and the rank-table entries that say where the streams start are held in registers a
-// column ahead, so that no decode waits on memory.  Then the waves multiply: a wave owns
-// 128 m x 32 n of the output, takes the weight operand from the LDS tile and the
-// activation operand straight from global memory (each lane's 16 bytes are contiguous in a
-// row of X, which is the MFMA operand layout), one block of 64 k ahead of the MFMAs.
-// Partial sums of the K slices go to an fp32 workspace [slice][m][n]; a second kernel adds
-// them in slice order and rounds to bf16.  The number of K slices is chosen per shape so
-// that the workgroups fill the CUs in whole rounds.
+// A workgroup of 8 waves owns 32 weight rows x up to 512 activation rows x one K slice (a
+// run of 512-element table units); two workgroups share a CU (four waves per SIMD), so
+// that one decodes (VALU) while the other multiplies (MFMA, memory).  Per 512-wide unit
+// column: every wave decodes 4 of the 32 rows into a 32 x 512 bf16 tile in LDS.  The
+// streams of a row unit reach LDS by DMA a few row units ahead of their decode (a ring of
+// slots per wave, ixh_staged.h), and the rank-table entries that say where the streams
+// start are held in registers a column ahead, so that no decode waits on memory.  Then the
+// waves multiply: a wave owns 64 m x 32 n of the output, takes the weight operand from
+// the LDS tile and the activation operand straight from global memory (each lane's 16
+// bytes are contiguous in a row of X, which is the MFMA operand layout), one block of
+// 64 k ahead of the MFMAs.  Partial sums of the K slices go to an fp32 workspace
+// [slice][m][n]; a second kernel adds them in slice order and rounds to bf16.  The number
+// of K slices is chosen per shape so that the workgroups fill the CUs in whole rounds.
 #include "ixh_staged.h"
 
 namespace ixh {
@@ -24,18 +24,23 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4p __attribute__((ext_vector_type(4)));
 
-constexpr int kPWaves = 4;
+constexpr int kPWaves = 8;
 constexpr uint32_t kPRows = 32;      // weight rows per workgroup
 constexpr uint32_t kPMaxM = 512;     // activation rows per launch
 constexpr uint32_t kPWStride = 520;  // bf16 per row of the weight tile (512 + pad: 260 words, = 4 mod 32 banks)
 constexpr uint32_t kPMaxSlices = 16;
-constexpr uint32_t kPRing = 4;       // slots per wave: row units in flight ahead of the decode, plus one
+constexpr uint32_t kPRowsPerWave = kPRows / kPWaves;        // rows of the weight tile a wave decodes
+constexpr uint32_t kPMTiles = kPMaxM / (32 * kPWaves);      // 32 x 32 output tiles of a wave
+constexpr uint32_t kPWaveM = 32 * kPMTiles;                 // activation rows of a wave
+// slots per wave: row units in flight ahead of the decode, plus one (fewer for the schemes with large slots, so
+// that two workgroups fit a CU's LDS)
+__host__ __device__ constexpr uint32_t prefill_ring(int n_levels) { return n_levels <= 5 ? 4u : 3u; }
 
 __host__ __device__ constexpr uint32_t prefill_slot_bytes(int n_levels) {
     return ((staged_slot_words(n_levels) + 5u * (uint32_t)(n_levels - 1) + 1u) * 4u + 15u) & ~15u;  // spans + record
 }
 __host__ __device__ constexpr uint32_t prefill_wave_bytes(int n_levels) {
-    return kPRing * prefill_slot_bytes(n_levels) + kStagedQueue * 2u;  // ring + queue of non-level-1 positions
+    return prefill_ring(n_levels) * prefill_slot_bytes(n_levels) + kStagedQueue * 2u;  // ring + queue of non-level-1 positions
 }
 __host__ __device__ constexpr uint32_t prefill_lds_bytes(int n_levels) {
     return kPRows * kPWStride * 2u + kPWaves * prefill_wave_bytes(n_levels);
@@ -54,7 +59,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 // An activation operand register is reloaded for the next block as soon as its MFMA has been issued.
 template <int NT>
 __device__ __forceinline__ void mfma_column(__amdgpu_buffer_rsrc_t x_rs, uint32_t x_off, uint32_t x_tile,
-                                            const uint16_t *b_lane, f32x16 (&acc)[4]) {
+                                            const uint16_t *b_lane, f32x16 (&acc)[kPMTiles]) {
     u32x4p a[NT][4];
 #pragma unroll
     for (int s = 0; s < 4; ++s)
@@ -81,7 +86,7 @@ __device__ __forceinline__ void mfma_column(__amdgpu_buffer_rsrc_t x_rs, uint32_
 }
 
 template <int L>
-__global__ void __launch_bounds__(kWave *kPWaves, 2)
+__global__ void __launch_bounds__(kWave *kPWaves, L <= 5 ? 4 : 2)  // four waves per SIMD (two workgroups per CU) where the registers allow
 k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const uint16_t *__restrict__ x, uint32_t m_rows,
           int64_t ldx, float *__restrict__ ws, uint32_t n_slices
 #ifdef IXH_VARIANTS
@@ -89,7 +94,7 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
 #endif
           ) {
 #ifdef IXH_VARIANTS  // timing experiments only
-#define PF_STAMP(k) do { if (trace && (threadIdx.x & 63) == 0) trace[(blockIdx.x * 4 + (threadIdx.x >> 6)) * 16 + (k)] = wall_clock64(); } while (0)
+#define PF_STAMP(k) do { if (trace && (threadIdx.x & 63) == 0) trace[(blockIdx.x * 8 + (threadIdx.x >> 6)) * 16 + (k)] = wall_clock64(); } while (0)
 #else
 #define PF_STAMP(k) do { } while (0)
 #endif
@@ -97,6 +102,7 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *const wt = reinterpret_cast<uint16_t *>(smem);  // [64][520]
     constexpr int kDma = staged_dma_count(L);
+    constexpr uint32_t kPRing = prefill_ring(L);
     static_assert((kPRing - 1) * kDma < 64, "ring too deep for the wait counter");
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
@@ -104,14 +110,14 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
     const uint32_t slice = blockIdx.x % n_slices, tile = blockIdx.x / n_slices;
     const uint32_t n0 = tile * kPRows;
     const uint32_t c_begin = slice * n_chunks / n_slices, c_end = (slice + 1) * n_chunks / n_slices;
-    const uint32_t total = (c_end - c_begin) * 8;  // row units this wave decodes
+    const uint32_t total = (c_end - c_begin) * kPRowsPerWave;  // row units this wave decodes
     const uint32_t entries = P.out_f * n_chunks + 1;
     const float scale = bf16_bits_to_f32(*P.scale);
 
     uint8_t *const my_area = smem + kPRows * kPWStride * 2 + wave * prefill_wave_bytes(L);
     const uint32_t my_slots = (uint32_t)(uintptr_t)(lds_ptr_t)my_area;
     uint16_t *const queue = reinterpret_cast<uint16_t *>(my_area + kPRing * prefill_slot_bytes(L));
-    const uint32_t row_first = n0 + wave * 8;
+    const uint32_t row_first = n0 + wave * kPRowsPerWave;
 
     // Rank-table entries in registers: lane 8 j + i holds, for row j of this wave and level i, the count before
     // unit column c (q0), c + 1 (q1), c + 2 (q2); the entry for c + 3 is fetched while column c is decoded.
@@ -127,7 +133,7 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
     // row unit t of this wave: column c_begin + t / 8, row t % 8; `ahead` says whether that column is the one
     // being decoded (q0, q1) or the next (q1, q2)
     auto stage_row = [&](uint32_t t, uint32_t c_now) {
-        const uint32_t c = c_begin + (t >> 3), j = t & 7;
+        const uint32_t c = c_begin + t / kPRowsPerWave, j = t % kPRowsPerWave;
         const bool ahead = c != c_now;
         const uint32_t lo = ahead ? q1 : q0, hi = ahead ? q2 : q1;
         uint32_t q_lo[L - 1], q_hi[L - 1];
@@ -144,17 +150,17 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
     for (uint32_t t = 0; t < kPRing - 1 && t < total; ++t) stage_row(t, c_begin);
     PF_STAMP(1);
 
-    // output tile of this wave: m in [128 w, +128), the 32 n of the workgroup
-    const uint32_t m_tiles = 128 * wave < m_rows ? min(4u, (m_rows - 128 * wave + 31) / 32) : 0u;
-    f32x16 acc[4];
+    // output tile of this wave: m in [64 w, +64), the 32 n of the workgroup
+    const uint32_t m_tiles = kPWaveM * wave < m_rows ? min(kPMTiles, (m_rows - kPWaveM * wave + 31) / 32) : 0u;
+    f32x16 acc[kPMTiles];
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < (int)kPMTiles; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[t][r] = 0.0f;
     // X through a buffer descriptor that ends with row m_rows - 1: rows past it read as zero
     const __amdgpu_buffer_rsrc_t x_rs = __builtin_amdgcn_make_buffer_rsrc(
         (void *)x, 0, (int)((((int64_t)m_rows - 1) * ldx + P.in_f) * 2), 0x00020000);
-    const uint32_t x_lane = (uint32_t)(((int64_t)(128 * wave + (lane & 31)) * ldx + 32 * (lane >> 5)) * 2);
+    const uint32_t x_lane = (uint32_t)(((int64_t)(kPWaveM * wave + (lane & 31)) * ldx + 32 * (lane >> 5)) * 2);
     const uint32_t x_tile = (uint32_t)(32 * ldx * 2);
 
     for (uint32_t c = c_begin; c < c_end; ++c) {
@@ -163,8 +169,8 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
         if (c == c_begin) PF_STAMP(2);
         // ---- decode the 64 x 512 weight tile of unit column c: wave w takes rows 8w .. 8w+7 ----
 #pragma unroll 1
-        for (uint32_t j = 0; j < 8; ++j) {
-            const uint32_t t = (c - c_begin) * 8 + j;
+        for (uint32_t j = 0; j < kPRowsPerWave; ++j) {
+            const uint32_t t = (c - c_begin) * kPRowsPerWave + j;
             if (t + kPRing - 1 < total) stage_row(t + kPRing - 1, c);
             // row unit t has landed once at most the loads of the units staged after it are outstanding
             const uint32_t after = min(kPRing - 1, total - 1 - t);
@@ -172,7 +178,7 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
             else if (after == 2) wait_vmcnt<2 * kDma>();
             else if (after == 1) wait_vmcnt<kDma>();
             else wait_vmcnt<0>();
-            uint16_t *wrow = wt + (wave * 8 + j) * kPWStride;
+            uint16_t *wrow = wt + (wave * kPRowsPerWave + j) * kPWStride;
 #ifdef IXH_PF_NO_DECODE
             if (false) {
 #else
@@ -201,8 +207,6 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
 #else
         switch (m_tiles) {
 #endif
-            case 4: mfma_column<4>(x_rs, x_col, x_tile, b_lane, acc); break;
-            case 3: mfma_column<3>(x_rs, x_col, x_tile, b_lane, acc); break;
             case 2: mfma_column<2>(x_rs, x_col, x_tile, b_lane, acc); break;
             case 1: mfma_column<1>(x_rs, x_col, x_tile, b_lane, acc); break;
             default: break;
@@ -215,10 +219,10 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
     const uint32_t n = n0 + (lane & 31);
     if (n < P.out_f) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int t = 0; t < (int)kPMTiles; ++t)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const uint32_t m = 128 * wave + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                const uint32_t m = kPWaveM * wave + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 if (m < m_rows) ws[((size_t)slice * m_rows + m) * P.out_f + n] = acc[t][r];
             }
     }
@@ -299,7 +303,7 @@ static int prefill_launch(const Dev &P, const int32_t *prefix, const uint16_t *x
     for (uint32_t m0 = 0; m0 < m_rows; m0 += kPMaxM) {
         const uint32_t mb = min(kPMaxM, m_rows - m0);
 #ifdef IXH_VARIANTS
-        if (!g_pf_trace) (void)hipMalloc(&g_pf_trace, 2048 * 4 * 16 * 8);
+        if (!g_pf_trace) (void)hipMalloc(&g_pf_trace, 2048 * 8 * 16 * 8);
         hipLaunchKernelGGL(k_prefill<L>, dim3(tiles * n_slices), dim3(kWave * kPWaves), lds, s, P, prefix, n_chunks,
                            x + (int64_t)m0 * ldx, mb, ldx, ws, n_slices, tiles * n_slices <= 2048 ? g_pf_trace : nullptr);
 #else
