@@ -138,6 +138,7 @@ __device__ __forceinline__ int decode_from_lds(const Dev &P, const StagedUnit<L>
 #pragma unroll
     for (int i = START; i < L - 1; ++i) {
         const uint64_t alive_mask = __ballot(alive);
+        if (alive_mask == 0) return v;  // every element has found its level: the deeper counts do not move
         const uint32_t rel = space + S.bm_off[i] + lanes_below(alive_mask);  // bit inside the staged span
         uint32_t bit = 0;
         if (alive) bit = (slds_u32(S.bm_addr[i] + (rel >> 5) * 4) >> (rel & 31)) & 1u;
@@ -225,27 +226,33 @@ __device__ __forceinline__ void decode_unit_lds(const Dev &P, const StagedUnit<L
         clo = __builtin_amdgcn_alignbit(w1, w0, bitpos);
         chi = __builtin_amdgcn_alignbit(w2, w1, bitpos);
     }
-    float f[8];
+    int v[8];  // values of the lane's eight elements (0 until a level claims the element)
     uint32_t off = 0;
     if (b <= 4) {  // eight codes fit 32 bits
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
             const uint32_t bit = (m >> t) & 1u;
-            const int v = ((int)__builtin_amdgcn_ubfe(clo, off, b) - thr) * (int)bit;
-            f[t] = (float)v * scale;
+            v[t] = ((int)__builtin_amdgcn_ubfe(clo, off, b) - thr) * (int)bit;
             off += bit * b;
         }
     } else {
+        const uint64_t window = ((uint64_t)chi << 32) | clo;
         const uint32_t code_mask = (1u << b) - 1u;
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
             const uint32_t bit = (m >> t) & 1u;
-            const uint32_t w = off < 32 ? __builtin_amdgcn_alignbit(chi, clo, off) : chi >> (off - 32);
-            const int v = ((int)(w & code_mask) - thr) * (int)bit;
-            f[t] = (float)v * scale;
+            v[t] = ((int)((uint32_t)(window >> off) & code_mask) - thr) * (int)bit;
             off += bit * b;
         }
     }
+    auto store = [&]() {  // dequantise, round to bf16, one 16-byte write
+        float f[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) f[t] = (float)v[t] * scale;
+        const staged_u32x4 packed = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                                     pack_bf16x2(f[6], f[7])};
+        *reinterpret_cast<staged_u32x4 *>(dst + e0) = packed;
+    };
     const uint32_t n_queued = n_el - n_taken;
     if (n_queued > kWave) {
         // Many elements above level 1 (a dense mix): the lane keeps its eight elements through every level.
@@ -267,15 +274,15 @@ __device__ __forceinline__ void decode_unit_lds(const Dev &P, const StagedUnit<L
             const uint32_t bitpos = (S.cnt0[i] + inc - n_t) * bi + S.st_off[i];
             const uint32_t wa = S.st_addr[i] + (bitpos >> 5) * 4;
             const uint32_t w0 = slds_u32(wa), w1 = slds_u32(wa + 4), w2 = slds_u32(wa + 8);
-            const uint32_t lo = __builtin_amdgcn_alignbit(w1, w0, bitpos), hi = __builtin_amdgcn_alignbit(w2, w1, bitpos);
+            const uint64_t window =
+                ((uint64_t)__builtin_amdgcn_alignbit(w2, w1, bitpos) << 32) | __builtin_amdgcn_alignbit(w1, w0, bitpos);
             uint32_t pos = 0, idx = 0, still = 0;
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
                 const uint32_t a_t = (alive >> t) & 1u;
                 const uint32_t bit = (bits >> idx) & a_t;
-                const uint32_t w = pos < 32 ? __builtin_amdgcn_alignbit(hi, lo, pos) : hi >> (pos - 32);
-                const float val = (float)((int)(w & code_mask) - thr_i) * scale;
-                f[t] = bit ? val : f[t];
+                const int val = (int)((uint32_t)(window >> pos) & code_mask) - thr_i;
+                v[t] = bit ? val : v[t];
                 pos += bit * bi;
                 idx += a_t;
                 still |= (a_t ^ bit) << t;
@@ -288,26 +295,21 @@ __device__ __forceinline__ void decode_unit_lds(const Dev &P, const StagedUnit<L
             const uint32_t addr = S.last_off + space + before;
             const uint32_t wa = addr & ~3u, sh = (addr & 3u) * 8u;
             const uint32_t w0 = slds_u32(wa), w1 = slds_u32(wa + 4), w2 = slds_u32(wa + 8);
-            const uint32_t lo = __builtin_amdgcn_alignbit(w1, w0, sh), hi = __builtin_amdgcn_alignbit(w2, w1, sh);
+            const uint64_t window =
+                ((uint64_t)__builtin_amdgcn_alignbit(w2, w1, sh) << 32) | __builtin_amdgcn_alignbit(w1, w0, sh);
             uint32_t pos = 0;
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
                 const uint32_t a_t = (alive >> t) & 1u;
-                const uint32_t w = pos < 32 ? __builtin_amdgcn_alignbit(hi, lo, pos) : hi >> (pos - 32);
-                const float val = (float)((int)(w & 0xFFu) - 127) * scale;
-                f[t] = a_t ? val : f[t];
+                const int val = (int)((uint32_t)(window >> pos) & 0xFFu) - 127;
+                v[t] = a_t ? val : v[t];
                 pos += a_t * 8u;
             }
         }
-        const staged_u32x4 packed = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
-                                     pack_bf16x2(f[6], f[7])};
-        *reinterpret_cast<staged_u32x4 *>(dst + e0) = packed;
+        store();
         return;
     }
-
-    const staged_u32x4 packed = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
-                                 pack_bf16x2(f[6], f[7])};
-    *reinterpret_cast<staged_u32x4 *>(dst + e0) = packed;
+    store();
 
     // positions of the elements above level 1, in order
     {
@@ -323,8 +325,8 @@ __device__ __forceinline__ void decode_unit_lds(const Dev &P, const StagedUnit<L
     for (uint32_t base = 0; base < n_queued; base += kWave) {
         const bool alive = base + lane < n_queued;
         const uint32_t p = alive ? queue[base + lane] : 0u;
-        const int v = decode_from_lds<L, 1>(P, S, space1 + base, alive, cnt);
-        if (alive) dst[p] = (uint16_t)f32_to_bf16_bits((float)v * scale);
+        const int ve = decode_from_lds<L, 1>(P, S, space1 + base, alive, cnt);
+        if (alive) dst[p] = (uint16_t)f32_to_bf16_bits((float)ve * scale);
     }
 }
 
