@@ -43,6 +43,7 @@ typedef __attribute__((address_space(3))) void *lds_ptr_t;
 constexpr int kRStages = 3;              // unit-quads in flight per wave
 constexpr uint32_t kRStageBytes = 1280;  // 1024 stream + 256 bitmap
 constexpr uint32_t kRQueue = 128;        // records per wave
+constexpr uint32_t kRTasks = 192;        // elements above level 1 of 64 records that are spread over the lanes
 constexpr uint32_t kRSlots = 64;         // rows per workgroup at most
 constexpr int kRMaxWaves = 12;           // waves per workgroup at most: 3 per SIMD, up to 168 VGPRs each
 constexpr uint32_t kRLutBytes = 64 * 32 * 4;
@@ -55,7 +56,7 @@ constexpr uint32_t kFlagStageSide = 2u;  // the 8-bit stream is dword aligned, t
 constexpr uint32_t kZeroCodes0 = 0xDB6DB6DBu, kZeroCodes1 = 0xB6DB6DB6u, kZeroCodes2 = 0x6DB6DB6Du;
 
 __host__ __device__ constexpr uint32_t wave_lds_bytes(int mt) {
-    return kRStages * kRStageBytes + kRQueue * 16 + kRSlots * mt * 4;
+    return kRStages * kRStageBytes + kRQueue * 16 + kRSlots * mt * 4 + kRTasks * 2;
 }
 
 // byte offsets of the regions of a workgroup's LDS; the pair table is at 0, the splice masks follow
@@ -124,71 +125,102 @@ struct SideView {
     uint32_t b2w0, l2w0, l3w0;  // first staged word of bitmap 1 / 5-bit stream / 8-bit stream
 };
 
-// Resolve queued lanes: every record is one bitmap word with elements above
-// level 1; the lane that takes it walks those elements and adds x*w to the row sums.
+// inclusive sum over the lanes at or below this one
+__device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
+    v = row_scan(v);
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1, 3
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2, 3
+    return v;
+}
+
+// Resolve queued records: every record is one bitmap word with elements above level 1.  The elements of 64
+// records are first spread over the lanes (one element per lane and round, through a task list in LDS), so
+// that the dependent reads of an element (bitmap 1, its code, x) are paid once per round and not once per
+// element of the fullest record; a batch with more than kRTasks elements is walked record by record instead.
 template <int MT>
 __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, uint32_t tq1_addr, uint32_t tq2_addr,
                                              uint32_t unit0, const uint4 *queue, uint32_t count, float *rowacc,
-                                             const uint16_t *__restrict__ x, int m,
+                                             uint16_t *tasks, const uint16_t *__restrict__ x, int m,
                                              int64_t ldx, float scale, uint32_t lane) {
     const uint32_t *__restrict__ b2 = P.bm[1];
     const uint32_t b2_words = P.bm_words[1];
+    // element `e` (bit of the record's word), the nth element above level 1 of its record
+    auto one = [&](const uint4 rec, uint32_t nth, uint32_t e) {
+        const uint32_t r0_lane = rec.y, unit = rec.z;
+        const uint32_t slot = rec.w >> 16, k0 = rec.w & 0xFFFFu;
+        // the activations this element meets: requested first, they arrive while the element is ranked
+        uint16_t xe[MT];
+#pragma unroll
+        for (int j = 0; j < MT; ++j) xe[j] = j < m ? x[(int64_t)j * ldx + k0 + e] : (uint16_t)0;
+        const uint32_t r0u = unit * kFastChunk - lds_u32(tq1_addr + (unit - unit0) * 4);
+        const uint32_t q2u = lds_u32(tq2_addr + (unit - unit0) * 4);
+        const uint32_t wf = r0u >> 5;
+        const uint32_t first_mask = ~0u << (r0u & 31);
+        const uint32_t r = r0_lane + nth;
+        // level-2 elements among bitmap-1 bits [r0u, r) (a unit spans at most 17 words), and the bit at r
+        const uint32_t wl = min(r >> 5, wf + 17u);
+        uint32_t cnt = 0;
+        for (uint32_t w = wf; w < wl; ++w) {
+            uint32_t bits = sv.staged ? lds_u32(sv.base + kRSideB2 + (w - sv.b2w0) * 4) : (w < b2_words ? b2[w] : 0u);
+            if (w == wf) bits &= first_mask;
+            cnt += __popc(bits);
+        }
+        const uint32_t bits = sv.staged ? lds_u32(sv.base + kRSideB2 + (wl - sv.b2w0) * 4)
+                                        : (wl < b2_words ? b2[wl] : 0u);
+        uint32_t low = (1u << (r & 31)) - 1u;
+        if (wl == wf) low &= first_mask;
+        cnt += __popc(bits & low);
+        int v = 0;
+        if ((bits >> (r & 31)) & 1u) {
+            const uint64_t bitpos = (uint64_t)(q2u + cnt) * 5u;
+            const uint32_t wi = (uint32_t)(bitpos >> 5), sh = (uint32_t)bitpos & 31u;
+            uint32_t lo, hi;
+            if (sv.staged) {
+                lo = lds_u32(sv.base + kRSideL2 + (wi - sv.l2w0) * 4);
+                hi = lds_u32(sv.base + kRSideL2 + (wi - sv.l2w0) * 4 + 4);
+            } else {
+                lo = wi < P.st_words[1] ? P.st[1][wi] : 0u;
+                hi = (sh > 27 && wi + 1 < P.st_words[1]) ? P.st[1][wi + 1] : 0u;
+            }
+            v = (int)((uint32_t)((((uint64_t)hi << 32) | lo) >> sh) & 31u) - 15;
+        } else {
+            const uint32_t i3 = r - (q2u + cnt);
+            // (the staged copy is made of whole dwords: the stream's last 1..3 bytes come from memory)
+            if (sv.staged && i3 < (P.last_bytes & ~3u)) v = (int)lds_u8(sv.base + kRSideL3 + (i3 - sv.l3w0 * 4)) - 127;
+            else v = i3 < P.last_bytes ? (int)P.last[i3] - 127 : 0;
+        }
+        const float w = dequant(v, scale);
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+            if (j < m) atomicAdd(&rowacc[slot * MT + j], bf16_bits_to_f32(xe[j]) * w);
+    };
     for (uint32_t base = 0; base < count; base += kWave) {
         const uint32_t idx = base + lane;
-        if (idx < count) {
-            const uint4 rec = queue[idx];
-            uint32_t zeros = rec.x;
-            const uint32_t r0_lane = rec.y, unit = rec.z;
-            const uint32_t slot = rec.w >> 16, k0 = rec.w & 0xFFFFu;
-            const uint32_t r0u = unit * kFastChunk - lds_u32(tq1_addr + (unit - unit0) * 4);
-            const uint32_t q2u = lds_u32(tq2_addr + (unit - unit0) * 4);
-            const uint32_t wf = r0u >> 5;
-            const uint32_t first_mask = ~0u << (r0u & 31);
+        const bool has = idx < count;
+        uint4 rec = make_uint4(0, 0, 0, 0);
+        if (has) rec = queue[idx];
+        uint32_t zeros = rec.x;
+        const uint32_t mine = (uint32_t)__popc(zeros);
+        const uint32_t incl = wave_scan(mine);
+        const uint32_t n_tasks = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+        if (n_tasks <= kRTasks) {
+            uint32_t t = incl - mine, nth = 0;
+            while (zeros != 0) {
+                tasks[t++] = (uint16_t)((lane << 10) | (nth++ << 5) | (uint32_t)__builtin_ctz(zeros));
+                zeros &= zeros - 1;
+            }
+            for (uint32_t tb = 0; tb < n_tasks; tb += kWave) {
+                if (tb + lane < n_tasks) {
+                    const uint32_t task = tasks[tb + lane];
+                    one(queue[base + (task >> 10)], (task >> 5) & 31u, task & 31u);
+                }
+            }
+        } else {
             uint32_t nth = 0;
             while (zeros != 0) {
-                const uint32_t e = __builtin_ctz(zeros);
+                const uint32_t e = (uint32_t)__builtin_ctz(zeros);
                 zeros &= zeros - 1;
-                const uint32_t r = r0_lane + nth++;
-                // level-2 elements among bitmap-1 bits [r0u, r) (a unit spans at most 17 words), and the bit at r
-                const uint32_t wl = min(r >> 5, wf + 17u);
-                uint32_t cnt = 0;
-                for (uint32_t w = wf; w < wl; ++w) {
-                    uint32_t bits = sv.staged ? lds_u32(sv.base + kRSideB2 + (w - sv.b2w0) * 4)
-                                              : (w < b2_words ? b2[w] : 0u);
-                    if (w == wf) bits &= first_mask;
-                    cnt += __popc(bits);
-                }
-                const uint32_t bits = sv.staged ? lds_u32(sv.base + kRSideB2 + (wl - sv.b2w0) * 4)
-                                                : (wl < b2_words ? b2[wl] : 0u);
-                uint32_t low = (1u << (r & 31)) - 1u;
-                if (wl == wf) low &= first_mask;
-                cnt += __popc(bits & low);
-                int v = 0;
-                if ((bits >> (r & 31)) & 1u) {
-                    const uint64_t bitpos = (uint64_t)(q2u + cnt) * 5u;
-                    const uint32_t wi = (uint32_t)(bitpos >> 5), s = (uint32_t)bitpos & 31u;
-                    uint32_t lo, hi;
-                    if (sv.staged) {
-                        lo = lds_u32(sv.base + kRSideL2 + (wi - sv.l2w0) * 4);
-                        hi = lds_u32(sv.base + kRSideL2 + (wi - sv.l2w0) * 4 + 4);
-                    } else {
-                        lo = wi < P.st_words[1] ? P.st[1][wi] : 0u;
-                        hi = (s > 27 && wi + 1 < P.st_words[1]) ? P.st[1][wi + 1] : 0u;
-                    }
-                    v = (int)((uint32_t)((((uint64_t)hi << 32) | lo) >> s) & 31u) - 15;
-                } else {
-                    const uint32_t i3 = r - (q2u + cnt);
-                    // (the staged copy is made of whole dwords: the stream's last 1..3 bytes come from memory)
-                    if (sv.staged && i3 < (P.last_bytes & ~3u)) v = (int)lds_u8(sv.base + kRSideL3 + (i3 - sv.l3w0 * 4)) - 127;
-                    else v = i3 < P.last_bytes ? (int)P.last[i3] - 127 : 0;
-                }
-                const float w = dequant(v, scale);
-#pragma unroll
-                for (int j = 0; j < MT; ++j) {
-                    if (j < m) {
-                        atomicAdd(&rowacc[slot * MT + j], bf16_bits_to_f32(x[(int64_t)j * ldx + k0 + e]) * w);
-                    }
-                }
+                one(rec, nth++, e);
             }
         }
     }
@@ -241,6 +273,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     uint8_t *const ring = wave_base;
     uint4 *const queue = reinterpret_cast<uint4 *>(wave_base + kRStages * kRStageBytes);
     float *const rowacc = reinterpret_cast<float *>(wave_base + kRStages * kRStageBytes + kRQueue * 16);
+    uint16_t *const tasks = reinterpret_cast<uint16_t *>(rowacc + kRSlots * MT);
 
     // ---- workgroup set-up: table slices and x first (they wait on memory), then the tables built here ----
     const uint32_t unit0 = row0 * n_chunks;
@@ -422,7 +455,8 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     };
 
     auto resolve = [&]() {
-        resolve_rows<MT>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc, x, m, ldx, scale,
+        if (!(dbg & 128))
+        resolve_rows<MT>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc, tasks, x, m, ldx, scale,
                          lane);
         qcount = 0;
     };
@@ -494,6 +528,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
             }
 
             // lanes with more than one element above level 1 (rare): splice on
+            if (!(dbg & 256))
             while (__ballot(nzrem != 0) != 0) splice_once(nw0, nw1, nw2, nzrem);
             cw0 = nw0; cw1 = nw1; cw2 = nw2;
         }
