@@ -55,8 +55,10 @@ constexpr uint32_t kFlagStageSide = 2u;  // the 8-bit stream is dword aligned, t
 
 constexpr uint32_t kZeroCodes0 = 0xDB6DB6DBu, kZeroCodes1 = 0xB6DB6DB6u, kZeroCodes2 = 0x6DB6DB6Du;
 
-__host__ __device__ constexpr uint32_t wave_lds_bytes(int mt) {
-    return kRStages * kRStageBytes + kRQueue * 16 + kRSlots * mt * 4 + kRTasks * 2;
+// a wave's region: ring, record queue, row sums, task list, and a copy of the activations of its own column
+// blocks (c blocks x mt rows x 512 bf16) for the elements above level 1
+__host__ __device__ constexpr uint32_t wave_lds_bytes(int mt, int c) {
+    return kRStages * kRStageBytes + kRQueue * 16 + kRSlots * mt * 4 + kRTasks * 2 + (uint32_t)(c * mt) * kFastChunk * 2;
 }
 
 // byte offsets of the regions of a workgroup's LDS; the pair table is at 0, the splice masks follow
@@ -64,14 +66,15 @@ struct RowsLds {
     uint32_t tq1, tq2, side, waves, total;
 };
 
-__host__ __device__ inline RowsLds rows_layout(uint32_t rows_cap, uint32_t n_chunks, uint32_t n_waves, int mt) {
+__host__ __device__ inline RowsLds rows_layout(uint32_t rows_cap, uint32_t n_chunks, uint32_t n_waves, int mt,
+                                               int c) {
     RowsLds L;
     const uint32_t tbl = ((rows_cap * n_chunks + 1u + 3u) & ~3u) * 4u;  // one entry past the slice: its end ranks
     L.tq1 = kRLutBytes + kRSpliceBytes;
     L.tq2 = L.tq1 + tbl;
     L.side = L.tq2 + tbl;
     L.waves = L.side + kRSideBytes;
-    L.total = L.waves + n_waves * wave_lds_bytes(mt);
+    L.total = L.waves + n_waves * wave_lds_bytes(mt, c);
     return L;
 }
 
@@ -125,6 +128,23 @@ struct SideView {
     uint32_t b2w0, l2w0, l3w0;  // first staged word of bitmap 1 / 5-bit stream / 8-bit stream
 };
 
+// A store through a restrict-qualified parameter: once inlined it carries alias-scope information, which is
+// what keeps the compiler from putting "wait for every LDS-DMA copy in flight" (s_waitcnt vmcnt(0)) in front
+// of an LDS access that has nothing to do with the ring the copies land in.
+__device__ __forceinline__ void push_record(uint4 *__restrict__ q, uint32_t idx, uint4 v) { q[idx] = v; }
+
+// Two LDS operations issued outside the compiler's memory model, for the code that runs while the wave has
+// LDS-DMA copies in flight: in front of a merged two-word LDS read and of an LDS atomic the compiler puts
+// "wait for every copy" (it cannot tell that they do not touch the ring), which would stall the ring.
+__device__ __forceinline__ uint64_t lds_read2_raw(uint32_t addr) {  // words at addr and addr + 4
+    uint64_t v;
+    asm volatile("ds_read2_b32 %0, %1 offset1:1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+}
+__device__ __forceinline__ void lds_add_f32_raw(uint32_t addr, float v) {  // complete after s_waitcnt lgkmcnt(0)
+    asm volatile("ds_add_f32 %0, %1" ::"v"(addr), "v"(v) : "memory");
+}
+
 // inclusive sum over the lanes at or below this one
 __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
     v = row_scan(v);
@@ -137,21 +157,24 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
 // records are first spread over the lanes (one element per lane and round, through a task list in LDS), so
 // that the dependent reads of an element (bitmap 1, its code, x) are paid once per round and not once per
 // element of the fullest record; a batch with more than kRTasks elements is walked record by record instead.
-template <int MT>
+// STAGED: the workgroup's share of bitmap 1 and of the 5-bit / 8-bit streams is in LDS; that version reads
+// no global memory at all (the activations come from the wave's LDS copy), so nothing in it waits for the
+// copies the wave has in flight: a load from global memory returns behind all of them.
+template <int MT, bool STAGED>
 __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, uint32_t tq1_addr, uint32_t tq2_addr,
-                                             uint32_t unit0, const uint4 *queue, uint32_t count, float *rowacc,
-                                             uint16_t *tasks, const uint16_t *__restrict__ x, int m,
-                                             int64_t ldx, float scale, uint32_t lane) {
+                                             uint32_t unit0, const uint4 *__restrict__ queue, uint32_t count,
+                                             uint32_t rowacc_addr, uint16_t *__restrict__ tasks,
+                                             uint32_t xs_addr, uint32_t xs_row, uint32_t k_first,
+                                             int m, float scale, uint32_t lane) {
     const uint32_t *__restrict__ b2 = P.bm[1];
     const uint32_t b2_words = P.bm_words[1];
     // element `e` (bit of the record's word), the nth element above level 1 of its record
     auto one = [&](const uint4 rec, uint32_t nth, uint32_t e) {
         const uint32_t r0_lane = rec.y, unit = rec.z;
         const uint32_t slot = rec.w >> 16, k0 = rec.w & 0xFFFFu;
-        // the activations this element meets: requested first, they arrive while the element is ranked
-        uint16_t xe[MT];
+        uint32_t xe[MT];  // the activations this element meets
 #pragma unroll
-        for (int j = 0; j < MT; ++j) xe[j] = j < m ? x[(int64_t)j * ldx + k0 + e] : (uint16_t)0;
+        for (int j = 0; j < MT; ++j) xe[j] = lds_u16(xs_addr + ((uint32_t)j * xs_row + k0 - k_first + e) * 2u);
         const uint32_t r0u = unit * kFastChunk - lds_u32(tq1_addr + (unit - unit0) * 4);
         const uint32_t q2u = lds_u32(tq2_addr + (unit - unit0) * 4);
         const uint32_t wf = r0u >> 5;
@@ -161,12 +184,12 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
         const uint32_t wl = min(r >> 5, wf + 17u);
         uint32_t cnt = 0;
         for (uint32_t w = wf; w < wl; ++w) {
-            uint32_t bits = sv.staged ? lds_u32(sv.base + kRSideB2 + (w - sv.b2w0) * 4) : (w < b2_words ? b2[w] : 0u);
+            uint32_t bits = STAGED ? lds_u32(sv.base + kRSideB2 + (w - sv.b2w0) * 4) : (w < b2_words ? b2[w] : 0u);
             if (w == wf) bits &= first_mask;
             cnt += __popc(bits);
         }
-        const uint32_t bits = sv.staged ? lds_u32(sv.base + kRSideB2 + (wl - sv.b2w0) * 4)
-                                        : (wl < b2_words ? b2[wl] : 0u);
+        const uint32_t bits = STAGED ? lds_u32(sv.base + kRSideB2 + (wl - sv.b2w0) * 4)
+                                     : (wl < b2_words ? b2[wl] : 0u);
         uint32_t low = (1u << (r & 31)) - 1u;
         if (wl == wf) low &= first_mask;
         cnt += __popc(bits & low);
@@ -175,9 +198,10 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
             const uint64_t bitpos = (uint64_t)(q2u + cnt) * 5u;
             const uint32_t wi = (uint32_t)(bitpos >> 5), sh = (uint32_t)bitpos & 31u;
             uint32_t lo, hi;
-            if (sv.staged) {
-                lo = lds_u32(sv.base + kRSideL2 + (wi - sv.l2w0) * 4);
-                hi = lds_u32(sv.base + kRSideL2 + (wi - sv.l2w0) * 4 + 4);
+            if (STAGED) {
+                const uint64_t pair = lds_read2_raw(sv.base + kRSideL2 + (wi - sv.l2w0) * 4);
+                lo = (uint32_t)pair;
+                hi = (uint32_t)(pair >> 32);
             } else {
                 lo = wi < P.st_words[1] ? P.st[1][wi] : 0u;
                 hi = (sh > 27 && wi + 1 < P.st_words[1]) ? P.st[1][wi + 1] : 0u;
@@ -185,14 +209,13 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
             v = (int)((uint32_t)((((uint64_t)hi << 32) | lo) >> sh) & 31u) - 15;
         } else {
             const uint32_t i3 = r - (q2u + cnt);
-            // (the staged copy is made of whole dwords: the stream's last 1..3 bytes come from memory)
-            if (sv.staged && i3 < (P.last_bytes & ~3u)) v = (int)lds_u8(sv.base + kRSideL3 + (i3 - sv.l3w0 * 4)) - 127;
+            if (STAGED) v = i3 < P.last_bytes ? (int)lds_u8(sv.base + kRSideL3 + (i3 - sv.l3w0 * 4)) - 127 : 0;
             else v = i3 < P.last_bytes ? (int)P.last[i3] - 127 : 0;
         }
         const float w = dequant(v, scale);
 #pragma unroll
         for (int j = 0; j < MT; ++j)
-            if (j < m) atomicAdd(&rowacc[slot * MT + j], bf16_bits_to_f32(xe[j]) * w);
+            if (j < m) lds_add_f32_raw(rowacc_addr + (slot * MT + j) * 4, bf16_bits_to_f32(xe[j]) * w);
     };
     for (uint32_t base = 0; base < count; base += kWave) {
         const uint32_t idx = base + lane;
@@ -224,6 +247,7 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
             }
         }
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the row sums have taken the additions
 }
 
 template <int MT, int C>
@@ -255,7 +279,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     const uint32_t n_steps = min(quads_per_wg, n_quads - quad0);
     const uint32_t row0 = quad0 * 4;
     const uint32_t rows_here = min(n_steps * 4, P.out_f - row0);
-    const RowsLds L = rows_layout(min(quads_per_wg * 4, P.out_f), n_chunks, n_waves, MT);
+    const RowsLds L = rows_layout(min(quads_per_wg * 4, P.out_f), n_chunks, n_waves, MT, C);
 
     // The pair table is addressed with (index bits | lane bits), which needs it at
     // LDS address 0; that holds because the kernel has no other LDS.  Should it
@@ -269,11 +293,12 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     uint4 *const splice = reinterpret_cast<uint4 *>(smem + kRLutBytes);  // [33][2]
     uint32_t *const tq1 = reinterpret_cast<uint32_t *>(smem + L.tq1);
     uint32_t *const tq2 = reinterpret_cast<uint32_t *>(smem + L.tq2);
-    uint8_t *const wave_base = smem + L.waves + wave * wave_lds_bytes(MT);
+    uint8_t *const wave_base = smem + L.waves + wave * wave_lds_bytes(MT, C);
     uint8_t *const ring = wave_base;
     uint4 *const queue = reinterpret_cast<uint4 *>(wave_base + kRStages * kRStageBytes);
     float *const rowacc = reinterpret_cast<float *>(wave_base + kRStages * kRStageBytes + kRQueue * 16);
     uint16_t *const tasks = reinterpret_cast<uint16_t *>(rowacc + kRSlots * MT);
+    uint32_t *const xs = reinterpret_cast<uint32_t *>(tasks + kRTasks);  // [MT][C * 512] bf16
 
     // ---- workgroup set-up: table slices and x first (they wait on memory), then the tables built here ----
     const uint32_t unit0 = row0 * n_chunks;
@@ -329,6 +354,14 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
 #pragma unroll
                 for (int t = 0; t < 16; ++t) xr[cc][j][t] = 0u;
             }
+            // The wave's LDS copy.  All four 16-lane rows write (the same values to the same place) on purpose:
+            // a store under a lane condition would leave the loads above "possibly pending" on the path around
+            // it, and the compiler would then wait for them inside the main loop, where the wait also covers
+            // the copies in flight.
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                *reinterpret_cast<u32x4 *>(xs + (j * C + cc) * (kFastChunk / 2) + li * 16 + 4 * t) =
+                    u32x4{xr[cc][j][4 * t], xr[cc][j][4 * t + 1], xr[cc][j][4 * t + 2], xr[cc][j][4 * t + 3]};
         }
     }
 
@@ -361,7 +394,9 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
             const __amdgpu_buffer_rsrc_t l2_rsrc =
                 __builtin_amdgcn_make_buffer_rsrc((void *)P.st[1], 0, (int)(P.st_words[1] * 4u), 0x00020000);
             const __amdgpu_buffer_rsrc_t l3_rsrc =
-                __builtin_amdgcn_make_buffer_rsrc((void *)P.last, 0, (int)P.last_bytes, 0x00020000);
+                // whole dwords: the range check is per dword, and the stream's last 1..3 bytes are wanted too
+                // (device allocations are 256-byte granular, so the dword is there to read)
+                __builtin_amdgcn_make_buffer_rsrc((void *)P.last, 0, (int)((P.last_bytes + 3u) & ~3u), 0x00020000);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(b2_rsrc, (lds_ptr_t)(smem + L.side + kRSideB2), 16,
                                                      (int)(sv.b2w0 * 4 + lane * 16), 0, 0, 0);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(l2_rsrc, (lds_ptr_t)(smem + L.side + kRSideL2), 16,
@@ -446,18 +481,24 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
         if (zeros != 0) {
             const uint32_t unit = unit0 + lrn + col;
             const uint32_t r0_lane = unit * kFastChunk + li * 32u - (q1u + excl);
-            queue[qcount + lanes_below(any)] =
-                make_uint4(zeros, r0_lane, unit, (slot << 16) | (col * kFastChunk + li * 32u));
+            push_record(queue, qcount + lanes_below(any),
+                        make_uint4(zeros, r0_lane, unit, (slot << 16) | (col * kFastChunk + li * 32u)));
         }
         qcount += (uint32_t)__popcll(any);
         zrem = zeros;
         splice_once(w0, w1, w2, zrem);
     };
 
+    const uint32_t xs_addr = (uint32_t)(uintptr_t)(lds_ptr_t)xs;
+    const uint32_t rowacc_addr = (uint32_t)(uintptr_t)(lds_ptr_t)rowacc;
     auto resolve = [&]() {
-        if (!(dbg & 128))
-        resolve_rows<MT>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc, tasks, x, m, ldx, scale,
-                         lane);
+        if (dbg & 128) {
+        } else if (sv.staged)
+            resolve_rows<MT, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks, xs_addr,
+                                   C * kFastChunk, col0 * kFastChunk, m, scale, lane);
+        else
+            resolve_rows<MT, false>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks, xs_addr,
+                                    C * kFastChunk, col0 * kFastChunk, m, scale, lane);
         qcount = 0;
     };
 
@@ -564,7 +605,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
         if ((int)j >= m) continue;
         float sum = 0.0f;
         for (uint32_t w = 0; w < n_waves; ++w)
-            sum += *reinterpret_cast<const float *>(smem + first_acc + w * wave_lds_bytes(MT) + t * 4);
+            sum += *reinterpret_cast<const float *>(smem + first_acc + w * wave_lds_bytes(MT, C) + t * 4);
         y[(int64_t)j * ldy + row0 + slot] = (uint16_t)f32_to_bf16_bits(sum);
     }
     IXH_STAMP(6);
@@ -598,7 +639,7 @@ static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, c
     static int per_cu_cache[17] = {0};
     int per_cu = per_cu_cache[waves];
     if (per_cu == 0) {
-        const size_t probe = rows_layout(min(16u, P.out_f), n_chunks, waves, MT).total;
+        const size_t probe = rows_layout(min(16u, P.out_f), n_chunks, waves, MT, C).total;
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rows<MT, C>, (int)(waves * kWave), probe) !=
                 hipSuccess || per_cu < 1)
             per_cu = -1;
@@ -620,7 +661,7 @@ static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, c
     const uint32_t rows_cap = min(quads * 4, P.out_f);
     uint32_t flags = 0;
     if (((uintptr_t)P.last & 3u) == 0) flags |= kFlagStageSide;
-    const size_t lds = rows_layout(rows_cap, n_chunks, waves, MT).total;
+    const size_t lds = rows_layout(rows_cap, n_chunks, waves, MT, C).total;
     if (lds > kLdsLimit) return IXH_EUNSUPPORTED;
     if (lds > 64 * 1024) {
         static bool raised = false;  // per instantiation
