@@ -1,9 +1,8 @@
 // Full decode to bf16 through LDS-staged streams: every wave walks a contiguous run of
 // 512-element table units, copies each unit's spans of every stream into LDS by DMA a few
 // units ahead (ring of slots, ixh_staged.h), decodes the unit into an LDS row and stores it
-// with one 16-byte write per lane.  Table entries for eight units at a time are held in
-// registers (lane 8 j + i: unit j of the batch, level i), the next batch is fetched while the
-// current one is decoded.  Needs the table at unit 512 and 16-byte aligned output.
+// with one 16-byte write per lane.  The table entries of a unit arrive one unit ahead of its
+// staging through scalar loads.  Needs the table at unit 512 and 16-byte aligned output.
 #include "ixh_staged.h"
 
 namespace ixh {
@@ -44,41 +43,22 @@ k_decode_staged(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, uin
     uint16_t *const queue = reinterpret_cast<uint16_t *>(my_area + kDRing * dstaged_slot_bytes(L));
     uint16_t *const row = queue + kStagedQueue;
 
-    const uint32_t t_lev = lane & 7, t_unit = lane >> 3;
-    const bool t_has = t_lev < (uint32_t)(L - 1);
-    const int32_t *const t_base = prefix + (size_t)(t_has ? t_lev : 0) * entries;
-    // entries of unit (batch, j) and of the unit after it; units past the end repeat the last entry
-    auto table_lo = [&](uint32_t batch) -> uint32_t {
-        return t_has ? (uint32_t)t_base[min(u_begin + batch * 8 + t_unit, n_units)] : 0u;
-    };
-    auto table_hi = [&](uint32_t batch) -> uint32_t {
-        return t_has ? (uint32_t)t_base[min(u_begin + batch * 8 + t_unit + 1, n_units)] : 0u;
-    };
-    uint32_t lo_cur = table_lo(0), hi_cur = table_hi(0), lo_nxt = table_lo(1), hi_nxt = table_hi(1);
-
-    auto stage = [&](uint32_t t, uint32_t batch_now) {
-        const bool ahead = (t >> 3) != batch_now;
-        const uint32_t lo = ahead ? lo_nxt : lo_cur, hi = ahead ? hi_nxt : hi_cur, j = t & 7;
+    // units are staged in order; their table entries arrive one unit ahead (scalar loads)
+    TableWalk<L> table;
+    table.start(prefix, entries, u_begin);
+    auto stage = [&](uint32_t t) {
         uint32_t q_lo[L - 1], q_hi[L - 1];
-#pragma unroll
-        for (int i = 0; i < L - 1; ++i) {
-            q_lo[i] = (uint32_t)__builtin_amdgcn_readlane((int)lo, (int)(j * 8 + i));
-            q_hi[i] = (uint32_t)__builtin_amdgcn_readlane((int)hi, (int)(j * 8 + i));
-        }
+        table.next(q_lo, q_hi);
         StagedUnit<L> S;
         const uint32_t slot = my_slots + (t % kDRing) * dstaged_slot_bytes(L);
         stage_unit<L>(P, u_begin + t, kStagedChunk, q_lo, q_hi, slot, lane, S);
         put_unit<L>(slot + staged_slot_words(L) * 4, lane, S);
     };
-    for (uint32_t t = 0; t < kDRing - 1 && t < total; ++t) stage(t, 0);
+    for (uint32_t t = 0; t < kDRing - 1 && t < total; ++t) stage(t);
 
 #pragma unroll 1
     for (uint32_t t = 0; t < total; ++t) {
-        if ((t & 7) == 0 && t) {
-            lo_cur = lo_nxt, hi_cur = hi_nxt;
-            lo_nxt = table_lo((t >> 3) + 1), hi_nxt = table_hi((t >> 3) + 1);
-        }
-        if (t + kDRing - 1 < total) stage(t + kDRing - 1, t >> 3);
+        if (t + kDRing - 1 < total) stage(t + kDRing - 1);
         // unit t has landed once at most the loads of the units staged after it are outstanding
         const uint32_t after = min(kDRing - 1, total - 1 - t);
         if (after >= 3) dwait_vmcnt<3 * kDma>();

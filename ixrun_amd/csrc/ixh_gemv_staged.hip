@@ -67,33 +67,18 @@ k_gemv_staged(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint
     uint16_t *const queue = reinterpret_cast<uint16_t *>(my_area + kGRing * gstaged_slot_bytes(L));
     uint16_t *const wrow = queue + kStagedQueue;
 
-    // table entries of eight units at a time in registers: lane 8 j + i holds level i of unit j of the batch
-    const uint32_t t_lev = lane & 7, t_unit = lane >> 3;
-    const bool t_has = t_lev < (uint32_t)(L - 1);
-    const int32_t *const t_base = prefix + (size_t)(t_has ? t_lev : 0) * entries;
-    auto table_lo = [&](uint32_t batch) -> uint32_t {
-        return t_has ? (uint32_t)t_base[min(u_begin + batch * 8 + t_unit, n_units)] : 0u;
-    };
-    auto table_hi = [&](uint32_t batch) -> uint32_t {
-        return t_has ? (uint32_t)t_base[min(u_begin + batch * 8 + t_unit + 1, n_units)] : 0u;
-    };
-    uint32_t lo_cur = table_lo(0), hi_cur = table_hi(0), lo_nxt = table_lo(1), hi_nxt = table_hi(1);
-
-    auto stage = [&](uint32_t t, uint32_t batch_now) {
-        const bool ahead = (t >> 3) != batch_now;
-        const uint32_t lo = ahead ? lo_nxt : lo_cur, hi = ahead ? hi_nxt : hi_cur, j = t & 7;
+    // units are staged in order; their table entries arrive one unit ahead (scalar loads)
+    TableWalk<L> table;
+    table.start(prefix, entries, u_begin);
+    auto stage = [&](uint32_t t) {
         uint32_t q_lo[L - 1], q_hi[L - 1];
-#pragma unroll
-        for (int i = 0; i < L - 1; ++i) {
-            q_lo[i] = (uint32_t)__builtin_amdgcn_readlane((int)lo, (int)(j * 8 + i));
-            q_hi[i] = (uint32_t)__builtin_amdgcn_readlane((int)hi, (int)(j * 8 + i));
-        }
+        table.next(q_lo, q_hi);
         StagedUnit<L> S;
         const uint32_t slot = my_slots + (t % kGRing) * gstaged_slot_bytes(L);
         stage_unit<L>(P, u_begin + t, kStagedChunk, q_lo, q_hi, slot, lane, S);
         put_unit<L>(slot + staged_slot_words(L) * 4, lane, S);
     };
-    for (uint32_t t = 0; t < kGRing - 1 && t < total; ++t) stage(t, 0);
+    for (uint32_t t = 0; t < kGRing - 1 && t < total; ++t) stage(t);
 
     float acc[MT];
 #pragma unroll
@@ -114,12 +99,8 @@ k_gemv_staged(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint
     // one unit: x_cur was requested an iteration ago, x_nxt is requested now; the two buffers swap roles every
     // unit (no register is read while a load into it is in flight)
     auto unit = [&](uint32_t t, staged_u32x4 (&x_cur)[MT], staged_u32x4 (&x_nxt)[MT]) {
-        if ((t & 7) == 0 && t) {
-            lo_cur = lo_nxt, hi_cur = hi_nxt;
-            lo_nxt = table_lo((t >> 3) + 1), hi_nxt = table_hi((t >> 3) + 1);
-        }
         load_x(t + 1, x_nxt);
-        if (t + kGRing - 1 < total) stage(t + kGRing - 1, t >> 3);
+        if (t + kGRing - 1 < total) stage(t + kGRing - 1);
         // Issued after x(t), in order: the copies of unit t+2 (one iteration ago), x(t+1), the copies of unit t+3.
         // Unit t's own copies are older than x(t).  Loads return in order, so once at most those remain
         // outstanding both have landed.

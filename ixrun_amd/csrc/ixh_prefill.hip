@@ -46,6 +46,11 @@ __host__ __device__ constexpr uint32_t prefill_lds_bytes(int n_levels) {
     return kPRows * kPWStride * 2u + kPWaves * prefill_wave_bytes(n_levels);
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every vector-memory operation
+// of the wave, which here would be the copies staged ahead for the next rows: they are private to the wave and
+// need not have landed.
+__device__ __forceinline__ void barrier_lds() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     static_assert(N >= 0 && N < 64, "s_waitcnt vmcnt holds 6 bits");
@@ -165,7 +170,7 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
 
     for (uint32_t c = c_begin; c < c_end; ++c) {
         const uint32_t q3 = table_at(c + 3);
-        __syncthreads();  // the previous column's MFMAs are done with the weight tile
+        barrier_lds();  // the previous column's MFMAs are done with the weight tile
         if (c == c_begin) PF_STAMP(2);
         // ---- decode the 64 x 512 weight tile of unit column c: wave w takes rows 8w .. 8w+7 ----
 #pragma unroll 1
@@ -196,7 +201,7 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
             if (c == c_begin) PF_STAMP(3 + j);
         }
         q0 = q1, q1 = q2, q2 = q3;
-        __syncthreads();  // weight tile complete
+        barrier_lds();  // weight tile complete
         if (c == c_begin) PF_STAMP(11);
 
         // ---- eight blocks of 64 k over the decoded tile ----

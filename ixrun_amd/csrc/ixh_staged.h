@@ -126,6 +126,37 @@ __device__ __forceinline__ void stage_unit(const Dev &P, uint32_t u, uint32_t ch
     }
 }
 
+// Rank-table entries of consecutive units, fetched one unit ahead of their use with scalar loads: entry index
+// k holds the level counts before unit k.  Scalar loads are waited for on their own counter (together with LDS
+// operations), so a wave that uses them does not wait for the vector-memory copies it has in flight; a vector
+// load would return behind all of those.
+template <int L>
+struct TableWalk {
+    const int32_t *base;  // table, [L-1][entries]
+    uint32_t entries, at;
+    uint32_t e_cur[L - 1], e_nxt[L - 1];  // entries at `at` and at `at + 1`
+
+    __device__ __forceinline__ void start(const int32_t *table, uint32_t n_entries, uint32_t first) {
+        base = table, entries = n_entries, at = first;
+#pragma unroll
+        for (int i = 0; i < L - 1; ++i) {
+            e_cur[i] = (uint32_t)base[(size_t)i * entries + min(first, entries - 1)];
+            e_nxt[i] = (uint32_t)base[(size_t)i * entries + min(first + 1, entries - 1)];
+        }
+    }
+    // entries of unit `at` and of the unit after it; moves on to unit at + 1 and requests the entry after that
+    __device__ __forceinline__ void next(uint32_t (&q_lo)[L - 1], uint32_t (&q_hi)[L - 1]) {
+        ++at;
+#pragma unroll
+        for (int i = 0; i < L - 1; ++i) {
+            q_lo[i] = e_cur[i];
+            q_hi[i] = e_nxt[i];
+            e_cur[i] = e_nxt[i];
+            e_nxt[i] = (uint32_t)base[(size_t)i * entries + min(at + 1, entries - 1)];
+        }
+    }
+};
+
 // Levels START .. L-1 of up to 64 elements of a staged unit, one per lane (lanes with
 // alive == false take no part).  `space` is the index, in the space of level START, of the
 // first alive lane's element; the alive lanes hold consecutive elements of that space.

@@ -338,3 +338,22 @@ def test_full_size_layers(oracle, dev, shape, m):
     err = check_outputs(bf16_bits(y), y64, f"full {shape} m={m}")
     print(f"{shape} m={m}: rel-L2 {err:.2e}, fractions {[round(c / p['N'], 5) for c in p['counts']]}, "
           f"packed {p['total_bytes']} B")
+
+
+def test_full_size_calibrated_layer(oracle, dev):
+    """5120 x 17408 with the 55/40/5 level mix of real LLM weights: the any-scheme kernels on runs of more than
+    eight table units per wave (GEMV pieces of 8-9 units, decode runs of 11), against the oracle."""
+    from ixrun_amd.engine import StreamingLinear
+
+    out_f, in_f = 5120, 17408
+    w, _ = calibrated_weight(out_f, in_f, seed=0, scale=0.0123046875)
+    p = quantize(w)
+    sl = StreamingLinear(p)
+    shared = torch.empty(p["N"], dtype=torch.bfloat16, device=dev)
+    sl._set_shared_buf(shared)
+    w_bits = oracle.decode_packed_bf16(p)
+    assert np.array_equal(bf16_bits(sl._decode()), w_bits)
+    x = activations(2, in_f, seed=1)
+    y = sl(x.to(dev))
+    y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
+    check_outputs(bf16_bits(y), y64, "full-size calibrated m=2")
