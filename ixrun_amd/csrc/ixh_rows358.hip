@@ -540,17 +540,9 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
                 }
             }
 
-            // window of unit i+1 (or, past the end, a void one) ...
-            uint32_t nw0 = cw0 + 1, nw1 = cw1 + 1, nw2 = cw2, nzrem = 0;
-            if (!(dbg & 2)) {
-                const bool last_cc = cc == C - 1;
-                const uint32_t n_i = min(i + 1, n_units - 1);
-                open_window(n_i, 4 * (last_cc ? step + 1 : step) + quarter, last_cc ? lrn_next : lrn_step,
-                            (last_cc ? valid_next : valid_step) && (i + 1 < n_units), last_cc ? 0 : cc + 1, nw0, nw1,
-                            nw2, nzrem);
-            }
-
-            // ... while the 16 code pairs of unit i go through the pair table and meet the x pairs
+            // The 16 code pairs of unit i go through the pair table and meet the x pairs.  Written first: the pair
+            // table reads and the first reads of the next window then sit in one basic block (the record store
+            // below ends it), so they are issued together and the dot products fill the wait for the window.
             if (!(dbg & 1))
 #pragma unroll
             for (int t = 0; t < 16; ++t) {
@@ -566,6 +558,16 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
                 for (int j = 0; j < MT; ++j)
                     acc[j][t % NA] = __builtin_amdgcn_fdot2_f32_bf16(
                         __builtin_bit_cast(bf16x2, wp), __builtin_bit_cast(bf16x2, xr[cc][j][t]), acc[j][t % NA], false);
+            }
+
+            // window of unit i+1 (or, past the end, a void one)
+            uint32_t nw0 = cw0 + 1, nw1 = cw1 + 1, nw2 = cw2, nzrem = 0;
+            if (!(dbg & 2)) {
+                const bool last_cc = cc == C - 1;
+                const uint32_t n_i = min(i + 1, n_units - 1);
+                open_window(n_i, 4 * (last_cc ? step + 1 : step) + quarter, last_cc ? lrn_next : lrn_step,
+                            (last_cc ? valid_next : valid_step) && (i + 1 < n_units), last_cc ? 0 : cc + 1, nw0, nw1,
+                            nw2, nzrem);
             }
 
             // lanes with more than one element above level 1 (rare): splice on
