@@ -144,6 +144,33 @@ int ixh_gemm(const IxhPacked *packed, const int32_t *prefix, const uint16_t *x, 
 
 size_t ixh_gemm_workspace_bytes(const IxhPacked *packed, int32_t m);
 
+/*
+ * The encoder on the device, in two calls because the stream lengths depend on the data.
+ * Together they replace int8x_quantize (ixrun/quantize.py:41-122, with pack_bits_stream
+ * and pack_bitmap of ixrun/bitpack.py:13-61, :87-89) for a bf16 weight that is already in
+ * device memory, and write byte for byte what that CPU encoder writes; the rank table of
+ * compute_row_prefixes(packed, 512) (ixrun/fused.py:67-78) comes out on the way.
+ *
+ * ixh_encode_scan: w is bf16 [out_f, in_f], contiguous.  Writes
+ *   scale        bf16( max(max|w|, bf16(1e-8)) / 127 )                   (quantize.py:64)
+ *   prefix       the chunk-512 rank table, (n_levels-1) * ixh_prefix_entries(N, 512) entries
+ *   totals       int64 [n_levels], elements per level ("counts"); nullable
+ * The caller reads totals (its own synchronisation), then allocates, for i < n_levels-1,
+ * bitmap i of ceil((N - totals[0] - .. - totals[i-1]) / 32) words and stream i of
+ * ceil(totals[i] * level_bits[i] / 32) words, and totals[n_levels-1] bytes for the last level.
+ *
+ * ixh_encode_pack: dst names those buffers (they are WRITTEN, despite the const of the
+ * struct's fields), the scale and the table written by ixh_encode_scan for the same w.
+ * No write goes past the lengths given in dst.
+ */
+size_t ixh_encode_workspace_bytes(int64_t out_f, int64_t in_f, int32_t n_levels);
+
+int ixh_encode_scan(const uint16_t *w, int64_t out_f, int64_t in_f, int32_t n_levels, const int32_t *level_bits,
+                    uint16_t *scale, int32_t *prefix, int64_t *totals, void *workspace, size_t workspace_bytes,
+                    ixh_stream_t stream);
+
+int ixh_encode_pack(const uint16_t *w, const IxhPacked *dst, const int32_t *prefix, ixh_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -58,6 +58,7 @@ _ENV_GEMV_FLAGS = int(os.environ.get("IXH_GEMV_FLAGS", "0"))
 EXPORTS = (
     "ixh_version", "ixh_last_error", "ixh_prefix_entries", "ixh_prefix_build", "ixh_decode",
     "ixh_gemv", "ixh_gemv_workspace_bytes", "ixh_gemm", "ixh_gemm_workspace_bytes",
+    "ixh_encode_workspace_bytes", "ixh_encode_scan", "ixh_encode_pack",
 )
 
 
@@ -93,6 +94,15 @@ def lib() -> C.CDLL:
         ]
         L.ixh_gemm_workspace_bytes.restype = C.c_size_t
         L.ixh_gemm_workspace_bytes.argtypes = [C.POINTER(IxhPacked), C.c_int32]
+        L.ixh_encode_workspace_bytes.restype = C.c_size_t
+        L.ixh_encode_workspace_bytes.argtypes = [C.c_int64, C.c_int64, C.c_int32]
+        L.ixh_encode_scan.restype = C.c_int
+        L.ixh_encode_scan.argtypes = [
+            C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.POINTER(C.c_int32), C.c_void_p, C.c_void_p, C.c_void_p,
+            C.c_void_p, C.c_size_t, C.c_void_p,
+        ]
+        L.ixh_encode_pack.restype = C.c_int
+        L.ixh_encode_pack.argtypes = [C.c_void_p, C.POINTER(IxhPacked), C.c_void_p, C.c_void_p]
         _lib = L
     return _lib
 
@@ -229,3 +239,41 @@ class DevicePacked:
             workspace.data_ptr() if workspace is not None else None,
             workspace.numel() * workspace.element_size() if workspace is not None else 0,
             current_stream(self.device)))
+
+
+def encode_device(weight: torch.Tensor, level_bits) -> tuple:
+    """Encode a bf16 [out_f, in_f] device tensor with the library's two encoder calls.
+
+    Returns ``(DevicePacked, table512, counts)``: the packed tensors (device), the int32
+    ``[n_levels-1, entries]`` rank table at unit 512 and the per-level element counts (host ints).  One
+    host synchronisation (reading the counts) sits between the two calls.
+    """
+    _require_cuda(weight, "weight")
+    if weight.dtype != torch.bfloat16 or weight.dim() != 2:
+        raise ValueError("the device encoder takes a 2-D bf16 weight")
+    level_bits = tuple(int(b) for b in level_bits)
+    n_levels = len(level_bits)
+    out_f, in_f = weight.shape
+    dev = weight.device
+    L = lib()
+    bits = (C.c_int32 * n_levels)(*level_bits)
+    entries = int(L.ixh_prefix_entries(out_f * in_f, 512))
+    ws_bytes = int(L.ixh_encode_workspace_bytes(out_f, in_f, n_levels))
+    workspace = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=dev)
+    scale = torch.empty(1, dtype=torch.bfloat16, device=dev)
+    table = torch.empty((max(n_levels - 1, 1), max(entries, 1)), dtype=torch.int32, device=dev)
+    totals = torch.empty(max(n_levels, 1), dtype=torch.int64, device=dev)
+    with torch.cuda.device(dev):
+        check(L.ixh_encode_scan(weight.data_ptr(), out_f, in_f, n_levels, bits, scale.data_ptr(), table.data_ptr(),
+                                totals.data_ptr(), workspace.data_ptr(), ws_bytes, current_stream(dev)))
+        counts = [int(c) for c in totals.cpu().tolist()]
+        left = out_f * in_f
+        bitmaps, streams = [], []
+        for i, b in enumerate(level_bits[:-1]):
+            bitmaps.append(torch.empty((left + 31) // 32, dtype=torch.int32, device=dev))
+            streams.append(torch.empty((counts[i] * b + 31) // 32, dtype=torch.int32, device=dev))
+            left -= counts[i]
+        streams.append(torch.empty(counts[-1], dtype=torch.uint8, device=dev))
+        dp = DevicePacked(level_bits, out_f, in_f, bitmaps, streams, scale)
+        check(L.ixh_encode_pack(weight.data_ptr(), C.byref(dp.struct), table.data_ptr(), current_stream(dev)))
+    return dp, table, counts

@@ -225,4 +225,56 @@ int ixh_gemm(const IxhPacked *packed, const int32_t *prefix, const uint16_t *x, 
     return rc;
 }
 
+static int encode_levels_ok(int32_t n_levels, const int32_t *level_bits) {
+    if (n_levels < 2 || n_levels > IXH_MAX_LEVELS) { set_error("n_levels %d not in 2..%d", n_levels, IXH_MAX_LEVELS); return IXH_EINVAL; }
+    if (!level_bits) { set_error("level_bits is NULL"); return IXH_EINVAL; }
+    if (level_bits[n_levels - 1] != 8) { set_error("last level must be 8-bit, got %d", level_bits[n_levels - 1]); return IXH_EINVAL; }
+    for (int i = 0; i < n_levels - 1; ++i) {
+        if (level_bits[i] < 1 || level_bits[i] > 7 || (i > 0 && level_bits[i] < level_bits[i - 1])) {
+            set_error("level_bits[%d] = %d: widths must ascend within 1..7 before the final 8", i, level_bits[i]);
+            return IXH_EINVAL;
+        }
+    }
+    return IXH_OK;
+}
+
+size_t ixh_encode_workspace_bytes(int64_t out_f, int64_t in_f, int32_t n_levels) {
+    if (out_f <= 0 || in_f <= 0 || n_levels < 2 || n_levels > IXH_MAX_LEVELS) return 0;
+    const uint64_t n = (uint64_t)out_f * (uint64_t)in_f;
+    if (n >= (1ull << 31)) return 0;
+    return encode_workspace_bytes(n, n_levels);
+}
+
+int ixh_encode_scan(const uint16_t *w, int64_t out_f, int64_t in_f, int32_t n_levels, const int32_t *level_bits,
+                    uint16_t *scale, int32_t *prefix, int64_t *totals, void *workspace, size_t workspace_bytes,
+                    ixh_stream_t stream) {
+    int rc = encode_levels_ok(n_levels, level_bits);
+    if (rc) return rc;
+    if (out_f <= 0 || in_f <= 0) { set_error("encode: empty weight (the reference's max() raises on it too)"); return IXH_EINVAL; }
+    const uint64_t n = (uint64_t)out_f * (uint64_t)in_f;
+    if (n >= (1ull << 31)) { set_error("out_f * in_f = %llu does not fit the 31-bit rank tables", (unsigned long long)n); return IXH_EINVAL; }
+    if (!w || !scale || !prefix) { set_error("encode: w, scale or prefix is NULL"); return IXH_EINVAL; }
+    const size_t need = encode_workspace_bytes(n, n_levels);
+    if (!workspace || workspace_bytes < need) {
+        set_error("workspace of %zu bytes needed, %zu given", need, workspace ? workspace_bytes : (size_t)0);
+        return IXH_EWORKSPACE;
+    }
+    int bits[IXH_MAX_LEVELS];
+    for (int i = 0; i < n_levels; ++i) bits[i] = level_bits[i];
+    rc = launch_encode_scan(w, (uint32_t)n, n_levels, bits, scale, prefix, totals, workspace, (hipStream_t)stream);
+    if (rc == IXH_ELAUNCH) set_error("encode_scan: launch failed");
+    return rc;
+}
+
+int ixh_encode_pack(const uint16_t *w, const IxhPacked *dst, const int32_t *prefix, ixh_stream_t stream) {
+    Dev d;
+    int rc = to_dev(dst, &d);
+    if (rc) return rc;
+    if (d.n == 0) { set_error("encode: empty weight"); return IXH_EINVAL; }
+    if (!w || !prefix) { set_error("encode: w or prefix is NULL"); return IXH_EINVAL; }
+    rc = launch_encode_pack(w, d, prefix, (hipStream_t)stream);
+    if (rc == IXH_ELAUNCH) set_error("encode_pack: launch failed");
+    return rc;
+}
+
 }  // extern "C"

@@ -46,6 +46,19 @@ __device__ __forceinline__ float dequant(int v, float scale) {
 
 __device__ __forceinline__ int threshold_of(int bits) { return (1 << (bits - 1)) - 1; }
 
+// inclusive sum over the lanes at or below this one (DPP: shifts inside the 16-lane rows, then the two
+// row broadcasts that carry the totals across rows)
+__device__ __forceinline__ uint32_t wave_scan_inclusive(uint32_t v) {
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, true);   // row_shr:1
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, true);   // row_shr:2
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, true);   // row_shr:4
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, true);   // row_shr:8
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1, 3
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2, 3
+    return v;
+}
+
+
 // Decode the 64 consecutive flat elements p0 .. p0+63 (one per lane; lanes with
 // alive == false take no part).  cnt[i] is the number of level-i elements
 // before p0 and is advanced past the group.  Works for any level scheme: lane
@@ -102,6 +115,10 @@ size_t prefill_workspace_bytes(const Dev &P, uint32_t m_rows);
 bool prefill_supports(const Dev &P, const uint16_t *x, int64_t ldx);
 int launch_prefill(const Dev &P, const int32_t *prefix, const uint16_t *x, uint32_t m_rows, int64_t ldx, uint16_t *y,
                    int64_t ldy, float *ws, hipStream_t s);
+size_t encode_workspace_bytes(uint64_t n, int n_levels);
+int launch_encode_scan(const uint16_t *w, uint32_t n, int n_levels, const int *bits, uint16_t *scale, int32_t *table,
+                       int64_t *totals, void *workspace, hipStream_t s);
+int launch_encode_pack(const uint16_t *w, const Dev &P, const int32_t *table, hipStream_t s);
 int launch_fill_u16(uint16_t *dst, uint32_t n, uint16_t value, hipStream_t s);
 void set_error(const char *fmt, ...);
 

@@ -198,18 +198,6 @@ __device__ __forceinline__ int decode64_lds(const Dev &P, const StagedUnit<L> &S
     return decode_from_lds<L, 0>(P, S, p0, alive, cnt);
 }
 
-// inclusive sum over the lanes at or below this one (DPP: shifts inside the 16-lane rows, then the two
-// row broadcasts that carry the totals across rows)
-__device__ __forceinline__ uint32_t wave_scan_inclusive(uint32_t v) {
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, true);   // row_shr:1
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, true);   // row_shr:2
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, true);   // row_shr:4
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, true);   // row_shr:8
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1, 3
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2, 3
-    return v;
-}
-
 typedef float staged_f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 staged_bf16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t staged_u32x4 __attribute__((ext_vector_type(4)));

@@ -64,7 +64,8 @@ class StreamingLinear(nn.Module):
         # rank tables: the kernels' own (unit = 512 where rows allow it) and
         # the two the reference exposes
         self._unit = pick_unit(self.in_features)
-        self.register_buffer("_table", self._dp.prefix_build(self._unit))
+        ready = packed.get("table512") if self._unit == 512 else None  # left by the device encoder
+        self.register_buffer("_table", ready.cuda() if ready is not None else self._dp.prefix_build(self._unit))
         if self.N % TRITON_BLOCK == 0 and TRITON_BLOCK % self._unit == 0:
             blk_table = self._table[:, :: TRITON_BLOCK // self._unit][:, : self.N // TRITON_BLOCK]
         else:

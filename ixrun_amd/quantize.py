@@ -20,7 +20,7 @@ import torch
 from .bitpack import pack_bits_stream, pack_bitmap, unpack_bits_stream
 from .config import BIT_TO_THRESHOLD, DEFAULT_LEVELS
 
-__all__ = ["int8x_quantize", "compute_positions", "decode_to_weight", "DEFAULT_LEVELS"]
+__all__ = ["int8x_quantize", "int8x_quantize_device", "compute_positions", "decode_to_weight", "DEFAULT_LEVELS"]
 
 
 def _level_ids(abs_v: torch.Tensor, level_bits: tuple) -> torch.Tensor:
@@ -88,6 +88,48 @@ def int8x_quantize(weight: torch.Tensor, level_bits: tuple = DEFAULT_LEVELS) -> 
         "total_bytes": total,
         "bits_per_weight": (total * 8) / n,
         "compression_vs_bf16": (n * 2) / total,
+    }
+
+
+@torch.no_grad()
+def int8x_quantize_device(weight: torch.Tensor, level_bits: tuple = DEFAULT_LEVELS) -> dict:
+    """``int8x_quantize`` for a bf16 weight that lives on the GPU, done by the library's encoder kernels.
+
+    The dictionary has the reference's keys (``ixrun/quantize.py:110-122``) with the same bytes in every
+    tensor as the CPU writer produces for this weight, but the tensors stay on the weight's device.  Two
+    extra keys carry what the encoder computes on the way and the modules would otherwise rebuild:
+    ``table512`` (the rank table at unit 512) and ``device_packed`` (the library's view of the tensors).
+    There is no CPU path behind this function: a CPU tensor or a missing library raises.
+    """
+    from ._lib import encode_device
+
+    level_bits = tuple(sorted(level_bits))
+    if level_bits[-1] != 8:
+        raise ValueError("last level must be 8-bit to cover the full int8 range")
+    out_f, in_f = weight.shape
+    n = out_f * in_f
+    if n == 0:
+        raise RuntimeError("max(): cannot quantize an empty weight")
+    dp, table, counts = encode_device(weight.detach().contiguous(), level_bits)
+    n_lv = len(level_bits)
+    bitmaps, streams = dp.tensors[: n_lv - 1], dp.tensors[n_lv - 1 : 2 * n_lv - 1]
+    total = 2 + streams[-1].numel()
+    total += 4 * sum(s.numel() for s in streams[:-1])
+    total += 4 * sum(bm.numel() for bm in bitmaps)
+    return {
+        "level_bits": level_bits,
+        "out_f": out_f,
+        "in_f": in_f,
+        "N": n,
+        "scale": dp.tensors[-1].reshape(()),
+        "bitmaps": list(bitmaps),
+        "streams": list(streams),
+        "counts": counts,
+        "total_bytes": total,
+        "bits_per_weight": (total * 8) / n,
+        "compression_vs_bf16": (n * 2) / total,
+        "table512": table,
+        "device_packed": dp,
     }
 
 

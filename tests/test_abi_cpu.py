@@ -83,6 +83,28 @@ def test_malformed_gemv_arguments():
         _lib.check(-1)
 
 
+def test_malformed_encode_arguments():
+    lib = _lib.lib()
+    bits = (C.c_int32 * 3)(3, 5, 8)
+    need = lib.ixh_encode_workspace_bytes(4, 1024, 3)
+    assert need >= 4096 + 2 * 4  # the partial maxima and one tile sum per table row
+    assert lib.ixh_encode_workspace_bytes(0, 1024, 3) == 0 and lib.ixh_encode_workspace_bytes(4, 1024, 9) == 0
+    scan = lambda out_f=4, in_f=1024, nl=3, lb=bits, w=0x1000, sc=0x1000, tab=0x1000, ws=0x1000, wsb=need: \
+        lib.ixh_encode_scan(w, out_f, in_f, nl, lb, sc, tab, None, ws, wsb, None)
+    assert scan(nl=1) == -1 and "n_levels" in lib.ixh_last_error().decode()
+    assert scan(lb=(C.c_int32 * 3)(3, 5, 7)) == -1 and "last level" in lib.ixh_last_error().decode()
+    assert scan(lb=(C.c_int32 * 3)(5, 3, 8)) == -1 and "ascend" in lib.ixh_last_error().decode()
+    assert scan(out_f=0) == -1 and "empty" in lib.ixh_last_error().decode()
+    assert scan(out_f=1 << 20, in_f=1 << 12) == -1 and "31-bit" in lib.ixh_last_error().decode()
+    assert scan(w=None) == -1 and scan(sc=None) == -1 and scan(tab=None) == -1
+    assert scan(wsb=need - 1) == -4 and "workspace" in lib.ixh_last_error().decode()
+    s = _packed(out_f=4, in_f=1024, bm0_words=128)
+    assert lib.ixh_encode_pack(None, C.byref(s), 0x1000, None) == -1
+    assert lib.ixh_encode_pack(0x1000, C.byref(s), None, None) == -1
+    s.bitmap_words[0] = 3
+    assert lib.ixh_encode_pack(0x1000, C.byref(s), 0x1000, None) == -1 and "bitmap 0" in lib.ixh_last_error().decode()
+
+
 def test_device_packed_refuses_cpu_tensors():
     from ixrun_amd.quantize import int8x_quantize
 
