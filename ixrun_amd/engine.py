@@ -23,7 +23,7 @@ from . import _lib
 from .config import TRITON_BLOCK
 from .fused import FUSED_TILE, _pick_split, pick_unit, shared_workspace
 from .linear import _set_parent_child, iter_quantizable_linears
-from .quantize import int8x_quantize
+from .quantize import int8x_quantize, portable_packed, quantize_for_deploy
 
 __all__ = ["Int8XEngine", "StreamingLinear", "GraphLinear", "ResourceScheduler"]
 
@@ -286,11 +286,12 @@ class Int8XEngine:
             layer_data = []
             for name, mod in targets:
                 bias = mod.bias.data if mod.bias is not None else None
-                layer_data.append((name, int8x_quantize(mod.weight.data, level_bits), bias))
+                layer_data.append((name, quantize_for_deploy(mod.weight.data, level_bits), bias))
             if cache_path is not None:
                 if verbose:
                     print(f"[engine][cache] saving packed weights to {cache_path}", flush=True)
-                torch.save({"level_bits": tuple(level_bits), "layers": layer_data}, cache_path)
+                torch.save({"level_bits": tuple(level_bits),
+                            "layers": [(n, portable_packed(p), b) for n, p, b in layer_data]}, cache_path)
 
         total_bytes = max_n = 0
         layers = []
@@ -325,7 +326,7 @@ class Int8XEngine:
         total_bytes = 0
         specs = []
         for name, mod in targets:
-            packed = int8x_quantize(mod.weight.data, level_bits)
+            packed = quantize_for_deploy(mod.weight.data, level_bits)
             bias = mod.bias.data if mod.bias is not None else None
             sl = StreamingLinear(packed, bias=bias)
             buf = torch.empty(packed["N"], dtype=torch.bfloat16, device="cuda")

@@ -11,7 +11,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .config import MIN_LINEAR_ELEMS, SKIP_PATTERNS
-from .quantize import int8x_quantize
+from .quantize import int8x_quantize, portable_packed, quantize_for_deploy
 from .triton_kernels import decode_weight_scatter, decode_weight_triton
 
 __all__ = ["Int8XLinear", "deploy_model", "iter_quantizable_linears"]
@@ -83,9 +83,12 @@ def deploy_model(model: nn.Module, level_bits=(3, 5, 8), cache: str = "full", us
     n_layers = total_bytes = n_elems = 0
     counts = [0] * len(tuple(level_bits))
     for name, mod in list(iter_quantizable_linears(model)):
-        packed = int8x_quantize(mod.weight.data, level_bits)
+        packed = quantize_for_deploy(mod.weight.data, level_bits) if use_triton else int8x_quantize(mod.weight.data, level_bits)
         bias = mod.bias.data if mod.bias is not None else None
-        _set_parent_child(model, name, Int8XLinear(packed, bias=bias, cache=cache, use_triton=use_triton))
+        layer = Int8XLinear(packed, bias=bias, cache=cache, use_triton=use_triton)
+        if cache == "full":  # the decoded weight is what stays on the GPU; the packed form goes back to the host
+            layer.packed = packed = portable_packed(packed)
+        _set_parent_child(model, name, layer)
         n_layers += 1
         total_bytes += packed["total_bytes"]
         n_elems += packed["N"]

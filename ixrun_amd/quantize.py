@@ -20,7 +20,7 @@ import torch
 from .bitpack import pack_bits_stream, pack_bitmap, unpack_bits_stream
 from .config import BIT_TO_THRESHOLD, DEFAULT_LEVELS
 
-__all__ = ["int8x_quantize", "int8x_quantize_device", "compute_positions", "decode_to_weight", "DEFAULT_LEVELS"]
+__all__ = ["int8x_quantize", "int8x_quantize_device", "quantize_for_deploy", "portable_packed", "compute_positions", "decode_to_weight", "DEFAULT_LEVELS"]
 
 
 def _level_ids(abs_v: torch.Tensor, level_bits: tuple) -> torch.Tensor:
@@ -131,6 +131,30 @@ def int8x_quantize_device(weight: torch.Tensor, level_bits: tuple = DEFAULT_LEVE
         "table512": table,
         "device_packed": dp,
     }
+
+
+REFERENCE_KEYS = ("level_bits", "out_f", "in_f", "N", "scale", "bitmaps", "streams", "counts", "total_bytes",
+                  "bits_per_weight", "compression_vs_bf16")
+
+
+def portable_packed(packed: dict) -> dict:
+    """The dictionary with the reference's keys only and every tensor on the CPU: what ``int8x_quantize``
+    returns and what the packed-cache file holds (``ixrun/quantize.py:110-122``, ``ixrun/engine.py:383``)."""
+    out = {k: packed[k] for k in REFERENCE_KEYS}
+    out["scale"] = packed["scale"].detach().cpu().reshape(())
+    out["bitmaps"] = [t.detach().cpu() for t in packed["bitmaps"]]
+    out["streams"] = [t.detach().cpu() for t in packed["streams"]]
+    return out
+
+
+@torch.no_grad()
+def quantize_for_deploy(weight: torch.Tensor, level_bits: tuple = DEFAULT_LEVELS) -> dict:
+    """What the deploy paths call per layer: with a GPU in the process a bf16 weight is moved there (if it is
+    not there already) and encoded by the device kernels, so the packed tensors are born where the modules
+    keep them; any other weight goes through the CPU writer.  Same bytes either way."""
+    if torch.cuda.is_available() and weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.numel() > 0:
+        return int8x_quantize_device(weight.cuda(), level_bits)
+    return int8x_quantize(weight, level_bits)
 
 
 @torch.no_grad()

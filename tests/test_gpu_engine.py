@@ -63,6 +63,15 @@ def test_deploy_modes(tmp_path, rows):
     assert stats["mode"] == "streaming" and stats["n_layers"] == 2 and isinstance(streaming.proj_in, StreamingLinear)
     streaming = streaming.cuda()
     assert close(streaming(x), want)
+    # the file holds what the CPU writer produces for these weights (the layers were encoded on the device)
+    from ixrun_amd.quantize import int8x_quantize
+
+    blob = torch.load(cache, map_location="cpu", weights_only=True)
+    for name, packed, _ in blob["layers"]:
+        ref = int8x_quantize(getattr(base, name).weight.data, (3, 5, 8))
+        assert list(packed.keys()) == list(ref.keys()) and packed["counts"] == ref["counts"]
+        assert torch.equal(packed["scale"], ref["scale"])
+        assert all(torch.equal(a, b) for a, b in zip(packed["bitmaps"] + packed["streams"], ref["bitmaps"] + ref["streams"]))
     again = copy.deepcopy(base)
     Int8XEngine._deploy_streaming(again, (3, 5, 8), verbose=False, cache_path=cache)  # now read from the file
     assert torch.equal(again.cuda()(x), streaming(x))
