@@ -250,6 +250,13 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the row sums have taken the additions
 }
 
+// s_setprio takes an immediate
+__device__ __forceinline__ void set_wave_priority(uint32_t p) {
+    if (p == 0) __builtin_amdgcn_s_setprio(0);
+    else if (p == 1) __builtin_amdgcn_s_setprio(1);
+    else __builtin_amdgcn_s_setprio(2);
+}
+
 template <int MT, int C>
 __global__ void __launch_bounds__(kRMaxWaves * kWave)
 k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t quads_per_wg_arg, uint32_t flags,
@@ -518,6 +525,10 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     constexpr int NA = MT == 1 ? 4 : (MT == 2 ? 2 : 1);  // independent accumulators per x row
 
     for (uint32_t step = 0; step < n_steps; ++step) {
+        // The waves that share a SIMD take turns at the issue priority, one row quad each: without this the
+        // oldest wave is served first throughout, finishes early and leaves the others to end the kernel with
+        // nothing to hide their waits behind.
+        if (!(dbg & 512)) set_wave_priority(((wave >> 2) + step) % 3u);
         float acc[MT][NA];
 #pragma unroll
         for (int j = 0; j < MT; ++j)
