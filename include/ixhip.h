@@ -105,6 +105,21 @@ int ixh_decode(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, in
                uint16_t *out_bf16, ixh_stream_t stream);
 
 /*
+ * Full decode of the group-scale sibling format ("ixgs"): the same (3,5,8) nested-bitmap
+ * streams, but every run of group_size consecutive elements has its own fp16 scale:
+ *   out_bf16[p] = bf16( f32(v[p]) * f32(group_scales[p / group_size]) ).
+ * Replaces _ixgs_decode_kernel / decode_weight_triton (ixgs/kernels.py:30-105, :121-142)
+ * and decode_weight_scatter (ixgs/quantize.py:113-151); the reference's per-element rank
+ * tensors (ixgs/kernels.py:107-118, three int32 per weight) are replaced by the same
+ * chunked rank table as ixh_decode.  packed->scale is not read and may be NULL; the codes
+ * are offset by 3 / 15 / 127 exactly as in the per-tensor format, so values up to +128
+ * (ixgs/quantize.py:63) decode correctly.  Fastest with chunk = 512, group_size a multiple
+ * of 8 and a 16-byte aligned out_bf16.
+ */
+int ixh_decode_gs(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, const uint16_t *group_scales,
+                  int64_t group_size, uint16_t *out_bf16, ixh_stream_t stream);
+
+/*
  * Fused decode + GEMV / skinny GEMM:
  *   y[m, r] = bf16( sum_k f32(x[m, k]) * f32(bf16(f32(v[r, k]) * f32(scale))) ),
  * fp32 accumulation, m < M <= 16; x is bf16 [M, ldx], y is bf16 [M, ldy].

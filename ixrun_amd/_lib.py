@@ -58,7 +58,7 @@ _ENV_GEMV_FLAGS = int(os.environ.get("IXH_GEMV_FLAGS", "0"))
 EXPORTS = (
     "ixh_version", "ixh_last_error", "ixh_prefix_entries", "ixh_prefix_build", "ixh_decode",
     "ixh_gemv", "ixh_gemv_workspace_bytes", "ixh_gemm", "ixh_gemm_workspace_bytes",
-    "ixh_encode_workspace_bytes", "ixh_encode_scan", "ixh_encode_pack",
+    "ixh_encode_workspace_bytes", "ixh_encode_scan", "ixh_encode_pack", "ixh_decode_gs",
 )
 
 
@@ -80,6 +80,9 @@ def lib() -> C.CDLL:
         L.ixh_prefix_build.argtypes = [C.POINTER(IxhPacked), C.c_int64, C.c_void_p, C.c_void_p]
         L.ixh_decode.restype = C.c_int
         L.ixh_decode.argtypes = [C.POINTER(IxhPacked), C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.ixh_decode_gs.restype = C.c_int
+        L.ixh_decode_gs.argtypes = [C.POINTER(IxhPacked), C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p,
+                                    C.c_void_p]
         L.ixh_gemv.restype = C.c_int
         L.ixh_gemv.argtypes = [
             C.POINTER(IxhPacked), C.c_void_p, C.c_int64, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p,
@@ -135,12 +138,13 @@ class DevicePacked:
             raise ValueError("need one bitmap per level but the last and one stream per level")
         self.level_bits, self.out_f, self.in_f = level_bits, int(out_f), int(in_f)
         self.N = self.out_f * self.in_f
-        self.tensors = list(bitmaps) + list(streams) + [scale]
+        # scale None: the group-scale format, whose scales are an argument of its decode call
+        self.tensors = list(bitmaps) + list(streams) + ([scale] if scale is not None else [])
         for i, t in enumerate(self.tensors):
             _require_cuda(t, f"packed tensor {i}")
-        if scale.dtype != torch.bfloat16 or scale.numel() != 1:
+        if scale is not None and (scale.dtype != torch.bfloat16 or scale.numel() != 1):
             raise ValueError("scale must be a one-element bf16 tensor")
-        self.device = scale.device
+        self.device = self.tensors[0].device
         s = IxhPacked()
         s.n_levels = n_levels
         for i, b in enumerate(level_bits):
@@ -159,7 +163,7 @@ class DevicePacked:
             raise ValueError("the last stream must be torch.uint8")
         s.last = last.data_ptr() if last.numel() else None
         s.last_bytes = last.numel()
-        s.scale = scale.data_ptr()
+        s.scale = scale.data_ptr() if scale is not None else None
         self.struct = s
 
     @classmethod
@@ -193,6 +197,19 @@ class DevicePacked:
             C.byref(self.struct), table.data_ptr(), int(chunk),
             out_i8.data_ptr() if out_i8 is not None else None,
             out_bf16.data_ptr() if out_bf16 is not None else None, current_stream(self.device)))
+
+    def decode_gs(self, table: torch.Tensor, chunk: int, group_scales: torch.Tensor, group_size: int,
+                  out_bf16: torch.Tensor) -> None:
+        """Decode with one fp16 scale per `group_size` consecutive elements (the group-scale format)."""
+        _require_cuda(group_scales, "group_scales")
+        _require_cuda(out_bf16, "decode output")
+        n_groups = -(-self.N // int(group_size)) if int(group_size) > 0 else 0  # the library rejects sizes <= 0
+        if group_scales.dtype != torch.float16 or group_scales.numel() < n_groups:
+            raise ValueError(f"group_scales must be fp16 with at least {n_groups} elements")
+        if out_bf16.dtype != torch.bfloat16 or out_bf16.numel() < self.N:
+            raise ValueError(f"decode output must be bf16 with at least {self.N} elements")
+        check(lib().ixh_decode_gs(C.byref(self.struct), table.data_ptr(), int(chunk), group_scales.data_ptr(),
+                                  int(group_size), out_bf16.data_ptr(), current_stream(self.device)))
 
     def gemv_workspace_bytes(self, chunk: int, m: int, flags: int = 0) -> int:
         return int(lib().ixh_gemv_workspace_bytes(C.byref(self.struct), int(chunk), int(m), int(flags)))

@@ -21,7 +21,7 @@ void set_error(const char *fmt, ...) {
 }
 
 // Validate an IxhPacked and turn it into the kernel-argument form.
-static int to_dev(const IxhPacked *pk, Dev *out) {
+static int to_dev(const IxhPacked *pk, Dev *out, bool need_scale = true) {
     if (!pk) { set_error("packed is NULL"); return IXH_EINVAL; }
     const int L = pk->n_levels;
     if (L < 2 || L > IXH_MAX_LEVELS) { set_error("n_levels %d not in 2..%d", L, IXH_MAX_LEVELS); return IXH_EINVAL; }
@@ -36,7 +36,7 @@ static int to_dev(const IxhPacked *pk, Dev *out) {
     if (pk->out_f < 0 || pk->in_f < 0) { set_error("negative shape"); return IXH_EINVAL; }
     const uint64_t n = (uint64_t)pk->out_f * (uint64_t)pk->in_f;
     if (n >= (1ull << 31)) { set_error("out_f * in_f = %llu does not fit the 31-bit rank tables", (unsigned long long)n); return IXH_EINVAL; }
-    if (n != 0 && !pk->scale) { set_error("scale is NULL"); return IXH_EINVAL; }
+    if (n != 0 && need_scale && !pk->scale) { set_error("scale is NULL"); return IXH_EINVAL; }
     Dev d;
     memset(&d, 0, sizeof(d));
     d.n_levels = L;
@@ -91,7 +91,7 @@ int64_t ixh_prefix_entries(int64_t n, int64_t chunk) {
 
 int ixh_prefix_build(const IxhPacked *packed, int64_t chunk, int32_t *prefix, ixh_stream_t stream) {
     Dev d;
-    int rc = to_dev(packed, &d);
+    int rc = to_dev(packed, &d, false);  // the table is counted from the bitmaps alone
     if (rc) return rc;
     if (chunk <= 0 || chunk >= (1ll << 31)) { set_error("chunk %lld out of range", (long long)chunk); return IXH_EINVAL; }
     if (!prefix) { set_error("prefix is NULL"); return IXH_EINVAL; }
@@ -100,22 +100,35 @@ int ixh_prefix_build(const IxhPacked *packed, int64_t chunk, int32_t *prefix, ix
     return rc;
 }
 
-int ixh_decode(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, int8_t *out_i8,
-               uint16_t *out_bf16, ixh_stream_t stream) {
+static int decode_any(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, int8_t *out_i8, uint16_t *out_bf16,
+                      GroupScales gs, ixh_stream_t stream) {
     Dev d;
-    int rc = to_dev(packed, &d);
+    int rc = to_dev(packed, &d, gs.fp16 == nullptr);
     if (rc) return rc;
     if (chunk <= 0 || chunk >= (1ll << 31)) { set_error("chunk %lld out of range", (long long)chunk); return IXH_EINVAL; }
     if (d.n == 0) return IXH_OK;
     if (!prefix) { set_error("prefix is NULL"); return IXH_EINVAL; }
     if (!out_i8 && !out_bf16) { set_error("both outputs are NULL"); return IXH_EINVAL; }
     static const bool no_staged = getenv("IXH_DECODE_GENERIC") != nullptr;  // measurement switch
-    if (!no_staged && decode_staged_supports(d, (uint32_t)chunk, out_i8, out_bf16))
-        rc = launch_decode_staged(d, prefix, out_bf16, (hipStream_t)stream);
+    if (!no_staged && decode_staged_supports(d, (uint32_t)chunk, out_i8, out_bf16, gs))
+        rc = launch_decode_staged(d, prefix, out_bf16, gs, (hipStream_t)stream);
     else
-        rc = launch_decode(d, prefix, (uint32_t)chunk, out_i8, out_bf16, (hipStream_t)stream);
+        rc = launch_decode(d, prefix, (uint32_t)chunk, out_i8, out_bf16, gs, (hipStream_t)stream);
     if (rc == IXH_ELAUNCH) set_error("decode: launch failed");
     return rc;
+}
+
+int ixh_decode(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, int8_t *out_i8,
+               uint16_t *out_bf16, ixh_stream_t stream) {
+    return decode_any(packed, prefix, chunk, out_i8, out_bf16, GroupScales{nullptr, 0}, stream);
+}
+
+int ixh_decode_gs(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, const uint16_t *group_scales,
+                  int64_t group_size, uint16_t *out_bf16, ixh_stream_t stream) {
+    if (!group_scales) { set_error("group_scales is NULL"); return IXH_EINVAL; }
+    if (group_size <= 0 || group_size >= (1ll << 31)) { set_error("group_size %lld out of range", (long long)group_size); return IXH_EINVAL; }
+    if (!out_bf16) { set_error("out_bf16 is NULL"); return IXH_EINVAL; }
+    return decode_any(packed, prefix, chunk, nullptr, out_bf16, GroupScales{group_scales, (uint32_t)group_size}, stream);
 }
 
 static int gemv_checks(const Dev &d, int64_t chunk, int32_t m) {

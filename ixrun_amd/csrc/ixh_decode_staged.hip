@@ -26,7 +26,7 @@ __device__ __forceinline__ void dwait_vmcnt() {
 template <int L>
 __global__ void __launch_bounds__(kWave *kDWaves)
 k_decode_staged(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, uint32_t units_per_wave,
-                uint16_t *__restrict__ out) {
+                uint16_t *__restrict__ out, GroupScales gs) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int kDma = staged_dma_count(L);
     static_assert((kDRing - 1) * kDma < 64, "ring too deep for the wait counter");
@@ -36,7 +36,7 @@ k_decode_staged(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, uin
     if (u_begin >= n_units) return;  // no barriers in this kernel
     const uint32_t total = min(units_per_wave, n_units - u_begin);
     const uint32_t entries = n_units + 1;
-    const float scale = bf16_bits_to_f32(*P.scale);
+    const float scale = gs.fp16 ? 0.0f : bf16_bits_to_f32(*P.scale);
 
     uint8_t *const my_area = smem + wave * dstaged_wave_bytes(L);
     const uint32_t my_slots = (uint32_t)(uintptr_t)(lds_ptr_t)my_area;
@@ -71,7 +71,8 @@ k_decode_staged(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, uin
         const uint32_t slot = my_slots + (t % kDRing) * dstaged_slot_bytes(L);
         StagedUnit<L> S;
         get_unit<L>(slot + staged_slot_words(L) * 4, S);
-        decode_unit_lds<L>(P, S, p_begin, n_el, scale, row, queue, lane);
+        decode_unit_lds<L>(P, S, p_begin, n_el,
+                           [&](uint32_t e) { return scale_of(gs, scale, min(p_begin + e, P.n - 1)); }, row, queue, lane);
         const staged_u32x4 v = *reinterpret_cast<const staged_u32x4 *>(row + 8 * lane);
         if (8 * lane + 8 <= n_el) {
             *reinterpret_cast<staged_u32x4 *>(out + (size_t)p_begin + 8 * lane) = v;
@@ -81,32 +82,33 @@ k_decode_staged(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, uin
     }
 }
 
-bool decode_staged_supports(const Dev &P, uint32_t chunk, const int8_t *o8, const uint16_t *o16) {
+bool decode_staged_supports(const Dev &P, uint32_t chunk, const int8_t *o8, const uint16_t *o16, GroupScales gs) {
+    if (gs.fp16 && gs.group % 8u != 0) return false;  // a lane's eight elements share one scale
     return chunk == kStagedChunk && !o8 && o16 && ((uintptr_t)o16 & 15u) == 0 && ((uintptr_t)P.last & 3u) == 0 &&
            P.n_levels >= 2 && P.n_levels <= IXH_MAX_LEVELS && P.n >= kStagedChunk;
 }
 
 template <int L>
-static int decode_staged_launch(const Dev &P, const int32_t *prefix, uint16_t *o16, hipStream_t s) {
+static int decode_staged_launch(const Dev &P, const int32_t *prefix, uint16_t *o16, GroupScales gs, hipStream_t s) {
     const uint32_t n_units = (uint32_t)(((uint64_t)P.n + kStagedChunk - 1) / kStagedChunk);
     // enough waves to fill the chip a few times over, each with a run long enough to keep its ring busy
     const uint32_t units_per_wave = max(8u, (n_units + 16383u) / 16384u);
     const uint32_t n_waves = (n_units + units_per_wave - 1) / units_per_wave;
     const uint32_t blocks = (n_waves + kDWaves - 1) / kDWaves;
     hipLaunchKernelGGL(k_decode_staged<L>, dim3(blocks), dim3(kWave * kDWaves), kDWaves * dstaged_wave_bytes(L), s, P,
-                       prefix, n_units, units_per_wave, o16);
+                       prefix, n_units, units_per_wave, o16, gs);
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }
 
-int launch_decode_staged(const Dev &P, const int32_t *prefix, uint16_t *o16, hipStream_t s) {
+int launch_decode_staged(const Dev &P, const int32_t *prefix, uint16_t *o16, GroupScales gs, hipStream_t s) {
     switch (P.n_levels) {
-        case 2: return decode_staged_launch<2>(P, prefix, o16, s);
-        case 3: return decode_staged_launch<3>(P, prefix, o16, s);
-        case 4: return decode_staged_launch<4>(P, prefix, o16, s);
-        case 5: return decode_staged_launch<5>(P, prefix, o16, s);
-        case 6: return decode_staged_launch<6>(P, prefix, o16, s);
-        case 7: return decode_staged_launch<7>(P, prefix, o16, s);
-        case 8: return decode_staged_launch<8>(P, prefix, o16, s);
+        case 2: return decode_staged_launch<2>(P, prefix, o16, gs, s);
+        case 3: return decode_staged_launch<3>(P, prefix, o16, gs, s);
+        case 4: return decode_staged_launch<4>(P, prefix, o16, gs, s);
+        case 5: return decode_staged_launch<5>(P, prefix, o16, gs, s);
+        case 6: return decode_staged_launch<6>(P, prefix, o16, gs, s);
+        case 7: return decode_staged_launch<7>(P, prefix, o16, gs, s);
+        case 8: return decode_staged_launch<8>(P, prefix, o16, gs, s);
         default: return IXH_EUNSUPPORTED;
     }
 }

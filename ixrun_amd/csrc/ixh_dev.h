@@ -44,6 +44,19 @@ __device__ __forceinline__ float dequant(int v, float scale) {
     return bf16_bits_to_f32(f32_to_bf16_bits((float)v * scale));
 }
 
+// Where the dequantisation scale of an element comes from: the tensor's bf16 scale, or, for the group-scale
+// sibling format (ixgs/quantize.py:56-61), the fp16 scale of the element's group of `group` consecutive elements.
+struct GroupScales {
+    const uint16_t *fp16;  // nullptr: per-tensor scale
+    uint32_t group;
+};
+
+__device__ __forceinline__ float fp16_bits_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+
+__device__ __forceinline__ float scale_of(const GroupScales &g, float tensor_scale, uint32_t p) {
+    return g.fp16 ? fp16_bits_to_f32(g.fp16[p / g.group]) : tensor_scale;
+}
+
 __device__ __forceinline__ int threshold_of(int bits) { return (1 << (bits - 1)) - 1; }
 
 // inclusive sum over the lanes at or below this one (DPP: shifts inside the 16-lane rows, then the two
@@ -102,15 +115,16 @@ __device__ __forceinline__ int decode64(const Dev &P, uint32_t p0, bool alive, u
 
 // ---- host-side launchers (one per translation unit of kernels) ----
 int launch_prefix_build(const Dev &P, uint32_t chunk, int32_t *prefix, hipStream_t s);
-int launch_decode(const Dev &P, const int32_t *prefix, uint32_t chunk, int8_t *o8, uint16_t *o16, hipStream_t s);
+int launch_decode(const Dev &P, const int32_t *prefix, uint32_t chunk, int8_t *o8, uint16_t *o16, GroupScales gs,
+                  hipStream_t s);
 int launch_gemv_generic(const Dev &P, const int32_t *prefix, uint32_t chunk, const uint16_t *x, int m,
                         int64_t ldx, uint16_t *y, int64_t ldy, float *y32, float *ws, bool atomic,
                         hipStream_t s);
 bool gemv_staged_supports(const Dev &P, uint32_t chunk, const uint16_t *x, int64_t ldx);
 int launch_gemv_staged(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
                        int64_t ldy, float *y32, float *ws, bool atomic, hipStream_t s);
-bool decode_staged_supports(const Dev &P, uint32_t chunk, const int8_t *o8, const uint16_t *o16);
-int launch_decode_staged(const Dev &P, const int32_t *prefix, uint16_t *o16, hipStream_t s);
+bool decode_staged_supports(const Dev &P, uint32_t chunk, const int8_t *o8, const uint16_t *o16, GroupScales gs);
+int launch_decode_staged(const Dev &P, const int32_t *prefix, uint16_t *o16, GroupScales gs, hipStream_t s);
 size_t prefill_workspace_bytes(const Dev &P, uint32_t m_rows);
 bool prefill_supports(const Dev &P, const uint16_t *x, int64_t ldx);
 int launch_prefill(const Dev &P, const int32_t *prefix, const uint16_t *x, uint32_t m_rows, int64_t ldx, uint16_t *y,

@@ -114,7 +114,7 @@ k_gemv_staged(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint
         const uint32_t slot = my_slots + (t % kGRing) * gstaged_slot_bytes(L);
         StagedUnit<L> S;
         get_unit<L>(slot + staged_slot_words(L) * 4, S);
-        decode_unit_lds<L>(P, S, u * kStagedChunk, kStagedChunk, scale, wrow, queue, lane);
+        decode_unit_lds<L>(P, S, u * kStagedChunk, kStagedChunk, [scale](uint32_t) { return scale; }, wrow, queue, lane);
         const staged_u32x4 w = *reinterpret_cast<const staged_u32x4 *>(wrow + 8 * lane);
         const uint32_t wk[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll

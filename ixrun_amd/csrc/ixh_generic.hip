@@ -100,7 +100,7 @@ int launch_fill_u16(uint16_t *dst, uint32_t n, uint16_t value, hipStream_t s) {
 template <int L>
 __global__ void __launch_bounds__(kWave *kWavesPerBlock)
 k_decode(Dev P, const int32_t *__restrict__ prefix, uint32_t chunk, uint32_t n_units,
-         int8_t *__restrict__ o8, uint16_t *__restrict__ o16) {
+         int8_t *__restrict__ o8, uint16_t *__restrict__ o16, GroupScales gs) {
     const uint32_t u = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
     if (u >= n_units) return;
     const uint32_t lane = threadIdx.x & 63;
@@ -108,7 +108,7 @@ k_decode(Dev P, const int32_t *__restrict__ prefix, uint32_t chunk, uint32_t n_u
     uint32_t cnt[L - 1];
 #pragma unroll
     for (int i = 0; i < L - 1; ++i) cnt[i] = (uint32_t)prefix[(size_t)i * entries + u];
-    const float scale = bf16_bits_to_f32(*P.scale);
+    const float scale = gs.fp16 ? 0.0f : bf16_bits_to_f32(*P.scale);
     const uint64_t e0 = (uint64_t)u * chunk;
     const uint32_t p_begin = (uint32_t)e0;
     const uint32_t p_end = (uint32_t)min(e0 + chunk, (uint64_t)P.n);
@@ -117,31 +117,31 @@ k_decode(Dev P, const int32_t *__restrict__ prefix, uint32_t chunk, uint32_t n_u
         const int v = decode64<L>(P, p0, alive, cnt);
         if (alive) {
             if (o8) o8[p0 + lane] = (int8_t)v;
-            if (o16) o16[p0 + lane] = (uint16_t)f32_to_bf16_bits((float)v * scale);
+            if (o16) o16[p0 + lane] = (uint16_t)f32_to_bf16_bits((float)v * scale_of(gs, scale, p0 + lane));
         }
     }
 }
 
 template <int L>
 static void decode_launch(const Dev &P, const int32_t *prefix, uint32_t chunk, uint32_t n_units, int8_t *o8,
-                          uint16_t *o16, hipStream_t s) {
+                          uint16_t *o16, GroupScales gs, hipStream_t s) {
     const uint32_t blocks = (n_units + kWavesPerBlock - 1) / kWavesPerBlock;
     hipLaunchKernelGGL(k_decode<L>, dim3(blocks), dim3(kWave * kWavesPerBlock), 0, s, P, prefix, chunk, n_units,
-                       o8, o16);
+                       o8, o16, gs);
 }
 
-int launch_decode(const Dev &P, const int32_t *prefix, uint32_t chunk, int8_t *o8, uint16_t *o16,
+int launch_decode(const Dev &P, const int32_t *prefix, uint32_t chunk, int8_t *o8, uint16_t *o16, GroupScales gs,
                   hipStream_t s) {
     const uint32_t n_units = (uint32_t)(((uint64_t)P.n + chunk - 1) / chunk);
     if (n_units == 0) return IXH_OK;
     switch (P.n_levels) {
-        case 2: decode_launch<2>(P, prefix, chunk, n_units, o8, o16, s); break;
-        case 3: decode_launch<3>(P, prefix, chunk, n_units, o8, o16, s); break;
-        case 4: decode_launch<4>(P, prefix, chunk, n_units, o8, o16, s); break;
-        case 5: decode_launch<5>(P, prefix, chunk, n_units, o8, o16, s); break;
-        case 6: decode_launch<6>(P, prefix, chunk, n_units, o8, o16, s); break;
-        case 7: decode_launch<7>(P, prefix, chunk, n_units, o8, o16, s); break;
-        case 8: decode_launch<8>(P, prefix, chunk, n_units, o8, o16, s); break;
+        case 2: decode_launch<2>(P, prefix, chunk, n_units, o8, o16, gs, s); break;
+        case 3: decode_launch<3>(P, prefix, chunk, n_units, o8, o16, gs, s); break;
+        case 4: decode_launch<4>(P, prefix, chunk, n_units, o8, o16, gs, s); break;
+        case 5: decode_launch<5>(P, prefix, chunk, n_units, o8, o16, gs, s); break;
+        case 6: decode_launch<6>(P, prefix, chunk, n_units, o8, o16, gs, s); break;
+        case 7: decode_launch<7>(P, prefix, chunk, n_units, o8, o16, gs, s); break;
+        case 8: decode_launch<8>(P, prefix, chunk, n_units, o8, o16, gs, s); break;
         default: set_error("n_levels %d not in 2..8", P.n_levels); return IXH_EINVAL;
     }
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;

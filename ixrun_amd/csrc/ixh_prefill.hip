@@ -192,7 +192,8 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
                 const uint32_t slot = my_slots + (t % kPRing) * prefill_slot_bytes(L);
                 StagedUnit<L> S;
                 get_unit<L>(slot + staged_slot_words(L) * 4, S);
-                decode_unit_lds<L>(P, S, ((row_first + j) * n_chunks + c) * kStagedChunk, kStagedChunk, scale, wrow,
+                decode_unit_lds<L>(P, S, ((row_first + j) * n_chunks + c) * kStagedChunk, kStagedChunk,
+                                   [scale](uint32_t) { return scale; }, wrow,
                                    queue, lane);
             } else {
 #pragma unroll 1

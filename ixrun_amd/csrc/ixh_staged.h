@@ -217,9 +217,11 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 // more (dense mixes), the lanes keep their eight elements and repeat the level-1 scheme level by level.
 constexpr uint32_t kStagedQueue = kStagedChunk;
 
-template <int L>
+// `scale_at(e)` gives the dequantisation scale of element e of the unit; it is asked once for a lane's eight
+// consecutive elements (e a multiple of 8), so scale groups must be multiples of eight elements.
+template <int L, class ScaleAt>
 __device__ __forceinline__ void decode_unit_lds(const Dev &P, const StagedUnit<L> &S, uint32_t p_begin, uint32_t n_el,
-                                                float scale, uint16_t *dst, uint16_t *queue, uint32_t lane) {
+                                                ScaleAt scale_at, uint16_t *dst, uint16_t *queue, uint32_t lane) {
     uint32_t cnt[L - 1];
 #pragma unroll
     for (int i = 0; i < L - 1; ++i) cnt[i] = S.cnt0[i];
@@ -266,6 +268,7 @@ __device__ __forceinline__ void decode_unit_lds(const Dev &P, const StagedUnit<L
     }
     auto store = [&]() {  // dequantise, round to bf16, one 16-byte write
         float f[8];
+        const float scale = scale_at(e0);
 #pragma unroll
         for (int t = 0; t < 8; ++t) f[t] = (float)v[t] * scale;
         const staged_u32x4 packed = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
@@ -345,7 +348,7 @@ __device__ __forceinline__ void decode_unit_lds(const Dev &P, const StagedUnit<L
         const bool alive = base + lane < n_queued;
         const uint32_t p = alive ? queue[base + lane] : 0u;
         const int ve = decode_from_lds<L, 1>(P, S, space1 + base, alive, cnt);
-        if (alive) dst[p] = (uint16_t)f32_to_bf16_bits((float)ve * scale);
+        if (alive) dst[p] = (uint16_t)f32_to_bf16_bits((float)ve * scale_at(p));
     }
 }
 

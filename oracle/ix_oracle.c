@@ -24,6 +24,14 @@
  *                                     kernel sums), ixrun/engine.py:171-173
  *                                     (decode then F.linear for M > 1)
  *
+ *   ixo_gs_quantize                   ixgs/quantize.py:49-63 (per-group fp16
+ *                                     scale = group max / 15, values clamped to
+ *                                     [-127, 128])
+ *   ixo_gs_encode                     ixgs/quantize.py:65-91 (tiers by value
+ *                                     range: [-3,4], [-15,16], rest)
+ *   ixo_gs_decode_i16                 ixgs/quantize.py:113-147, ixgs/kernels.py:46-99
+ *   ixo_gs_dequant_bf16               ixgs/quantize.py:149-150, ixgs/kernels.py:102-104
+ *
  * Pinning (what each function is checked against, see tests/test_oracle.py):
  *   bit packing   closed form word[j] = sum code_i << (i*b - 32j); the known
  *                 answer pack([0..7], 3) = 0x00FAC688; round trips on the sizes
@@ -35,6 +43,11 @@
  *                 rank by linear scan on tiny inputs, round trip to the int8
  *   prefix        brute-force running counts; known answer q1=[0,3], q2=[0,2]
  *   gemm          one-hot x gives a decoded column exactly; ones give row sums
+ *   group scale   fp16 conversion against numpy's float16 (every bit pattern, and
+ *                 fp32 values on and next to every rounding boundary); the reference
+ *                 test's own property (ixgs/test_gs.py:38-52): decode equals
+ *                 bf16(round(w / s) * s) with s the fp16-rounded scale, on its
+ *                 heavy-tailed recipe; a hand-derived known answer; round trip
  * Parity unpinned: the M > 1 path of the reference ends in an external BLAS
  * whose summation order is not fixed by any reference test; ixo_gemm_f64 is the
  * build's own yardstick there.
@@ -262,4 +275,125 @@ void ixo_fused_gemv_f32(int64_t out_f, int64_t in_f, const int *level_bits, int 
         }
         y[r] = f32_to_bf16(acc);
     }
+}
+
+/* ======================================================================
+ * Group-scale sibling format (reference: ixgs/).  Same streams as (3,5,8)
+ * with code offsets 3 / 15 / 127; membership is by value range, and every
+ * group of `group` consecutive elements has its own fp16 scale.
+ * ====================================================================== */
+
+/* fp32 -> fp16 bit pattern, round to nearest even (torch .to(float16)) */
+static uint16_t f32_to_f16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    uint32_t sign = (u >> 16) & 0x8000u, a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return (uint16_t)(sign | 0x7E00u);            /* NaN */
+    if (a >= 0x47800000u) return (uint16_t)(sign | 0x7C00u);           /* >= 65536 (or inf): inf; 65520..65536 below */
+    if (a < 0x33000000u) return (uint16_t)sign;                         /* < 2^-25: zero */
+    int e = (int)(a >> 23) - 127;
+    uint32_t m = (a & 0x7FFFFFu) | 0x800000u;                          /* 24-bit significand */
+    int shift = e >= -14 ? 13 : 13 + (-14 - e);                        /* bits dropped */
+    uint32_t kept = m >> shift, rem = m & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (kept & 1u))) kept++;
+    uint32_t h;
+    if (e >= -14) h = ((uint32_t)(e + 15) << 10) + (kept - 0x400u);   /* carry into the exponent is the right answer */
+    else h = kept;                                                      /* subnormal; kept == 0x400 becomes the first normal */
+    if (h >= 0x7C00u) h = 0x7C00u;
+    return (uint16_t)(sign | h);
+}
+
+static float f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 31u, m = h & 0x3FFu, u;
+    if (e == 31) u = sign | 0x7F800000u | (m << 13);
+    else if (e != 0) u = sign | ((e + 112u) << 23) | (m << 13);
+    else if (m == 0) u = sign;
+    else {
+        int k = 0;
+        while (!(m & 0x400u)) { m <<= 1; ++k; }
+        u = sign | ((uint32_t)(113 - k) << 23) | ((m & 0x3FFu) << 13);
+    }
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+uint16_t ixo_f32_to_f16(float f) { return f32_to_f16(f); }
+float ixo_f16_to_f32(uint16_t h) { return f16_to_f32(h); }
+
+/* scales[g] = fp16( max(group max / 15, 1e-10) ); q = clamp(round_half_even(w / f32(scale)), -127, 128).
+ * A group whose fp16 scale is zero (all-zero group, or max below 4.5e-7) divides by zero in the
+ * reference and its integers are undefined there; here they are 0, which decodes to 0. */
+void ixo_gs_quantize(const uint16_t *w, int64_t n, int64_t group, uint16_t *scales, int16_t *q) {
+    int64_t n_groups = (n + group - 1) / group;
+    for (int64_t g = 0; g < n_groups; ++g) {
+        int64_t a = g * group, b = a + group < n ? a + group : n;
+        float gmax = 0.0f;
+        for (int64_t i = a; i < b; ++i) {
+            float v = fabsf(bf16_to_f32(w[i]));
+            if (v > gmax) gmax = v;
+        }
+        float s32 = gmax / 15.0f;
+        if (s32 < 1e-10f) s32 = 1e-10f;
+        uint16_t h = f32_to_f16(s32);
+        float s = f16_to_f32(h);
+        scales[g] = h;
+        for (int64_t i = a; i < b; ++i) {
+            float r = s == 0.0f ? 0.0f : rintf(bf16_to_f32(w[i]) / s);
+            if (r > 128.0f) r = 128.0f;
+            if (r < -127.0f) r = -127.0f;
+            q[i] = (int16_t)r;
+        }
+    }
+}
+
+/* b1: one bit per element (1 = tier 1); b2: one bit per element outside tier 1 (1 = tier 2);
+ * l1: 3-bit codes v+3; l2: 5-bit codes v+15; l3: bytes v+127.  Buffers zero-filled by the caller,
+ * counts[3] written.  (The reference pads an empty b2 / l3 to one element; padding is the caller's.) */
+void ixo_gs_encode(const int16_t *q, int64_t n, uint32_t *b1, uint32_t *b2, uint32_t *l1, uint32_t *l2, uint8_t *l3,
+                   int64_t *counts) {
+    int64_t n1 = 0, n2 = 0, n3 = 0, rest = 0;
+    for (int64_t p = 0; p < n; ++p) {
+        int v = q[p];
+        if (v >= -3 && v <= 4) {
+            b1[p >> 5] |= 1u << (p & 31);
+            int64_t bit = n1 * 3;
+            uint64_t c = (uint64_t)(uint32_t)(v + 3) << (bit & 31);
+            l1[bit >> 5] |= (uint32_t)c;
+            if (c >> 32) l1[(bit >> 5) + 1] |= (uint32_t)(c >> 32);
+            ++n1;
+        } else {
+            if (v >= -15 && v <= 16) {
+                b2[rest >> 5] |= 1u << (rest & 31);
+                int64_t bit = n2 * 5;
+                uint64_t c = (uint64_t)(uint32_t)(v + 15) << (bit & 31);
+                l2[bit >> 5] |= (uint32_t)c;
+                if (c >> 32) l2[(bit >> 5) + 1] |= (uint32_t)(c >> 32);
+                ++n2;
+            } else {
+                l3[n3++] = (uint8_t)(v + 127);
+            }
+            ++rest;
+        }
+    }
+    counts[0] = n1; counts[1] = n2; counts[2] = n3;
+}
+
+void ixo_gs_decode_i16(int64_t n, const uint32_t *b1, const uint32_t *b2, const uint32_t *l1, const uint32_t *l2,
+                       const uint8_t *l3, int16_t *q) {
+    int64_t n1 = 0, n2 = 0, n3 = 0, rest = 0;
+    for (int64_t p = 0; p < n; ++p) {
+        if ((b1[p >> 5] >> (p & 31)) & 1u) {
+            q[p] = (int16_t)((int)read_code(l1, n1++, 3) - 3);
+        } else {
+            if ((b2[rest >> 5] >> (rest & 31)) & 1u) q[p] = (int16_t)((int)read_code(l2, n2++, 5) - 15);
+            else q[p] = (int16_t)((int)l3[n3++] - 127);
+            ++rest;
+        }
+    }
+}
+
+/* w = bf16( f32(v) * f32(fp16 scale of the element's group) ) */
+void ixo_gs_dequant_bf16(const int16_t *q, int64_t n, int64_t group, const uint16_t *scales, uint16_t *w) {
+    for (int64_t i = 0; i < n; ++i) w[i] = f32_to_bf16((float)q[i] * f16_to_f32(scales[i / group]));
 }

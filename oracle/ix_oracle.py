@@ -37,6 +37,10 @@ def lib():
         _lib.ixo_f32_to_bf16.argtypes = [C.c_float]
         _lib.ixo_bf16_to_f32.restype = C.c_float
         _lib.ixo_bf16_to_f32.argtypes = [C.c_uint16]
+        _lib.ixo_f32_to_f16.restype = C.c_uint16
+        _lib.ixo_f32_to_f16.argtypes = [C.c_float]
+        _lib.ixo_f16_to_f32.restype = C.c_float
+        _lib.ixo_f16_to_f32.argtypes = [C.c_uint16]
     return _lib
 
 
@@ -216,3 +220,54 @@ def decode_packed_bf16(packed: dict) -> np.ndarray:
     p = packed_to_numpy(packed)
     q = decode_i8(p["N"], p["level_bits"], p["bitmaps"], p["streams"], p["last"])
     return dequant_bf16(q, p["scale_bits"]).reshape(p["out_f"], p["in_f"])
+
+
+# ---- group-scale sibling format (reference: ixgs/) ----
+
+def gs_quantize(w_bits: np.ndarray, group: int = 64):
+    """bf16 bit patterns -> (fp16 scale bits [ceil(n/group)], int16 values in [-127, 128])."""
+    w = np.ascontiguousarray(w_bits, dtype=np.uint16).reshape(-1)
+    scales = np.zeros((w.size + group - 1) // group, dtype=np.uint16)
+    q = np.zeros(w.size, dtype=np.int16)
+    lib().ixo_gs_quantize(_ptr(w, C.c_uint16), C.c_int64(w.size), C.c_int64(group), _ptr(scales, C.c_uint16),
+                          _ptr(q, C.c_int16))
+    return scales, q
+
+
+def gs_encode(q: np.ndarray) -> dict:
+    """int16 values -> dict(b1, b2, l1, l2 as uint32 words, l3 bytes, counts), unpadded."""
+    q = np.ascontiguousarray(q, dtype=np.int16).reshape(-1)
+    in1 = (q >= -3) & (q <= 4)
+    in2 = ~in1 & (q >= -15) & (q <= 16)
+    n1, n2 = int(in1.sum()), int(in2.sum())
+    n3 = q.size - n1 - n2
+    b1 = np.zeros((q.size + 31) // 32, dtype=np.uint32)
+    b2 = np.zeros((n2 + n3 + 31) // 32 + 1, dtype=np.uint32)
+    l1 = np.zeros((n1 * 3 + 31) // 32 + 1, dtype=np.uint32)
+    l2 = np.zeros((n2 * 5 + 31) // 32 + 1, dtype=np.uint32)
+    l3 = np.zeros(max(n3, 1), dtype=np.uint8)
+    counts = (C.c_int64 * 3)()
+    lib().ixo_gs_encode(_ptr(q, C.c_int16), C.c_int64(q.size), _ptr(b1, C.c_uint32), _ptr(b2, C.c_uint32),
+                        _ptr(l1, C.c_uint32), _ptr(l2, C.c_uint32), _ptr(l3, C.c_uint8), counts)
+    assert list(counts) == [n1, n2, n3]
+    return {"N": int(q.size), "b1": b1, "b2": b2[:-1], "l1": l1[:-1], "l2": l2[:-1], "l3": l3[:n3],
+            "counts": [n1, n2, n3]}
+
+
+def gs_decode_i16(n: int, b1, b2, l1, l2, l3) -> np.ndarray:
+    pad = lambda a: np.concatenate([_as_u32(a), np.zeros(1, np.uint32)])
+    l3 = np.concatenate([np.ascontiguousarray(l3, dtype=np.uint8), np.zeros(1, np.uint8)])
+    q = np.zeros(n, dtype=np.int16)
+    b1, b2, l1, l2 = pad(b1), pad(b2), pad(l1), pad(l2)
+    lib().ixo_gs_decode_i16(C.c_int64(n), _ptr(b1, C.c_uint32), _ptr(b2, C.c_uint32), _ptr(l1, C.c_uint32),
+                            _ptr(l2, C.c_uint32), _ptr(l3, C.c_uint8), _ptr(q, C.c_int16))
+    return q
+
+
+def gs_dequant_bf16(q: np.ndarray, scales: np.ndarray, group: int = 64) -> np.ndarray:
+    q = np.ascontiguousarray(q, dtype=np.int16).reshape(-1)
+    scales = np.ascontiguousarray(scales, dtype=np.uint16)
+    w = np.zeros(q.size, dtype=np.uint16)
+    lib().ixo_gs_dequant_bf16(_ptr(q, C.c_int16), C.c_int64(q.size), C.c_int64(group), _ptr(scales, C.c_uint16),
+                              _ptr(w, C.c_uint16))
+    return w

@@ -63,7 +63,7 @@ def test_malformed_packed_is_refused(mutate, needle):
     lib = _lib.lib()
     s = _packed()
     mutate(s)
-    rc = lib.ixh_prefix_build(C.byref(s), 8, 0x1000, None)
+    rc = lib.ixh_decode(C.byref(s), 0x1000, 8, None, 0x1000, None)
     assert rc == -1 and needle in lib.ixh_last_error().decode()
 
 
