@@ -60,6 +60,10 @@ WORKLOADS = {
     "encode_5120x17408_student_t": (5120, 17408, 0, "student_t"),
     "encode_5120x17408_calibrated": (5120, 17408, 0, "calibrated"),
     "encode_5120x17408_five_level": (5120, 17408, 0, "student_t", (3, 4, 5, 6, 8)),
+    # full decode to bf16 in HBM (m is unused): the per-tensor format and the group-scale sibling format
+    "decode_5120x17408_student_t": (5120, 17408, 0, "student_t"),
+    "decode_5120x17408_calibrated": (5120, 17408, 0, "calibrated"),
+    "decode_gs_5120x17408_student_t": (5120, 17408, 0, "student_t"),
 }
 
 
@@ -194,6 +198,86 @@ def bench_encode(args, dev):
     print(json.dumps(out))
 
 
+def bench_decode(args, dev):
+    """Full decode: one step = one ixh_decode (or ixh_decode_gs) launch over one packed layer into a bf16 buffer.
+    Distinct packed copies are rotated as in the headline workload.  Algorithmic bytes: packed streams (+ group
+    scales) read, 2 bytes per weight written."""
+    from ixrun_amd import _lib
+    from oracle import ix_oracle as oracle
+
+    out_f, in_f, _, recipe, *rest = WORKLOADS[args.workload]
+    weight = make_weight(out_f, in_f, recipe)
+    n = out_f * in_f
+    grouped = args.workload.startswith("decode_gs_")
+    if grouped:
+        from ixrun_amd import ixgs
+
+        packed = ixgs.int8gs_quantize(weight)
+        packed_bytes = packed["total_bytes"]
+        mk = lambda: (_lib.DevicePacked((3, 5, 8), out_f, in_f, [packed["b1"].to(dev), packed["b2"].to(dev)],
+                                        [packed["l1"].to(dev), packed["l2"].to(dev), packed["l3"].to(dev)], None),
+                      packed["group_scales"].to(dev))
+    else:
+        from ixrun_amd.quantize import int8x_quantize
+
+        packed = int8x_quantize(weight, (3, 5, 8))
+        packed_bytes = packed["total_bytes"]
+        mk = lambda: (_lib.DevicePacked.from_dict(packed, dev), None)
+    copies = args.copies or max(2, -(-600_000_000 // packed_bytes))
+    layers = [mk() for _ in range(copies)]
+    tables = [dp.prefix_build(512) for dp, _ in layers]
+    out = torch.empty(n, dtype=torch.bfloat16, device=dev)
+
+    def step(i):
+        dp, scales = layers[i % copies]
+        if grouped:
+            dp.decode_gs(tables[i % copies], 512, scales, packed["group_size"], out)
+        else:
+            dp.decode(tables[i % copies], 512, out_bf16=out)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    steps = args.steps
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        step(i)
+    stop.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(stop) / steps
+    alg_bytes = packed_bytes + 2 * n
+    # CPU beside it: the oracle's C walk (decode + dequantise) on the first rows, one core
+    rows = 640
+    if grouped:
+        scales, q = oracle.gs_quantize(weight[:rows].contiguous().view(torch.int16).numpy().view(np.uint16), 64)
+        e = oracle.gs_encode(q)
+        t0 = time.perf_counter()
+        oracle.gs_dequant_bf16(oracle.gs_decode_i16(q.size, e["b1"], e["b2"], e["l1"], e["l2"], e["l3"]), scales, 64)
+        t_c = time.perf_counter() - t0
+        level_fractions = [c / n for c in packed["counts"]]
+    else:
+        from ixrun_amd.quantize import int8x_quantize
+
+        sub = int8x_quantize(weight[:rows].contiguous(), (3, 5, 8))
+        t0 = time.perf_counter()
+        oracle.decode_packed_bf16(sub)
+        t_c = time.perf_counter() - t0
+        level_fractions = [c / n for c in packed["counts"]]
+    print(json.dumps({
+        "metric": "full decode to bf16, G weights/s", "value": n / (ms * 1e-3) / 1e9, "unit": "G weights/s", "n_gpus": 1,
+        "steps": steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8 codes x bf16/fp16 scale -> bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "out_f": out_f, "in_f": in_f, "weights": recipe,
+                   "level_fractions": level_fractions, "packed_bytes": packed_bytes, "distinct_copies": copies},
+        "roofline": {"bound": "hbm", "achieved": alg_bytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": alg_bytes / (ms * 1e-3) / HBM_PEAK, "traffic": None,
+                     "note": "algorithmic bytes = packed layer read + 2 bytes per weight written"},
+        "cpu_baseline": {"value": rows * in_f / t_c / 1e9, "unit": "G weights/s", "cores": 1, "kind": "port",
+                         "sample": f"first {rows} rows through the oracle's C decoder ({t_c:.2f} s)"},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -216,6 +300,8 @@ def main():
 
     if args.workload.startswith("encode_"):
         return bench_encode(args, dev)
+    if args.workload.startswith("decode_"):
+        return bench_decode(args, dev)
 
     from ixrun_amd.engine import StreamingLinear
 
