@@ -134,13 +134,12 @@ def bench_encode(args, dev):
     bits = (C.c_int32 * len(level_bits))(*level_bits)
     ws_bytes = int(L.ixh_encode_workspace_bytes(out_f, in_f, len(level_bits)))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    totals = torch.empty(len(level_bits), dtype=torch.int64, device=dev)
     scale = dp.tensors[-1]
     stream = _lib.current_stream(dev)
 
     def scan(i):
         _lib.check(L.ixh_encode_scan(w_dev[i % copies].data_ptr(), out_f, in_f, len(level_bits), bits, scale.data_ptr(),
-                                     table.data_ptr(), totals.data_ptr(), ws.data_ptr(), ws_bytes, stream))
+                                     table.data_ptr(), ws.data_ptr(), ws_bytes, stream))
 
     def pack(i):
         _lib.check(L.ixh_encode_pack(w_dev[i % copies].data_ptr(), C.byref(dp.struct), table.data_ptr(), stream))

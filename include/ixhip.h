@@ -168,11 +168,12 @@ size_t ixh_gemm_workspace_bytes(const IxhPacked *packed, int32_t m);
  *
  * ixh_encode_scan: w is bf16 [out_f, in_f], contiguous.  Writes
  *   scale        bf16( max(max|w|, bf16(1e-8)) / 127 )                   (quantize.py:64)
- *   prefix       the chunk-512 rank table, (n_levels-1) * ixh_prefix_entries(N, 512) entries
- *   totals       int64 [n_levels], elements per level ("counts"); nullable
- * The caller reads totals (its own synchronisation), then allocates, for i < n_levels-1,
- * bitmap i of ceil((N - totals[0] - .. - totals[i-1]) / 32) words and stream i of
- * ceil(totals[i] * level_bits[i] / 32) words, and totals[n_levels-1] bytes for the last level.
+ *   prefix       the chunk-512 rank table, (n_levels-1) rows of E = ixh_prefix_entries(N, 512)
+ *                entries; the last entry of row i, prefix[i*E + E-1], is the number of level-i
+ *                elements ("counts[i]"); the last level holds what is left of N
+ * The caller reads those totals (its own synchronisation), then allocates, for i < n_levels-1,
+ * bitmap i of ceil((N - counts[0] - .. - counts[i-1]) / 32) words and stream i of
+ * ceil(counts[i] * level_bits[i] / 32) words, and counts[n_levels-1] bytes for the last level.
  *
  * ixh_encode_pack: dst names those buffers (they are WRITTEN, despite the const of the
  * struct's fields), the scale and the table written by ixh_encode_scan for the same w.
@@ -181,7 +182,7 @@ size_t ixh_gemm_workspace_bytes(const IxhPacked *packed, int32_t m);
 size_t ixh_encode_workspace_bytes(int64_t out_f, int64_t in_f, int32_t n_levels);
 
 int ixh_encode_scan(const uint16_t *w, int64_t out_f, int64_t in_f, int32_t n_levels, const int32_t *level_bits,
-                    uint16_t *scale, int32_t *prefix, int64_t *totals, void *workspace, size_t workspace_bytes,
+                    uint16_t *scale, int32_t *prefix, void *workspace, size_t workspace_bytes,
                     ixh_stream_t stream);
 
 int ixh_encode_pack(const uint16_t *w, const IxhPacked *dst, const int32_t *prefix, ixh_stream_t stream);

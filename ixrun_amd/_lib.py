@@ -101,7 +101,7 @@ def lib() -> C.CDLL:
         L.ixh_encode_workspace_bytes.argtypes = [C.c_int64, C.c_int64, C.c_int32]
         L.ixh_encode_scan.restype = C.c_int
         L.ixh_encode_scan.argtypes = [
-            C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.POINTER(C.c_int32), C.c_void_p, C.c_void_p, C.c_void_p,
+            C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.POINTER(C.c_int32), C.c_void_p, C.c_void_p,
             C.c_void_p, C.c_size_t, C.c_void_p,
         ]
         L.ixh_encode_pack.restype = C.c_int
@@ -279,11 +279,11 @@ def encode_device(weight: torch.Tensor, level_bits) -> tuple:
     workspace = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=dev)
     scale = torch.empty(1, dtype=torch.bfloat16, device=dev)
     table = torch.empty((max(n_levels - 1, 1), max(entries, 1)), dtype=torch.int32, device=dev)
-    totals = torch.empty(max(n_levels, 1), dtype=torch.int64, device=dev)
     with torch.cuda.device(dev):
         check(L.ixh_encode_scan(weight.data_ptr(), out_f, in_f, n_levels, bits, scale.data_ptr(), table.data_ptr(),
-                                totals.data_ptr(), workspace.data_ptr(), ws_bytes, current_stream(dev)))
-        counts = [int(c) for c in totals.cpu().tolist()]
+                                workspace.data_ptr(), ws_bytes, current_stream(dev)))
+        counts = [int(c) for c in table[:, -1].cpu().tolist()]  # the one synchronisation
+        counts.append(out_f * in_f - sum(counts))
         left = out_f * in_f
         bitmaps, streams = [], []
         for i, b in enumerate(level_bits[:-1]):

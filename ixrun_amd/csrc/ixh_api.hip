@@ -259,7 +259,7 @@ size_t ixh_encode_workspace_bytes(int64_t out_f, int64_t in_f, int32_t n_levels)
 }
 
 int ixh_encode_scan(const uint16_t *w, int64_t out_f, int64_t in_f, int32_t n_levels, const int32_t *level_bits,
-                    uint16_t *scale, int32_t *prefix, int64_t *totals, void *workspace, size_t workspace_bytes,
+                    uint16_t *scale, int32_t *prefix, void *workspace, size_t workspace_bytes,
                     ixh_stream_t stream) {
     int rc = encode_levels_ok(n_levels, level_bits);
     if (rc) return rc;
@@ -274,7 +274,7 @@ int ixh_encode_scan(const uint16_t *w, int64_t out_f, int64_t in_f, int32_t n_le
     }
     int bits[IXH_MAX_LEVELS];
     for (int i = 0; i < n_levels; ++i) bits[i] = level_bits[i];
-    rc = launch_encode_scan(w, (uint32_t)n, n_levels, bits, scale, prefix, totals, workspace, (hipStream_t)stream);
+    rc = launch_encode_scan(w, (uint32_t)n, n_levels, bits, scale, prefix, workspace, (hipStream_t)stream);
     if (rc == IXH_ELAUNCH) set_error("encode_scan: launch failed");
     return rc;
 }

@@ -131,7 +131,7 @@ int launch_prefill(const Dev &P, const int32_t *prefix, const uint16_t *x, uint3
                    int64_t ldy, float *ws, hipStream_t s);
 size_t encode_workspace_bytes(uint64_t n, int n_levels);
 int launch_encode_scan(const uint16_t *w, uint32_t n, int n_levels, const int *bits, uint16_t *scale, int32_t *table,
-                       int64_t *totals, void *workspace, hipStream_t s);
+                       void *workspace, hipStream_t s);
 int launch_encode_pack(const uint16_t *w, const Dev &P, const int32_t *table, hipStream_t s);
 int launch_fill_u16(uint16_t *dst, uint32_t n, uint16_t value, hipStream_t s);
 void set_error(const char *fmt, ...);

@@ -2,7 +2,7 @@
 // byte for byte what the reference's CPU writer produces (ixrun/quantize.py:41-122 with the bit packing of
 // ixrun/bitpack.py:13-61, :87-89).  Three passes over the weights, all bound by HBM reads:
 //   1. k_enc_absmax      largest magnitude, one partial result per workgroup (no atomics, nothing to clear);
-//                        k_enc_scale turns the partial results into the bf16 scale
+//                        k_enc_scale (one wave) turns the partial results into the bf16 scale
 //   2. k_enc_count<L>    quantise, count every level per 512-element unit; the counts are then summed into
 //                        the rank table (k_enc_tile_sums, k_enc_scan), which is the table the decoders take
 //   3. k_enc_pack<L>     quantise again, one wave per unit: the table says at which bit of every stream the
@@ -18,7 +18,7 @@ namespace ixh {
 
 constexpr uint32_t kEncUnit = 512;          // elements per wave and step: eight per lane
 constexpr int kEncWaves = 4;                // waves per workgroup
-constexpr uint32_t kEncParts = 1024;        // partial maxima of pass 1
+constexpr uint32_t kEncParts = 256;         // partial maxima of pass 1 (one per workgroup of 1024 lanes)
 constexpr uint32_t kEncWindow = kEncUnit * 7 / 32 + 4;  // LDS words for one unit's piece of the widest stream
 constexpr uint32_t kScanTile = 8192;        // table entries per workgroup of the scan
 
@@ -72,21 +72,25 @@ struct EncLevels {
     int bits[IXH_MAX_LEVELS];
 };
 
-__global__ void __launch_bounds__(256) k_enc_absmax(const uint16_t *__restrict__ w, uint32_t n, uint32_t *parts) {
+__global__ void __launch_bounds__(1024) k_enc_absmax(const uint16_t *__restrict__ w, uint32_t n, uint32_t *parts) {
     const bool aligned = (reinterpret_cast<uintptr_t>(w) & 15u) == 0;
     uint32_t m = 0;
-    const uint32_t stride = gridDim.x * 256u * 8u;
-    for (uint64_t p = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * 8u; p < n; p += stride) {
+    const uint32_t stride = gridDim.x * 1024u * 8u;
+    for (uint64_t p = ((uint64_t)blockIdx.x * 1024u + threadIdx.x) * 8u; p < n; p += stride) {
         float f[8];
         load8(w, (uint32_t)p, n, aligned, f);
 #pragma unroll
         for (int t = 0; t < 8; ++t) m = max(m, (__float_as_uint(f[t]) >> 16) & 0x7fffu);
     }
-    __shared__ uint32_t wave_m[4];
+    __shared__ uint32_t wave_m[16];
     m = wave_max(m);
     if ((threadIdx.x & 63) == 0) wave_m[threadIdx.x >> 6] = m;
     __syncthreads();
-    if (threadIdx.x == 0) parts[blockIdx.x] = max(max(wave_m[0], wave_m[1]), max(wave_m[2], wave_m[3]));
+    if (threadIdx.x < 16) {
+        m = wave_m[threadIdx.x];
+        for (int off = 8; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off));
+        if (threadIdx.x == 0) parts[blockIdx.x] = m;
+    }
 }
 
 __global__ void __launch_bounds__(kWave) k_enc_scale(const uint32_t *__restrict__ parts, uint16_t *scale_out) {
@@ -106,7 +110,6 @@ k_enc_count(const uint16_t *__restrict__ w, uint32_t n, uint32_t n_units, const 
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t u0 = (blockIdx.x * kEncWaves + (threadIdx.x >> 6)) * kCountUnits;
     if (u0 >= n_units) return;
-    const float inv_scale = __fdiv_rn(1.0f, bf16_bits_to_f32(*scale_in));
     const bool aligned = (reinterpret_cast<uintptr_t>(w) & 15u) == 0;
     float thr[L - 1];
 #pragma unroll
@@ -114,6 +117,7 @@ k_enc_count(const uint16_t *__restrict__ w, uint32_t n, uint32_t n_units, const 
     float f[kCountUnits][8];
 #pragma unroll
     for (int k = 0; k < kCountUnits; ++k) load8(w, min((u0 + k) * kEncUnit + lane * 8u, n), n, aligned, f[k]);
+    const float inv_scale = __fdiv_rn(1.0f, bf16_bits_to_f32(*scale_in));
     const uint32_t entries = n_units + 1;
 #pragma unroll
     for (int k = 0; k < kCountUnits; ++k) {
@@ -132,15 +136,13 @@ k_enc_count(const uint16_t *__restrict__ w, uint32_t n, uint32_t n_units, const 
         for (int i = 0; i < L - 1; ++i) acc[i / 3] |= above[i] << (10 * (i % 3));
 #pragma unroll
         for (int j = 0; j < (L + 1) / 3; ++j) acc[j] = wave_scan_inclusive(acc[j]);
-        if (lane == 63) {
-            // elements of the unit (those past n were loaded as zero and are above nothing)
-            uint32_t prev = min(kEncUnit, n - u * kEncUnit);
+        // elements of the unit (those past n were loaded as zero and are above nothing)
+        uint32_t prev = min(kEncUnit, n - u * kEncUnit);
 #pragma unroll
-            for (int i = 0; i < L - 1; ++i) {
-                const uint32_t ab = (acc[i / 3] >> (10 * (i % 3))) & 1023u;
-                table[(size_t)i * entries + u + 1] = (int32_t)(prev - ab);
-                prev = ab;
-            }
+        for (int i = 0; i < L - 1; ++i) {
+            const uint32_t ab = (acc[i / 3] >> (10 * (i % 3))) & 1023u;
+            if (lane == 63) table[(size_t)i * entries + u + 1] = (int32_t)(prev - ab);
+            prev = ab;
         }
     }
 }
@@ -153,8 +155,8 @@ __global__ void __launch_bounds__(1024) k_enc_tile_sums(const int32_t *__restric
     uint32_t s = 0;
     for (uint32_t k = threadIdx.x; k < kScanTile && base + k < n_units; k += 1024) s += (uint32_t)row[base + k];
     __shared__ uint32_t wave_s[16];
-    for (int off = 32; off > 0; off >>= 1) s += (uint32_t)__shfl_xor((int)s, off);
-    if ((threadIdx.x & 63) == 0) wave_s[threadIdx.x >> 6] = s;
+    s = wave_scan_inclusive(s);
+    if ((threadIdx.x & 63) == 63) wave_s[threadIdx.x >> 6] = s;
     __syncthreads();
     if (threadIdx.x == 0) {
         uint32_t t = 0;
@@ -164,18 +166,17 @@ __global__ void __launch_bounds__(1024) k_enc_tile_sums(const int32_t *__restric
 }
 
 // In place, per row: row[0] = 0, row[u + 1] = counts of units 0 .. u.  Each thread takes eight consecutive entries.
-__global__ void __launch_bounds__(1024) k_enc_scan(int32_t *table, uint32_t n_units, const uint32_t *__restrict__ sums,
-                                                    int64_t *totals, uint32_t n) {
+__global__ void __launch_bounds__(1024) k_enc_scan(int32_t *table, uint32_t n_units, const uint32_t *__restrict__ sums) {
     int32_t *row = table + (size_t)blockIdx.y * (n_units + 1);
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    __shared__ uint32_t wave_s[16];
-    __shared__ uint32_t carry_in;
-    // ranks before this tile: the sums of the tiles in front of it
-    if (wave == 0) {
+    __shared__ uint32_t wave_s[16], wave_c[16];
+    // ranks before this tile: the partial sums of the tiles in front of it
+    {
         uint32_t c = 0;
-        for (uint32_t t = lane; t < blockIdx.x; t += kWave) c += sums[blockIdx.y * gridDim.x + t];
-        for (int off = 32; off > 0; off >>= 1) c += (uint32_t)__shfl_xor((int)c, off);
-        if (lane == 0) carry_in = c;
+        const uint32_t *mine_sums = sums + (size_t)blockIdx.y * gridDim.x;
+        for (uint32_t t = tid; t < blockIdx.x; t += 1024) c += mine_sums[t];
+        c = wave_scan_inclusive(c);
+        if (lane == 63) wave_c[wave] = c;
     }
     const uint32_t first = blockIdx.x * kScanTile + tid * 8u;
     uint32_t v[8];
@@ -188,32 +189,26 @@ __global__ void __launch_bounds__(1024) k_enc_scan(int32_t *table, uint32_t n_un
     const uint32_t incl = wave_scan_inclusive(mine);
     if (lane == 63) wave_s[wave] = incl;
     __syncthreads();
-    uint32_t run = carry_in + incl - mine;
-    for (uint32_t k = 0; k < wave; ++k) run += wave_s[k];
+    uint32_t run = incl - mine;
+    for (uint32_t k = 0; k < 16; ++k) run += wave_c[k] + (k < wave ? wave_s[k] : 0u);
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
         run += v[t];
         if (first + t < n_units) row[first + t + 1] = (int32_t)run;
     }
     if (blockIdx.x == 0 && tid == 0) row[0] = 0;
-    // level totals for the caller: the last entry of each row; the last level takes what is left.  Written by
-    // the workgroup that owns the row's last entry; the last level's total by a later, tiny kernel.
-    if (totals && n_units != 0 && first <= n_units - 1 && n_units - 1 < first + 8) totals[blockIdx.y] = (int64_t)run;
-    (void)n;
 }
 
-__global__ void k_enc_last_total(int64_t *totals, int n_levels, uint32_t n, uint32_t n_units) {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    int64_t rest = n;
-    for (int i = 0; i < n_levels - 1; ++i) {
-        if (n_units == 0) totals[i] = 0;
-        rest -= totals[i];
-    }
-    totals[n_levels - 1] = rest;
-}
+// every stream that is assembled with OR, in one launch
+struct EncClear {
+    uint32_t *dst[2 * (IXH_MAX_LEVELS - 1)];
+    uint32_t words[2 * (IXH_MAX_LEVELS - 1)];
+    int n;
+};
 
-__global__ void __launch_bounds__(256) k_enc_clear(uint32_t *dst, uint32_t words) {
-    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < words; i += gridDim.x * 256u) dst[i] = 0u;
+__global__ void __launch_bounds__(256) k_enc_clear(EncClear c) {
+    for (int k = 0; k < c.n; ++k)
+        for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < c.words[k]; i += gridDim.x * 256u) c.dst[k][i] = 0u;
 }
 
 // Destination of the encoder: the same fields as Dev, writable.
@@ -423,19 +418,21 @@ size_t encode_workspace_bytes(uint64_t n, int n_levels) {
 template <int L>
 static void scan_launch(const uint16_t *w, uint32_t n, uint32_t n_units, const EncLevels &lv, const uint16_t *scale,
                         int32_t *table, hipStream_t s) {
-    hipLaunchKernelGGL(k_enc_count<L>, dim3((n_units + kEncWaves * kCountUnits - 1) / (kEncWaves * kCountUnits)), dim3(kWave * kEncWaves),
-                       0, s, w, n, n_units, scale, lv, table);
+    const uint32_t per_block = kEncWaves * kCountUnits;
+    hipLaunchKernelGGL(k_enc_count<L>, dim3((n_units + per_block - 1) / per_block), dim3(kWave * kEncWaves), 0, s, w, n,
+                       n_units, scale, lv, table);
 }
 
 int launch_encode_scan(const uint16_t *w, uint32_t n, int n_levels, const int *bits, uint16_t *scale, int32_t *table,
-                       int64_t *totals, void *workspace, hipStream_t s) {
+                       void *workspace, hipStream_t s) {
     const uint32_t n_units = (n + kEncUnit - 1) / kEncUnit;
+    const uint32_t tiles = max(1u, (n_units + kScanTile - 1) / kScanTile);
     uint32_t *parts = static_cast<uint32_t *>(workspace);
     uint32_t *sums = parts + kEncParts;
     EncLevels lv;
     lv.n_levels = n_levels;
     for (int i = 0; i < IXH_MAX_LEVELS; ++i) lv.bits[i] = i < n_levels ? bits[i] : 0;
-    hipLaunchKernelGGL(k_enc_absmax, dim3(kEncParts), dim3(256), 0, s, w, n, parts);
+    hipLaunchKernelGGL(k_enc_absmax, dim3(kEncParts), dim3(1024), 0, s, w, n, parts);
     hipLaunchKernelGGL(k_enc_scale, dim3(1), dim3(kWave), 0, s, parts, scale);
     switch (n_levels) {
         case 2: scan_launch<2>(w, n, n_units, lv, scale, table, s); break;
@@ -446,11 +443,8 @@ int launch_encode_scan(const uint16_t *w, uint32_t n, int n_levels, const int *b
         case 7: scan_launch<7>(w, n, n_units, lv, scale, table, s); break;
         default: scan_launch<8>(w, n, n_units, lv, scale, table, s); break;
     }
-    const uint32_t tiles = max(1u, (n_units + kScanTile - 1) / kScanTile);
-    if (n_units != 0)
-        hipLaunchKernelGGL(k_enc_tile_sums, dim3(tiles, n_levels - 1), dim3(1024), 0, s, table, n_units, sums);
-    hipLaunchKernelGGL(k_enc_scan, dim3(tiles, n_levels - 1), dim3(1024), 0, s, table, n_units, sums, totals, n);
-    if (totals) hipLaunchKernelGGL(k_enc_last_total, dim3(1), dim3(64), 0, s, totals, n_levels, n, n_units);
+    hipLaunchKernelGGL(k_enc_tile_sums, dim3(tiles, n_levels - 1), dim3(1024), 0, s, table, n_units, sums);
+    hipLaunchKernelGGL(k_enc_scan, dim3(tiles, n_levels - 1), dim3(1024), 0, s, table, n_units, sums);
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }
 
@@ -476,14 +470,22 @@ int launch_encode_pack(const uint16_t *w, const Dev &P, const int32_t *table, hi
     }
     out.last = const_cast<uint8_t *>(P.last);
     out.last_bytes = P.last_bytes;
+    EncClear clr;
+    clr.n = 0;
+    uint32_t most = 0;
     for (int i = 0; i < P.n_levels - 1; ++i) {
-        if (out.bm_words[i] && i > 0)  // bitmap 0 is written in whole words
-            hipLaunchKernelGGL(k_enc_clear, dim3(min(2048u, (out.bm_words[i] + 255u) / 256u)), dim3(256), 0, s, out.bm[i],
-                               out.bm_words[i]);
-        if (out.st_words[i])
-            hipLaunchKernelGGL(k_enc_clear, dim3(min(2048u, (out.st_words[i] + 255u) / 256u)), dim3(256), 0, s, out.st[i],
-                               out.st_words[i]);
+        if (out.bm_words[i] && i > 0) {  // bitmap 0 is written in whole words
+            clr.dst[clr.n] = out.bm[i];
+            clr.words[clr.n++] = out.bm_words[i];
+            most = max(most, out.bm_words[i]);
+        }
+        if (out.st_words[i]) {
+            clr.dst[clr.n] = out.st[i];
+            clr.words[clr.n++] = out.st_words[i];
+            most = max(most, out.st_words[i]);
+        }
     }
+    if (clr.n) hipLaunchKernelGGL(k_enc_clear, dim3(min(2048u, (most + 255u) / 256u)), dim3(256), 0, s, clr);
     if (n_units != 0) {
         switch (P.n_levels) {
             case 2: pack_launch<2>(w, n, n_units, P.scale, lv, table, out, s); break;
