@@ -290,6 +290,13 @@ k_enc_pack(const uint16_t *__restrict__ w, uint32_t n, uint32_t n_units, const u
     const float inv_scale = __fdiv_rn(1.0f, bf16_bits_to_f32(*scale_in));
     const bool aligned = (reinterpret_cast<uintptr_t>(w) & 15u) == 0;
     const uint32_t entries = n_units + 1;
+    // the unit's first rank in every level and the next unit's: requested now, needed after the first level
+    uint32_t ranks0[L - 1], ranks1[L - 1];
+#pragma unroll
+    for (int i = 0; i < L - 1; ++i) {
+        ranks0[i] = (uint32_t)table[(size_t)i * entries + u];
+        ranks1[i] = (uint32_t)table[(size_t)i * entries + u + 1];
+    }
     const uint32_t e0 = u * kEncUnit, e1 = min(e0 + kEncUnit, n);  // the unit's elements
     const uint32_t p = e0 + lane * 8u;
     float f[8];
@@ -344,7 +351,7 @@ k_enc_pack(const uint16_t *__restrict__ w, uint32_t n, uint32_t n_units, const u
     const uint32_t incl = wave_scan_inclusive(n_codes | (n_above << 16));
     const uint32_t bits_before = (incl & 0xffffu) - n_codes, above_before = (incl >> 16) - n_above;
     const uint32_t total_above = (uint32_t)__builtin_amdgcn_readlane((int)(incl >> 16), 63);
-    uint32_t rank0 = (uint32_t)table[u], rank1 = (uint32_t)table[u + 1];
+    uint32_t rank0 = ranks0[0], rank1 = ranks1[0];
     {
         const uint64_t bit0 = (uint64_t)rank0 * b0, bit1 = (uint64_t)rank1 * b0;
         window_or(win, ((uint32_t)bit0 & 31u) + bits_before, codes, n_codes);
@@ -368,8 +375,8 @@ k_enc_pack(const uint16_t *__restrict__ w, uint32_t n, uint32_t n_units, const u
     for (int i = 1; i < L - 1; ++i) {
         const uint32_t b = (uint32_t)lv.bits[i];
         const int thr_i = threshold_of((int)b);
-        rank0 = (uint32_t)table[(size_t)i * entries + u];
-        rank1 = (uint32_t)table[(size_t)i * entries + u + 1];
+        rank0 = ranks0[i];
+        rank1 = ranks1[i];
         const uint64_t bit0 = (uint64_t)rank0 * b, bit1 = (uint64_t)rank1 * b;
         uint32_t seen_alive = space0 & 31u, seen_codes = (uint32_t)bit0 & 31u;  // window positions, in bits
         if (space1 > space0) {
