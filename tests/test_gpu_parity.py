@@ -186,7 +186,7 @@ def run_gemv(dp, chunk, x, m, dev, flags=0, atomic=False):
 
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("shape", [(64, 512), (37, 1024), (130, 1536), (256, 4608)])
-@pytest.mark.parametrize("m", [1, 2, 3, 8, 16])
+@pytest.mark.parametrize("m", [1, 2, 3, 8, 9, 13, 16])
 def test_gemv_fast_and_general(oracle, dev, kind, shape, m):
     from ixrun_amd import _lib
 
