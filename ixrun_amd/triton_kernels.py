@@ -48,14 +48,16 @@ def precompute_block_offsets(packed: dict, blk: int = TRITON_BLOCK, device=None)
 def decode_weight_triton(packed: dict, device=None, dtype=torch.bfloat16) -> torch.Tensor:
     """Decode a packed dict to a ``[out_f, in_f]`` weight on the GPU.
 
-    Same call as the reference's ``decode_weight_triton``
-    (``ixrun/triton_kernels.py:224-259``).  Without any GPU in the process the
-    reference decodes with the torch scatter path and so does this function;
-    with a GPU the HIP kernel is the only path and a missing ``libixhip.so``
-    raises.  Every level scheme goes through the kernel, not only (3,5,8).
+    Same call as the reference's ``decode_weight_triton`` (``ixrun/triton_kernels.py:224-259``), with two
+    differences: every level scheme goes through the kernel, not only (3,5,8), and there is no silent
+    fallback.  The reference switches to its torch scatter decoder when Triton or the GPU is missing; here a
+    process without a GPU or without the built ``libixhip.so`` gets an error, and ``decode_weight_scatter`` is
+    the CPU decoder to call by name (``Int8XLinear`` does so in a process that has no GPU at all, as the
+    reference's does at ``ixrun/linear.py:84-86``).
     """
     if not torch.cuda.is_available():
-        return decode_weight_scatter(packed, device, dtype)
+        raise RuntimeError("decode_weight_triton runs the HIP kernel and needs the GPU; "
+                           "decode_weight_scatter is the CPU decoder")
     device = torch.device(device) if device is not None else torch.device("cuda")
     dp = _lib.DevicePacked.from_dict(packed, device)
     out = torch.empty(packed["N"], dtype=torch.bfloat16, device=device)
