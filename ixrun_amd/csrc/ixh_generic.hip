@@ -41,30 +41,70 @@ k_count_level(Dev P, int level, uint32_t chunk, uint32_t n_units, int32_t *prefi
     if (lane == 0) prefix[(size_t)level * entries + u + 1] = (int32_t)count;
 }
 
-// In place: row[0] = 0, row[u+1] = row[1] + ... + row[u+1].  One block.
-__global__ void __launch_bounds__(1024) k_scan_row(int32_t *row, uint32_t n_units) {
-    __shared__ uint32_t partial[1024];
-    const uint32_t t = threadIdx.x;
-    const uint32_t seg = (n_units + 1023) / 1024;
-    const uint32_t a = min(t * seg, n_units), b = min(a + seg, n_units);
-    uint32_t sum = 0;
-    for (uint32_t u = a; u < b; ++u) sum += (uint32_t)row[u + 1];
-    partial[t] = sum;
-    __syncthreads();
-    if (t == 0) {
-        uint32_t run = 0;
-        for (int i = 0; i < 1024; ++i) {
-            const uint32_t v = partial[i];
-            partial[i] = run;
-            run += v;
-        }
-        row[0] = 0;
+// In place: row[0] = 0, row[u+1] = row[1] + ... + row[u+1], without a workspace, in three launches over tiles of
+// kScanTile entries.  k_scan_tiles scans every tile by itself; the last entry of a tile then holds the tile's sum.
+// k_scan_tile_ends (one workgroup) turns those last entries into their final values.  k_scan_tile_add adds the
+// final value of the tile in front to every other entry of a tile: it reads only entries it never writes.
+constexpr uint32_t kScanTile = 8192;
+
+__global__ void __launch_bounds__(1024) k_scan_tiles(int32_t *row, uint32_t n_units) {
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    __shared__ uint32_t wave_s[16];
+    const uint32_t first = blockIdx.x * kScanTile + tid * 8u;
+    uint32_t v[8], mine = 0;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        v[t] = first + t < n_units ? (uint32_t)row[first + t + 1] : 0u;
+        mine += v[t];
     }
+    const uint32_t incl = wave_scan_inclusive(mine);
+    if (lane == 63) wave_s[wave] = incl;
     __syncthreads();
-    uint32_t run = partial[t];
-    for (uint32_t u = a; u < b; ++u) {
-        run += (uint32_t)row[u + 1];
-        row[u + 1] = (int32_t)run;
+    uint32_t run = incl - mine;
+    for (uint32_t k = 0; k < wave; ++k) run += wave_s[k];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        run += v[t];
+        if (first + t < n_units) row[first + t + 1] = (int32_t)run;
+    }
+    if (blockIdx.x == 0 && tid == 0) row[0] = 0;
+}
+
+__global__ void __launch_bounds__(1024) k_scan_tile_ends(int32_t *row, uint32_t n_units, uint32_t tiles) {
+    __shared__ uint32_t carry;
+    __shared__ uint32_t wave_s[16];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid == 0) carry = 0;
+    __syncthreads();
+    for (uint32_t base = 0; base < tiles; base += 1024) {
+        const uint32_t t = base + tid;
+        const uint32_t at = min((t + 1) * kScanTile, n_units);  // entry index of the tile's last unit, plus one
+        const uint32_t mine = t < tiles ? (uint32_t)row[at] : 0u;
+        const uint32_t incl = wave_scan_inclusive(mine);
+        if (lane == 63) wave_s[wave] = incl;
+        __syncthreads();
+        uint32_t run = carry + incl;
+        for (uint32_t k = 0; k < wave; ++k) run += wave_s[k];
+        if (t < tiles) row[at] = (int32_t)run;
+        __syncthreads();
+        if (tid == 1023) carry = run;
+        __syncthreads();
+    }
+}
+
+__global__ void __launch_bounds__(1024) k_scan_tile_add(int32_t *row, uint32_t n_units) {
+    const uint32_t tile = blockIdx.x + 1;  // the first tile is final already
+    const uint32_t add = (uint32_t)row[tile * kScanTile];  // final value of the last entry of the tile in front
+    const uint32_t last = min((tile + 1) * kScanTile, n_units);
+    for (uint32_t e = tile * kScanTile + 1 + threadIdx.x; e < last; e += 1024) row[e] = (int32_t)((uint32_t)row[e] + add);
+}
+
+static void launch_scan_row(int32_t *row, uint32_t n_units, hipStream_t s) {
+    const uint32_t tiles = max(1u, (n_units + kScanTile - 1) / kScanTile);
+    hipLaunchKernelGGL(k_scan_tiles, dim3(tiles), dim3(1024), 0, s, row, n_units);
+    if (tiles > 1) {
+        hipLaunchKernelGGL(k_scan_tile_ends, dim3(1), dim3(1024), 0, s, row, n_units, tiles);
+        hipLaunchKernelGGL(k_scan_tile_add, dim3(tiles - 1), dim3(1024), 0, s, row, n_units);
     }
 }
 
@@ -77,7 +117,7 @@ int launch_prefix_build(const Dev &P, uint32_t chunk, int32_t *prefix, hipStream
             hipLaunchKernelGGL(k_count_level, dim3(blocks), dim3(kWave * kWavesPerBlock), 0, s, P, i, chunk,
                                n_units, prefix);
         }
-        hipLaunchKernelGGL(k_scan_row, dim3(1), dim3(1024), 0, s, prefix + (size_t)i * entries, n_units);
+        launch_scan_row(prefix + (size_t)i * entries, n_units, s);
     }
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }

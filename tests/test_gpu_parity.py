@@ -86,7 +86,9 @@ KINDS = ["outlier", "student_t", "calibrated_pow2", "calibrated_odd_scale", "onl
 # ---------------------------------------------------------------- rank tables
 @pytest.mark.parametrize("shape,level_bits,chunk", [
     ((64, 1024), (3, 5, 8), 512), ((96, 1024), (3, 5, 8), 1024), ((33, 96), (3, 4, 5, 6, 8), 32),
-    ((5, 7), (3, 5, 8), 7), ((17, 100), (3, 5, 8), 1024), ((300, 1536), (3, 5, 8), 512), ((7, 33), (2, 8), 5)])
+    ((5, 7), (3, 5, 8), 7), ((17, 100), (3, 5, 8), 1024), ((300, 1536), (3, 5, 8), 512), ((7, 33), (2, 8), 5),
+    # more table entries than one scan tile of 8192: 38 664, 73 728 (nine whole tiles) and 8193 units
+    ((300, 1031), (3, 5, 8), 8), ((256, 4608), (3, 4, 5, 6, 8), 16), ((8193, 4), (3, 5, 8), 4), ((2048, 2048), (3, 5, 8), 512)])
 def test_prefix_build(oracle, dev, shape, level_bits, chunk):
     p = quantize(outlier_weight(*shape, seed=7), level_bits)
     dp = device_packed(p, dev)
