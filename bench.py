@@ -52,6 +52,7 @@ WORKLOADS = {
     "prefill_5120x5120_m512_five_level": (5120, 5120, 512, "student_t", (3, 4, 5, 6, 8)),
     "prefill_5120x5120_m512_358": (5120, 5120, 512, "student_t"),
     "prefill_5120x17408_m512_358": (5120, 17408, 512, "student_t"),
+    "prefill_5120x17408_m512_five_level": (5120, 17408, 512, "student_t", (3, 4, 5, 6, 8)),
     "prefill_5120x5120_m64_five_level": (5120, 5120, 64, "student_t", (3, 4, 5, 6, 8)),
     "prefill_5120x5120_m128_five_level": (5120, 5120, 128, "student_t", (3, 4, 5, 6, 8)),
     "prefill_5120x5120_m256_five_level": (5120, 5120, 256, "student_t", (3, 4, 5, 6, 8)),
