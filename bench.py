@@ -35,6 +35,12 @@ MEASURED_TRAFFIC_BYTES = {
     "down_proj_5120x17408_m1_student_t": 23078.5 * 2.0 * 1024 + 16.0 * 1024,
     "down_proj_5120x17408_m1_calibrated": 33545.4 * 2.0 * 1024 + 640.0 * 1024,
     "prefill_5120x5120_m512_five_level": 50297.9 * 2.0 * 1024 + 30720.0 * 1024,
+    "attn_proj_5120x5120_m1_student_t": 7118.0 * 2.0 * 1024 + 16.0 * 1024,
+    "gate_up_17408x5120_m4_student_t": 23193.0 * 2.0 * 1024 + 181.0 * 1024,
+    "decode_5120x17408_student_t": 25672.0 * 2.0 * 1024 + 174080.0 * 1024,
+    "decode_gs_5120x17408_student_t": 33772.0 * 2.0 * 1024 + 174080.0 * 1024,
+    # all kernels of one encode step together (absmax, count, scans, clear, pack)
+    "encode_5120x17408_student_t": (87053 + 87092 + 1402 + 15 + 92442) * 2.0 * 1024 + (32 + 2040 + 1362 + 32694 + 63405) * 1024,
 }
 
 WORKLOADS = {
@@ -187,7 +193,7 @@ def bench_encode(args, dev):
                    "distinct_copies": copies},
         "us": {"scan_median": float(np.median(t_scan) * 1e3), "pack_median": float(np.median(t_pack) * 1e3)},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": alg_bytes / (ms * 1e-3) / HBM_PEAK, "traffic": None,
+                     "frac": alg_bytes / (ms * 1e-3) / HBM_PEAK, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "note": f"algorithmic bytes = weight read once + packed output + table; the three passes move "
                              f"about {moved / 1e6:.0f} MB ({moved / (ms * 1e-3) / 1e9:.0f} GB/s)"},
         "host_wall_ms_per_step": wall_ms / steps,
@@ -271,7 +277,7 @@ def bench_decode(args, dev):
         "config": {"workload": args.workload, "out_f": out_f, "in_f": in_f, "weights": recipe,
                    "level_fractions": level_fractions, "packed_bytes": packed_bytes, "distinct_copies": copies},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": alg_bytes / (ms * 1e-3) / HBM_PEAK, "traffic": None,
+                     "frac": alg_bytes / (ms * 1e-3) / HBM_PEAK, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "note": "algorithmic bytes = packed layer read + 2 bytes per weight written"},
         "cpu_baseline": {"value": rows * in_f / t_c / 1e9, "unit": "G weights/s", "cores": 1, "kind": "port",
                          "sample": f"first {rows} rows through the oracle's C decoder ({t_c:.2f} s)"},
