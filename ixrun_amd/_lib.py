@@ -21,6 +21,7 @@ IXH_GEMV_FORCE_GENERIC = 2
 IXH_GEMV_COLUMN_KERNEL = 4
 IXH_GEMV_FORCE_358 = 8
 IXH_GEMV_STAGED = 16
+IXH_GEMV_DENSE = 32
 
 IXH_EUNSUPPORTED = -2
 ERROR_NAMES = {-1: "IXH_EINVAL", -2: "IXH_EUNSUPPORTED", -3: "IXH_ELAUNCH", -4: "IXH_EWORKSPACE"}

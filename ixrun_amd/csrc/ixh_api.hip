@@ -184,7 +184,7 @@ int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, cons
     // The (3,5,8) kernels are built for tensors that are almost all level 1 (every other element costs
     // them a queue record); denser mixes go to the general kernel unless the caller insists.
     const bool mostly_l1 = (uint64_t)d.st_words[0] * 32u / 3u >= (uint64_t)d.n / 100u * 97u;
-    const bool fast = !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED)) && is_358(d) &&
+    const bool fast = !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED | IXH_GEMV_DENSE)) && is_358(d) &&
                       fast358_supports(d, (uint32_t)chunk, m) &&
                       (mostly_l1 || (flags & (IXH_GEMV_COLUMN_KERNEL | IXH_GEMV_FORCE_358)));
     if (fast && !atomic && !(flags & IXH_GEMV_COLUMN_KERNEL)) {
@@ -202,6 +202,10 @@ int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, cons
     if (fast && rc == IXH_EUNSUPPORTED)
         rc = launch_gemv_358(d, prefix, (uint32_t)chunk, x, m, ldx, y, ldy, y32, (float *)workspace, atomic,
                              (hipStream_t)stream);
+    if (rc == IXH_EUNSUPPORTED && !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED)) &&
+        (!mostly_l1 || (flags & IXH_GEMV_DENSE)) && gemv_dense358_supports(d, (uint32_t)chunk, m, x))
+        // (3,5,8), one activation row, many elements above level 1: level-by-level products over compacted x
+        rc = launch_gemv_dense358(d, prefix, x, y, y32, (float *)workspace, atomic, (hipStream_t)stream);
     if (rc == IXH_EUNSUPPORTED && !(flags & IXH_GEMV_FORCE_GENERIC) && gemv_staged_supports(d, (uint32_t)chunk, x, ldx))
         // any scheme, any mix, whole 512-element units: streams staged in LDS, eight elements per lane
         rc = launch_gemv_staged(d, prefix, x, m, ldx, y, ldy, y32, (float *)workspace, atomic, (hipStream_t)stream);

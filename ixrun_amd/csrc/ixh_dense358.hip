@@ -1,0 +1,293 @@
+// (3,5,8) fused decode + GEMV for one activation row when every level is well populated (e.g. the 55 / 40 / 5 %
+// mix of real LLM weights), where decoding element by element costs ~45 instructions per weight and lane.
+//
+// This kernel does not decode by position.  The codes of a level are dense in their stream, so the dot product of
+// a run of weights is taken level by level over whole codes at fixed positions:
+//     sum_k w_k x_k = sum_{k in level 1} w_k x_k + sum_{k in level 2} w_k x_k + sum_{k in level 3} w_k x_k
+// and what depends on the bitmaps is moved to the activations: the x values of a span are scattered ("compacted")
+// into three arrays in LDS, one per level, in the order of that level's codes.  Scattering costs an LDS write per
+// weight and a dozen integer instructions (two bit tests, three running counters, a select); the three dense passes
+// then cost about one instruction per weight.
+//
+// A wave takes spans of up to 2048 consecutive elements of one weight row (four 512-element table units).  The
+// rank table gives the span's first code in every stream and its level counts.  Lane l owns bitmap word l (32
+// elements, 16 x pairs in registers): popcount + wave prefix sums give the lane's first slot in each compacted array
+// (bitmap 1 is read at the lane's first element not in level 1).  The dense passes split each level's codes evenly over
+// the 64 lanes (an even number E of codes per lane, wave-uniform), read them with plain loads at addresses that
+// depend only on the table, and meet the compacted x pairs in v_dot2_f32_bf16: level 1 through the table of
+// dequantised pairs (two 3-bit codes -> one LDS read), levels 2 and 3 by arithmetic, each weight rounded to bf16 as
+// the reference's decoder does (ixrun/triton_kernels.py:168-177).  The array of each level is padded with zeros up
+// to 64 * E slots, so codes read past a level's end meet a zero.
+//
+// No LDS-DMA and no hand-counted waits here: the kernel is bound by instruction issue (about 650 vector instructions
+// per 2048 weights), six waves per SIMD cover the load latency.  Partial sums of the spans of a row are combined
+// through the workspace in span order (or added to y32 with atomics).
+#include "ixh_fast358.h"
+
+namespace ixh {
+
+typedef uint32_t d_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t d_u32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 d_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float d_f32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kDnWaves = 4;                  // waves per workgroup
+constexpr uint32_t kDnSpan = 2048;           // elements per span: four table units of one row
+constexpr uint32_t kDnSlots = kDnSpan + 3 * 128;  // compacted x slots per wave: three arrays, each padded to 64 * E
+constexpr uint32_t kDnLutBytes = 64 * 32 * 4;     // pair table: 64 code pairs x 32 lane copies
+
+enum : int { kDnDirect = 0, kDnAtomic = 1, kDnWorkspace = 2 };
+
+// sum over the wave, valid in lane 63 (DPP: shifts inside the 16-lane rows, then the two row broadcasts)
+#define IXH_DN_DPP_ADD(v, ctrl, row_mask, bound) \
+    v += __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), ctrl, row_mask, 0xf, bound))
+__device__ __forceinline__ float dn_wave_sum(float v) {
+    IXH_DN_DPP_ADD(v, 0x111, 0xf, true);
+    IXH_DN_DPP_ADD(v, 0x112, 0xf, true);
+    IXH_DN_DPP_ADD(v, 0x114, 0xf, true);
+    IXH_DN_DPP_ADD(v, 0x118, 0xf, true);
+    IXH_DN_DPP_ADD(v, 0x142, 0xa, false);
+    IXH_DN_DPP_ADD(v, 0x143, 0xc, false);
+    return v;
+}
+#undef IXH_DN_DPP_ADD
+
+__device__ __forceinline__ uint32_t dn_pack(float lo, float hi) {
+    const d_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, d_bf16x2));
+}
+
+__device__ __forceinline__ float dn_dot2(uint32_t w, uint32_t x, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(d_bf16x2, w), __builtin_bit_cast(d_bf16x2, x), acc, false);
+}
+
+__global__ void __launch_bounds__(kWave *kDnWaves)
+k_gemv358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t spans_per_row, uint32_t n_spans,
+                const uint16_t *__restrict__ x, uint16_t *__restrict__ y,
+                float *__restrict__ y32, float *__restrict__ ws, int out_mode) {
+    __shared__ __attribute__((aligned(16))) uint32_t lut[kDnLutBytes / 4];
+    __shared__ __attribute__((aligned(16))) uint16_t xc_all[kDnWaves][kDnSlots];
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const float scale = bf16_bits_to_f32(*P.scale);
+    const float m15 = -15.0f * scale, m127 = -127.0f * scale;  // exact: 7 + 8 significant bits at most
+
+    // pair table: entry (c0 | c1 << 3) = the two dequantised level-1 weights, one copy per bank
+    for (uint32_t e = tid; e < 64 * 32; e += kWave * kDnWaves) {
+        const uint32_t idx = e >> 5;
+        lut[e] = dn_pack(dequant((int)(idx & 7u) - 3, scale), dequant((int)(idx >> 3) - 3, scale));
+    }
+    __syncthreads();
+
+    uint16_t *const xc = xc_all[wave];
+    const uint32_t lut_lane = (lane & 31u) << 2;
+    const uint32_t entries = P.out_f * n_chunks + 1;
+    const uint32_t *__restrict__ b1 = P.bm[0];
+    const __amdgpu_buffer_rsrc_t l1_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[0], 0, (int)(P.st_words[0] * 4u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t l2_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[1], 0, (int)(P.st_words[1] * 4u), 0x00020000);
+    // whole dwords of the byte stream (device allocations are 256-byte granular, the last dword is there to read)
+    const __amdgpu_buffer_rsrc_t l3_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.last, 0, (int)((P.last_bytes + 3u) & ~3u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t b2_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[1], 0, (int)(P.bm_words[1] * 4u), 0x00020000);
+
+    // spans are dealt to the waves of the launch in turn: with a launch that is resident as a whole, every wave
+    // gets the same number of spans (give or take one)
+    const uint32_t n_waves = gridDim.x * kDnWaves;
+    for (uint32_t s = blockIdx.x * kDnWaves + wave; s < n_spans; s += n_waves) {
+        const uint32_t row = s / spans_per_row, k = s - row * spans_per_row;
+        const uint32_t c0 = 4 * k, nb = min(4u, n_chunks - c0);
+        const uint32_t u0 = row * n_chunks + c0;
+        const uint32_t n_el = nb * kFastChunk, p0 = u0 * kFastChunk;
+        const uint32_t q1a = (uint32_t)prefix[u0], q1b = (uint32_t)prefix[u0 + nb];
+        const uint32_t q2a = (uint32_t)prefix[entries + u0], q2b = (uint32_t)prefix[entries + u0 + nb];
+        const uint32_t n1 = q1b - q1a, n2 = q2b - q2a, n3 = n_el - n1 - n2;
+        // codes per lane in the dense passes (even), and the padded sizes of the compacted arrays
+        const uint32_t e1 = 2 * ((n1 + 127) / 128), e2 = 2 * ((n2 + 127) / 128), e3 = 2 * ((n3 + 127) / 128);
+        const uint32_t base2 = 64 * e1, base3 = base2 + 64 * e2;
+
+        // ---- loads whose addresses follow from the table alone ----
+        const bool valid = 32 * lane < n_el;
+        const uint32_t w1 = valid ? b1[(p0 >> 5) + lane] : 0u;
+        uint32_t xr[16];
+        if (valid) {
+            const uint4 *xp = reinterpret_cast<const uint4 *>(x + c0 * kFastChunk + 32 * lane);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint4 v = xp[t];
+                xr[4 * t] = v.x; xr[4 * t + 1] = v.y; xr[4 * t + 2] = v.z; xr[4 * t + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 16; ++t) xr[t] = 0u;
+        }
+        // The code streams, read through buffer descriptors: a dword past a stream's end reads as zero, so no lane
+        // needs a bounds test; lanes whose share lies past the level's last code read codes of the next span, which
+        // then meet the zero pads of the compacted arrays.
+        // level-1 codes of this lane: e1 of them from code q1a + lane * e1 on (96 bits at most)
+        uint32_t c1w[3];
+        {
+            const uint64_t bit = (uint64_t)(q1a + lane * e1) * 3u;
+            const uint32_t wi = (uint32_t)(bit >> 5), sh = (uint32_t)bit & 31u;
+            const d_u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(l1_rsrc, (int)(wi * 4u), 0, 0);
+            c1w[0] = __builtin_amdgcn_alignbit(d[1], d[0], sh);
+            c1w[1] = __builtin_amdgcn_alignbit(d[2], d[1], sh);
+            c1w[2] = __builtin_amdgcn_alignbit(d[3], d[2], sh);
+        }
+        // level-2 codes: e2 of them from code q2a + lane * e2 on (160 bits at most)
+        uint32_t c2w[5];
+        {
+            const uint64_t bit = (uint64_t)(q2a + lane * e2) * 5u;
+            const uint32_t wi = (uint32_t)(bit >> 5), sh = (uint32_t)bit & 31u;
+            const d_u32x4 da = __builtin_amdgcn_raw_buffer_load_b128(l2_rsrc, (int)(wi * 4u), 0, 0);
+            const d_u32x2 db = __builtin_amdgcn_raw_buffer_load_b64(l2_rsrc, (int)(wi * 4u + 16u), 0, 0);
+            const uint32_t d[6] = {da[0], da[1], da[2], da[3], db[0], db[1]};
+#pragma unroll
+            for (int j = 0; j < 5; ++j) c2w[j] = __builtin_amdgcn_alignbit(d[j + 1], d[j], sh);
+        }
+        // level-3 bytes: e3 of them from byte (p0 - q1a - q2a) + lane * e3 on (32 bytes at most), read as dwords
+        uint32_t c3w[8];
+        {
+            const uint32_t at = (p0 - q1a - q2a) + lane * e3;
+            const uint32_t wi = at >> 2, sh = (at & 3u) * 8u;
+            const d_u32x4 da = __builtin_amdgcn_raw_buffer_load_b128(l3_rsrc, (int)(wi * 4u), 0, 0);
+            const d_u32x4 db = __builtin_amdgcn_raw_buffer_load_b128(l3_rsrc, (int)(wi * 4u + 16u), 0, 0);
+            const uint32_t dc = __builtin_amdgcn_raw_buffer_load_b32(l3_rsrc, (int)(wi * 4u + 32u), 0, 0);
+            const uint32_t d[9] = {da[0], da[1], da[2], da[3], db[0], db[1], db[2], db[3], dc};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) c3w[j] = __builtin_amdgcn_alignbit(d[j + 1], d[j], sh);
+        }
+
+        // ---- clear the compacted arrays (the pads must read as zero) ----
+        for (uint32_t j = lane; j < kDnSlots / 8; j += kWave) reinterpret_cast<d_u32x4 *>(xc)[j] = d_u32x4{0, 0, 0, 0};
+
+        // ---- ranks: first slot of this lane in each array ----
+        const uint32_t cnt1 = (uint32_t)__popc(w1);
+        const uint32_t alive = valid ? 32u - cnt1 : 0u;
+        const uint32_t packed = wave_scan_inclusive(cnt1 | (alive << 16));
+        const uint32_t first1 = (packed & 0xffffu) - cnt1;          // level-1 elements in the lanes below
+        const uint32_t first_a = (packed >> 16) - alive;            // elements above level 1 in the lanes below
+        uint32_t bits2;  // bit j: the lane's j-th element above level 1 is level 2
+        {
+            const uint32_t g = (p0 - q1a) + first_a;
+            const d_u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(b2_rsrc, (int)((g >> 5) * 4u), 0, 0);
+            // alive = 0 shifts the mask out entirely (a 64-bit shift: 32 is a legal count)
+            bits2 = __builtin_amdgcn_alignbit(w[1], w[0], g & 31u) & (uint32_t)(0xFFFFFFFFull >> (32u - alive));
+        }
+        const uint32_t cnt2 = (uint32_t)__popc(bits2);
+        const uint32_t first2 = wave_scan_inclusive(cnt2) - cnt2;
+        const uint32_t first3 = first_a - first2;
+
+        // ---- scatter the lane's 32 activations to their levels' arrays ----
+        {
+            // LDS byte addresses of the lane's next slot in each array; the counters step by two bytes
+            const uint32_t xc_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)xc;
+            uint32_t s1 = xc_addr + 2u * first1, s2 = xc_addr + 2u * (base2 + first2), s3 = xc_addr + 2u * (base3 + first3);
+            uint32_t ja = 0;
+#pragma unroll
+            for (int t = 0; t < 32; ++t) {
+                const uint32_t in1 = (w1 >> t) & 1u;
+                const uint32_t out1 = in1 ^ 1u;
+                const uint32_t in2 = ((bits2 >> ja) & 1u) & out1;
+                const uint32_t in3 = out1 ^ in2;
+                const uint32_t at = in1 ? s1 : (in2 ? s2 : s3);
+                const uint16_t xv = (uint16_t)((t & 1) ? xr[t >> 1] >> 16 : xr[t >> 1]);
+                // lanes past the span scatter zeros behind the last array's entries
+                *reinterpret_cast<__attribute__((address_space(3))) uint16_t *>((uintptr_t)at) = xv;
+                s1 += 2u * in1; s2 += 2u * in2; s3 += 2u * in3; ja += out1;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+
+        // ---- dense passes ----
+        float acc = 0.0f;
+        {   // level 1: pairs of 3-bit codes through the pair table
+            const uint32_t *xp = reinterpret_cast<const uint32_t *>(xc) + (lane * e1) / 2;
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                if (2u * t >= e1) break;  // wave-uniform
+                const int bit = 6 * t, ob = bit & 31, d = bit >> 5;
+                const uint32_t lo = c1w[d];
+                const uint32_t hi = d < 2 ? c1w[d + 1] : 0u;
+                uint32_t a;  // pair index at bits 12..7
+                if (ob > 26) a = __builtin_amdgcn_alignbit(hi, lo, ob - 7);
+                else if (ob >= 7) a = lo >> (ob - 7);
+                else a = lo << (7 - ob);
+                const uint32_t wp = lut[((a & 0x1F80u) | lut_lane) >> 2];
+                acc = dn_dot2(wp, xp[t], acc);
+            }
+        }
+        {   // level 2: pairs of 5-bit codes, dequantised by arithmetic
+            const uint32_t *xp = reinterpret_cast<const uint32_t *>(xc) + (base2 + lane * e2) / 2;
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                if (2u * t >= e2) break;
+                uint32_t c[2];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int bit = 10 * t + 5 * h, ob = bit & 31, d = bit >> 5;
+                    c[h] = ob <= 27 ? (c2w[d] >> ob) & 31u
+                                    : __builtin_amdgcn_alignbit(d < 4 ? c2w[d + 1] : 0u, c2w[d], ob) & 31u;
+                }
+                // (c - 15) * scale as c * scale - 15 * scale: both products and their difference are exact in fp32
+                // (codes and 15 have at most 5 significant bits, the bf16 scale 8), so nothing is rounded twice
+                const uint32_t wp = dn_pack(__fmaf_rn((float)c[0], scale, m15), __fmaf_rn((float)c[1], scale, m15));
+                acc = dn_dot2(wp, xp[t], acc);
+            }
+        }
+        {   // level 3: pairs of bytes
+            const uint32_t *xp = reinterpret_cast<const uint32_t *>(xc) + (base3 + lane * e3) / 2;
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                if (2u * t >= e3) break;
+                const uint32_t word = c3w[t >> 1];
+                const uint32_t ca = (word >> (16 * (t & 1))) & 255u, cb = (word >> (16 * (t & 1) + 8)) & 255u;
+                const uint32_t wp = dn_pack(__fmaf_rn((float)ca, scale, m127), __fmaf_rn((float)cb, scale, m127));
+                acc = dn_dot2(wp, xp[t], acc);
+            }
+        }
+        const float total = dn_wave_sum(acc);
+        if (lane == 63) {
+            if (out_mode == kDnDirect) y[row] = (uint16_t)f32_to_bf16_bits(total);
+            else if (out_mode == kDnAtomic) atomicAdd(y32 + row, total);
+            else ws[(size_t)k * P.out_f + row] = total;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+bool gemv_dense358_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x) {
+    return P.n_levels == 3 && P.bits[0] == 3 && P.bits[1] == 5 && P.bits[2] == 8 && chunk == kFastChunk && m == 1 &&
+           P.in_f % kFastChunk == 0 && P.in_f != 0 && ((uintptr_t)x & 15u) == 0 && ((uintptr_t)P.last & 3u) == 0;
+}
+
+uint32_t gemv_dense358_pieces(const Dev &P) { return (P.in_f / kFastChunk + 3) / 4; }
+
+int launch_gemv_dense358(const Dev &P, const int32_t *prefix, const uint16_t *x, uint16_t *y, float *y32, float *ws,
+                         bool atomic, hipStream_t s) {
+    const uint32_t n_chunks = P.in_f / kFastChunk;
+    const uint32_t spans_per_row = (n_chunks + 3) / 4;
+    const uint32_t n_spans = P.out_f * spans_per_row;
+    if (n_spans == 0) return IXH_OK;
+    // one resident set of workgroups; each wave walks the spans with the stride of the launch
+    static const uint32_t resident = [] {
+        int dev = 0, n_cu = 256, per_cu = 0;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_dense, kWave * kDnWaves, 0) != hipSuccess || per_cu < 1)
+            per_cu = 4;
+        return (uint32_t)n_cu * (uint32_t)per_cu;
+    }();
+    const uint32_t blocks = min(resident, (n_spans + kDnWaves - 1) / kDnWaves);
+    const int out_mode = atomic ? kDnAtomic : (spans_per_row == 1 ? kDnDirect : kDnWorkspace);
+    hipLaunchKernelGGL(k_gemv358_dense, dim3(blocks), dim3(kWave * kDnWaves), 0, s, P, prefix, n_chunks, spans_per_row,
+                       n_spans, x, y, y32, ws, out_mode);
+    if (hipGetLastError() != hipSuccess) return IXH_ELAUNCH;
+    if (out_mode == kDnWorkspace) return launch_reduce_chunks(ws, spans_per_row, 1, P.out_f, y, P.out_f, s);
+    return IXH_OK;
+}
+
+}  // namespace ixh

@@ -14,6 +14,10 @@ int launch_gemv_358(const Dev &P, const int32_t *prefix, uint32_t chunk, const u
 // single-launch row-block kernel (ixh_rows358.hip); IXH_EUNSUPPORTED if the shape does not fit it
 int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
                          int64_t ldy, hipStream_t s);
+// level-by-level kernel for one activation row and mixes with many elements above level 1 (ixh_dense358.hip)
+bool gemv_dense358_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x);
+int launch_gemv_dense358(const Dev &P, const int32_t *prefix, const uint16_t *x, uint16_t *y, float *y32, float *ws,
+                         bool atomic, hipStream_t s);
 int launch_reduce_chunks(const float *ws, uint32_t n_chunks, int m, uint32_t out_f, uint16_t *y, int64_t ldy,
                          hipStream_t s);
 

@@ -203,6 +203,10 @@ def test_gemv_fast_and_general(oracle, dev, kind, shape, m):
                                  (0, in_f, False), (0, 256, True)]:
         y = run_gemv(dp, chunk, x, m, dev, flags=flags, atomic=atomic)
         check_outputs(y, y64, f"{kind} {shape} m={m} flags={flags} chunk={chunk} atomic={atomic}")
+    if m == 1:  # the level-by-level kernel, forced also for the mixes it is not built for
+        for atomic in (False, True):
+            y = run_gemv(dp, 512, x, 1, dev, flags=_lib.IXH_GEMV_DENSE, atomic=atomic)
+            check_outputs(y, y64, f"{kind} {shape} level-by-level kernel atomic={atomic}")
 
 
 @pytest.mark.parametrize("kind", ["student_t", "calibrated_odd_scale", "rare_other", "only_l3"])
@@ -219,7 +223,7 @@ def test_gemv_wide_rows(oracle, dev, kind, shape):
     for m in (1, 2, 4, 7):
         x = activations(m, in_f, seed=m)
         y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
-        for flags in (0, _lib.IXH_GEMV_FORCE_358, _lib.IXH_GEMV_COLUMN_KERNEL):
+        for flags in (0, _lib.IXH_GEMV_FORCE_358, _lib.IXH_GEMV_COLUMN_KERNEL) + ((_lib.IXH_GEMV_DENSE,) if m == 1 else ()):
             check_outputs(run_gemv(dp, 512, x, m, dev, flags=flags), y64, f"{kind} {shape} m={m} flags={flags}")
 
 

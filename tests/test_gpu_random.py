@@ -75,7 +75,7 @@ def test_random_configuration(oracle, dev, seed):
     y64 = oracle.gemm_f64(want_bits.reshape(out_f, in_f), bf16_bits(x))
     chunks = [in_f] + ([512] if in_f % 512 == 0 else [])
     for chunk in chunks:
-        for flags in (0, _lib.IXH_GEMV_STAGED, _lib.IXH_GEMV_FORCE_GENERIC):
+        for flags in (0, _lib.IXH_GEMV_STAGED, _lib.IXH_GEMV_FORCE_GENERIC, _lib.IXH_GEMV_DENSE):
             check_outputs(run_gemv(dp, chunk, x, m, dev, flags=flags), y64, f"{what} chunk={chunk} flags={flags}")
         check_outputs(run_gemv(dp, chunk, x, m, dev, atomic=True), y64, f"{what} chunk={chunk} atomic")
     if in_f % 512 == 0:
