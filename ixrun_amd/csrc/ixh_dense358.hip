@@ -28,6 +28,7 @@ namespace ixh {
 
 typedef uint32_t d_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t d_u32x2 __attribute__((ext_vector_type(2)));
+typedef uint16_t dn_u16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 d_bf16x2 __attribute__((ext_vector_type(2)));
 typedef float d_f32x2 __attribute__((ext_vector_type(2)));
 
@@ -181,22 +182,38 @@ k_gemv358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         const uint32_t first3 = first_a - first2;
 
         // ---- scatter the lane's 32 activations to their levels' arrays ----
+        // Two elements per step, t and t + 16, with their counters in the two halves of one register (packed
+        // 16-bit arithmetic): each half holds "LDS byte address / 2" of the next slot of its level, which fits
+        // 16 bits.  The second half starts where the first one will end: behind the level counts of the lane's
+        // first 16 elements.  in1 / in2 / in3 are 0 or 1 per half; the slot is picked by multiply-add.
         {
-            // LDS byte addresses of the lane's next slot in each array; the counters step by two bytes
-            const uint32_t xc_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)xc;
-            uint32_t s1 = xc_addr + 2u * first1, s2 = xc_addr + 2u * (base2 + first2), s3 = xc_addr + 2u * (base3 + first3);
-            uint32_t ja = 0;
+            const uint32_t xc_half = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)xc >> 1;
+            const uint32_t low1 = (uint32_t)__popc(w1 & 0xffffu);               // level-1 elements among the first 16
+            const uint32_t low_a = valid ? 16u - low1 : 0u;                       // elements above level 1 among them
+            const uint32_t low2 = (uint32_t)__popc(bits2 & ((1u << low_a) - 1u));  // of which level 2
+            const uint32_t a1 = xc_half + first1, a2 = xc_half + base2 + first2, a3 = xc_half + base3 + first3;
+            dn_u16x2 s1 = __builtin_bit_cast(dn_u16x2, a1 | ((a1 + low1) << 16));
+            dn_u16x2 s2 = __builtin_bit_cast(dn_u16x2, a2 | ((a2 + low2) << 16));
+            dn_u16x2 s3 = __builtin_bit_cast(dn_u16x2, a3 | ((a3 + low_a - low2) << 16));
+            // the level-2 flags each half walks through: bits2 from bit 0, and from bit low_a
+            const dn_u16x2 flags = __builtin_bit_cast(dn_u16x2, (bits2 & 0xffffu) | ((bits2 >> low_a) << 16));
+            dn_u16x2 ja = {0, 0};
+            const dn_u16x2 one = {1, 1};
 #pragma unroll
-            for (int t = 0; t < 32; ++t) {
-                const uint32_t in1 = (w1 >> t) & 1u;
-                const uint32_t out1 = in1 ^ 1u;
-                const uint32_t in2 = ((bits2 >> ja) & 1u) & out1;
-                const uint32_t in3 = out1 ^ in2;
-                const uint32_t at = in1 ? s1 : (in2 ? s2 : s3);
-                const uint16_t xv = (uint16_t)((t & 1) ? xr[t >> 1] >> 16 : xr[t >> 1]);
+            for (int t = 0; t < 16; ++t) {
+                const dn_u16x2 in1 = __builtin_bit_cast(dn_u16x2, (w1 >> t) & 0x00010001u);
+                const dn_u16x2 out1 = in1 ^ one;
+                const dn_u16x2 in2 = (flags >> ja) & out1;
+                const dn_u16x2 in3 = out1 ^ in2;
+                const dn_u16x2 at = in1 * (s1 - s3) + (in2 * (s2 - s3) + s3);
+                const uint32_t at32 = __builtin_bit_cast(uint32_t, at);
+                const uint32_t x_lo = xr[t >> 1], x_hi = xr[8 + (t >> 1)];
                 // lanes past the span scatter zeros behind the last array's entries
-                *reinterpret_cast<__attribute__((address_space(3))) uint16_t *>((uintptr_t)at) = xv;
-                s1 += 2u * in1; s2 += 2u * in2; s3 += 2u * in3; ja += out1;
+                *reinterpret_cast<__attribute__((address_space(3))) uint16_t *>((uintptr_t)((at32 & 0xffffu) << 1)) =
+                    (uint16_t)((t & 1) ? x_lo >> 16 : x_lo);
+                *reinterpret_cast<__attribute__((address_space(3))) uint16_t *>((uintptr_t)((at32 >> 16) << 1)) =
+                    (uint16_t)((t & 1) ? x_hi >> 16 : x_hi);
+                s1 += in1; s2 += in2; s3 += in3; ja += out1;
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
