@@ -34,7 +34,7 @@ typedef float d_f32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kDnWaves = 4;                  // waves per workgroup
 constexpr uint32_t kDnSpan = 2048;           // elements per span: four table units of one row
-constexpr uint32_t kDnSlots = kDnSpan + 3 * 128;  // compacted x slots per wave: three arrays, each padded to 64 * E
+constexpr uint32_t kDnSlots = kDnSpan + 3 * 256;  // compacted x slots per wave: three arrays, each padded to 64 * E
 constexpr uint32_t kDnLutBytes = 64 * 32 * 4;     // pair table: 64 code pairs x 32 lane copies
 
 enum : int { kDnDirect = 0, kDnAtomic = 1, kDnWorkspace = 2 };
@@ -105,8 +105,9 @@ k_gemv358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         const uint32_t q1a = (uint32_t)prefix[u0], q1b = (uint32_t)prefix[u0 + nb];
         const uint32_t q2a = (uint32_t)prefix[entries + u0], q2b = (uint32_t)prefix[entries + u0 + nb];
         const uint32_t n1 = q1b - q1a, n2 = q2b - q2a, n3 = n_el - n1 - n2;
-        // codes per lane in the dense passes (even), and the padded sizes of the compacted arrays
-        const uint32_t e1 = 2 * ((n1 + 127) / 128), e2 = 2 * ((n2 + 127) / 128), e3 = 2 * ((n3 + 127) / 128);
+        // codes per lane in the dense passes (a multiple of four: the passes run in groups of two pairs), and the
+        // padded sizes of the compacted arrays
+        const uint32_t e1 = 4 * ((n1 + 255) / 256), e2 = 4 * ((n2 + 255) / 256), e3 = 4 * ((n3 + 255) / 256);
         const uint32_t base2 = 64 * e1, base3 = base2 + 64 * e2;
 
         // ---- loads whose addresses follow from the table alone ----
@@ -221,49 +222,66 @@ k_gemv358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
         // ---- dense passes ----
         float acc = 0.0f;
+        // Each pass runs in groups of two pairs; a group is entered only if the level has codes for it.  (The empty
+        // asm statements keep the group tests branches: as selects, all 24 groups would run for every span.)
         {   // level 1: pairs of 3-bit codes through the pair table
             const uint32_t *xp = reinterpret_cast<const uint32_t *>(xc) + (lane * e1) / 2;
 #pragma unroll
-            for (int t = 0; t < 16; ++t) {
-                if (2u * t >= e1) break;  // wave-uniform
-                const int bit = 6 * t, ob = bit & 31, d = bit >> 5;
-                const uint32_t lo = c1w[d];
-                const uint32_t hi = d < 2 ? c1w[d + 1] : 0u;
-                uint32_t a;  // pair index at bits 12..7
-                if (ob > 26) a = __builtin_amdgcn_alignbit(hi, lo, ob - 7);
-                else if (ob >= 7) a = lo >> (ob - 7);
-                else a = lo << (7 - ob);
-                const uint32_t wp = lut[((a & 0x1F80u) | lut_lane) >> 2];
-                acc = dn_dot2(wp, xp[t], acc);
+            for (int g = 0; g < 8; ++g) {
+                if (e1 > 4u * g) {
+                    asm volatile("");
+#pragma unroll
+                    for (int t = 2 * g; t < 2 * g + 2; ++t) {
+                        const int bit = 6 * t, ob = bit & 31, d = bit >> 5;
+                        const uint32_t lo = c1w[d];
+                        const uint32_t hi = d < 2 ? c1w[d + 1] : 0u;
+                        uint32_t a;  // pair index at bits 12..7
+                        if (ob > 26) a = __builtin_amdgcn_alignbit(hi, lo, ob - 7);
+                        else if (ob >= 7) a = lo >> (ob - 7);
+                        else a = lo << (7 - ob);
+                        const uint32_t wp = lut[((a & 0x1F80u) | lut_lane) >> 2];
+                        acc = dn_dot2(wp, xp[t], acc);
+                    }
+                }
             }
         }
         {   // level 2: pairs of 5-bit codes, dequantised by arithmetic
             const uint32_t *xp = reinterpret_cast<const uint32_t *>(xc) + (base2 + lane * e2) / 2;
 #pragma unroll
-            for (int t = 0; t < 16; ++t) {
-                if (2u * t >= e2) break;
-                uint32_t c[2];
+            for (int g = 0; g < 8; ++g) {
+                if (e2 > 4u * g) {
+                    asm volatile("");
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const int bit = 10 * t + 5 * h, ob = bit & 31, d = bit >> 5;
-                    c[h] = ob <= 27 ? (c2w[d] >> ob) & 31u
-                                    : __builtin_amdgcn_alignbit(d < 4 ? c2w[d + 1] : 0u, c2w[d], ob) & 31u;
+                    for (int t = 2 * g; t < 2 * g + 2; ++t) {
+                        uint32_t c[2];
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const int bit = 10 * t + 5 * h, ob = bit & 31, d = bit >> 5;
+                            c[h] = ob <= 27 ? (c2w[d] >> ob) & 31u
+                                            : __builtin_amdgcn_alignbit(d < 4 ? c2w[d + 1] : 0u, c2w[d], ob) & 31u;
+                        }
+                        // (c - 15) * scale as c * scale - 15 * scale: both products and their difference are exact in
+                        // fp32 (codes and 15 have at most 5 significant bits, the bf16 scale 8): nothing is rounded twice
+                        const uint32_t wp = dn_pack(__fmaf_rn((float)c[0], scale, m15), __fmaf_rn((float)c[1], scale, m15));
+                        acc = dn_dot2(wp, xp[t], acc);
+                    }
                 }
-                // (c - 15) * scale as c * scale - 15 * scale: both products and their difference are exact in fp32
-                // (codes and 15 have at most 5 significant bits, the bf16 scale 8), so nothing is rounded twice
-                const uint32_t wp = dn_pack(__fmaf_rn((float)c[0], scale, m15), __fmaf_rn((float)c[1], scale, m15));
-                acc = dn_dot2(wp, xp[t], acc);
             }
         }
         {   // level 3: pairs of bytes
             const uint32_t *xp = reinterpret_cast<const uint32_t *>(xc) + (base3 + lane * e3) / 2;
 #pragma unroll
-            for (int t = 0; t < 16; ++t) {
-                if (2u * t >= e3) break;
-                const uint32_t word = c3w[t >> 1];
-                const uint32_t ca = (word >> (16 * (t & 1))) & 255u, cb = (word >> (16 * (t & 1) + 8)) & 255u;
-                const uint32_t wp = dn_pack(__fmaf_rn((float)ca, scale, m127), __fmaf_rn((float)cb, scale, m127));
-                acc = dn_dot2(wp, xp[t], acc);
+            for (int g = 0; g < 8; ++g) {
+                if (e3 > 4u * g) {
+                    asm volatile("");
+#pragma unroll
+                    for (int t = 2 * g; t < 2 * g + 2; ++t) {
+                        const uint32_t word = c3w[t >> 1];
+                        const uint32_t ca = (word >> (16 * (t & 1))) & 255u, cb = (word >> (16 * (t & 1) + 8)) & 255u;
+                        const uint32_t wp = dn_pack(__fmaf_rn((float)ca, scale, m127), __fmaf_rn((float)cb, scale, m127));
+                        acc = dn_dot2(wp, xp[t], acc);
+                    }
+                }
             }
         }
         const float total = dn_wave_sum(acc);
