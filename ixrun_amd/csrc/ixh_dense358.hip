@@ -65,7 +65,7 @@ __device__ __forceinline__ float dn_dot2(uint32_t w, uint32_t x, float acc) {
 __global__ void __launch_bounds__(kWave *kDnWaves)
 k_gemv358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t spans_per_row, uint32_t n_spans,
                 const uint16_t *__restrict__ x, uint16_t *__restrict__ y,
-                float *__restrict__ y32, float *__restrict__ ws, int out_mode) {
+                float *__restrict__ y32, float *__restrict__ ws, int out_mode, bool by_rows) {
     __shared__ __attribute__((aligned(16))) uint32_t lut[kDnLutBytes / 4];
     __shared__ __attribute__((aligned(16))) uint16_t xc_all[kDnWaves][kDnSlots];
     const uint32_t tid = threadIdx.x, lane = tid & 63;
@@ -94,11 +94,17 @@ k_gemv358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     const __amdgpu_buffer_rsrc_t b2_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[1], 0, (int)(P.bm_words[1] * 4u), 0x00020000);
 
-    // spans are dealt to the waves of the launch in turn: with a launch that is resident as a whole, every wave
-    // gets the same number of spans (give or take one)
+    // Work is dealt to the waves of the launch in turn; the launch is resident as a whole, so every wave gets the
+    // same number of items (give or take one).  An item is a whole row (its spans are summed in the wave and the
+    // result leaves as it is) or, when rows would not spread evenly, one span (partial sums meet in the workspace).
     const uint32_t n_waves = gridDim.x * kDnWaves;
-    for (uint32_t s = blockIdx.x * kDnWaves + wave; s < n_spans; s += n_waves) {
-        const uint32_t row = s / spans_per_row, k = s - row * spans_per_row;
+    const uint32_t n_items = by_rows ? P.out_f : n_spans;
+    for (uint32_t item = blockIdx.x * kDnWaves + wave; item < n_items; item += n_waves) {
+      const uint32_t row = by_rows ? item : item / spans_per_row;
+      const uint32_t k_first = by_rows ? 0u : item - row * spans_per_row;
+      const uint32_t k_end = by_rows ? spans_per_row : k_first + 1u;
+      float row_total = 0.0f;  // meaningful in lane 63
+      for (uint32_t k = k_first; k < k_end; ++k) {
         const uint32_t c0 = 4 * k, nb = min(4u, n_chunks - c0);
         const uint32_t u0 = row * n_chunks + c0;
         const uint32_t n_el = nb * kFastChunk, p0 = u0 * kFastChunk;
@@ -284,14 +290,15 @@ k_gemv358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
                 }
             }
         }
-        const float total = dn_wave_sum(acc);
-        if (lane == 63) {
-            if (out_mode == kDnDirect) y[row] = (uint16_t)f32_to_bf16_bits(total);
-            else if (out_mode == kDnAtomic) atomicAdd(y32 + row, total);
-            else ws[(size_t)k * P.out_f + row] = total;
-        }
+        row_total += dn_wave_sum(acc);
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
+      }
+      if (lane == 63) {
+          if (out_mode == kDnDirect) y[row] = (uint16_t)f32_to_bf16_bits(row_total);
+          else if (out_mode == kDnAtomic) atomicAdd(y32 + row, row_total);
+          else ws[(size_t)k_first * P.out_f + row] = row_total;
+      }
     }
 }
 
@@ -316,10 +323,16 @@ int launch_gemv_dense358(const Dev &P, const int32_t *prefix, const uint16_t *x,
             per_cu = 4;
         return (uint32_t)n_cu * (uint32_t)per_cu;
     }();
-    const uint32_t blocks = min(resident, (n_spans + kDnWaves - 1) / kDnWaves);
-    const int out_mode = atomic ? kDnAtomic : (spans_per_row == 1 ? kDnDirect : kDnWorkspace);
+    // Whole rows per wave when they spread over the resident waves within 12 %: one launch, no workspace, each
+    // output summed in one register.  Otherwise spans are dealt out and a second kernel adds a row's partial sums.
+    const uint32_t waves_res = resident * kDnWaves;
+    const uint32_t rounds = (P.out_f + waves_res - 1) / waves_res;
+    const bool by_rows = spans_per_row == 1 || (uint64_t)rounds * waves_res * 100u <= (uint64_t)P.out_f * 112u;
+    const uint32_t n_items = by_rows ? P.out_f : n_spans;
+    const uint32_t blocks = min(resident, (n_items + kDnWaves - 1) / kDnWaves);
+    const int out_mode = atomic ? kDnAtomic : (by_rows ? kDnDirect : kDnWorkspace);
     hipLaunchKernelGGL(k_gemv358_dense, dim3(blocks), dim3(kWave * kDnWaves), 0, s, P, prefix, n_chunks, spans_per_row,
-                       n_spans, x, y, y32, ws, out_mode);
+                       n_spans, x, y, y32, ws, out_mode, by_rows);
     if (hipGetLastError() != hipSuccess) return IXH_ELAUNCH;
     if (out_mode == kDnWorkspace) return launch_reduce_chunks(ws, spans_per_row, 1, P.out_f, y, P.out_f, s);
     return IXH_OK;
