@@ -33,7 +33,7 @@ MFMA_BF16_PEAK = 2.5e15  # FLOP/s dense bf16, MI355X published
 # x 2.0 and x 1.0); the counter summaries are kept under profiles/.  Workloads without a counter run report null.
 MEASURED_TRAFFIC_BYTES = {
     "down_proj_5120x17408_m1_student_t": 23078.5 * 2.0 * 1024 + 16.0 * 1024,
-    "down_proj_5120x17408_m1_calibrated": 33545.4 * 2.0 * 1024 + 640.0 * 1024,
+    "down_proj_5120x17408_m1_calibrated": 33662.0 * 2.0 * 1024 + 40.0 * 1024,
     "prefill_5120x5120_m512_five_level": 50297.9 * 2.0 * 1024 + 30720.0 * 1024,
     "attn_proj_5120x5120_m1_student_t": 7118.0 * 2.0 * 1024 + 16.0 * 1024,
     "gate_up_17408x5120_m4_student_t": 23193.0 * 2.0 * 1024 + 181.0 * 1024,
