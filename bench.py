@@ -38,7 +38,8 @@ MEASURED_TRAFFIC_BYTES = {
     "attn_proj_5120x5120_m1_student_t": 7118.0 * 2.0 * 1024 + 16.0 * 1024,
     "gate_up_17408x5120_m4_student_t": 23193.0 * 2.0 * 1024 + 181.0 * 1024,
     "decode_5120x17408_student_t": 25672.0 * 2.0 * 1024 + 174080.0 * 1024,
-    "decode_gs_5120x17408_student_t": 33772.0 * 2.0 * 1024 + 174080.0 * 1024,
+    "decode_5120x17408_calibrated": 36308.0 * 2.0 * 1024 + 174080.0 * 1024,
+    "decode_gs_5120x17408_student_t": 33559.0 * 2.0 * 1024 + 174080.0 * 1024,
     # all kernels of one encode step together (absmax, count, scans, clear, pack)
     "encode_5120x17408_student_t": (87053 + 87092 + 1402 + 15 + 92442) * 2.0 * 1024 + (32 + 2040 + 1362 + 32694 + 63405) * 1024,
 }

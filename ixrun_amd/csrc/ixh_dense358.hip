@@ -6,28 +6,30 @@
 //     sum_k w_k x_k = sum_{k in level 1} w_k x_k + sum_{k in level 2} w_k x_k + sum_{k in level 3} w_k x_k
 // and what depends on the bitmaps is moved to the activations: the x values of a span are scattered ("compacted")
 // into three arrays in LDS, one per level, in the order of that level's codes.  Scattering costs an LDS write per
-// weight and a dozen integer instructions (two bit tests, three running counters, a select); the three dense passes
-// then cost about one instruction per weight.
+// weight and about nine integer instructions (two elements per step, with the running slot addresses in packed
+// 16-bit halves); the three dense passes then cost about one instruction per weight.
 //
 // A wave takes spans of up to 2048 consecutive elements of one weight row (four 512-element table units).  The
 // rank table gives the span's first code in every stream and its level counts.  Lane l owns bitmap word l (32
 // elements, 16 x pairs in registers): popcount + wave prefix sums give the lane's first slot in each compacted array
 // (bitmap 1 is read at the lane's first element not in level 1).  The dense passes split each level's codes evenly over
-// the 64 lanes (an even number E of codes per lane, wave-uniform), read them with plain loads at addresses that
-// depend only on the table, and meet the compacted x pairs in v_dot2_f32_bf16: level 1 through the table of
+// the 64 lanes (E codes per lane, a multiple of four, wave-uniform), read them through buffer descriptors at addresses
+// that depend only on the table, and meet the compacted x pairs in v_dot2_f32_bf16: level 1 through the table of
 // dequantised pairs (two 3-bit codes -> one LDS read), levels 2 and 3 by arithmetic, each weight rounded to bf16 as
 // the reference's decoder does (ixrun/triton_kernels.py:168-177).  The array of each level is padded with zeros up
 // to 64 * E slots, so codes read past a level's end meet a zero.
 //
-// No LDS-DMA and no hand-counted waits here: the kernel is bound by instruction issue (about 650 vector instructions
-// per 2048 weights), six waves per SIMD cover the load latency.  Partial sums of the spans of a row are combined
-// through the workspace in span order (or added to y32 with atomics).
+// No LDS-DMA and no hand-counted waits here: the kernel is bound by instruction issue (about 520 vector instructions
+// per 2048 weights), five waves per SIMD cover the load latency.  A wave sums whole rows when rows spread evenly over
+// the launch; otherwise partial sums of the spans of a row are combined through the workspace in span order (or
+// added to y32 with atomics).
 #include "ixh_fast358.h"
 
 namespace ixh {
 
 typedef uint32_t d_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t d_u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t d_u32x3 __attribute__((ext_vector_type(3)));
 typedef uint16_t dn_u16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 d_bf16x2 __attribute__((ext_vector_type(2)));
 typedef float d_f32x2 __attribute__((ext_vector_type(2)));
@@ -35,6 +37,7 @@ typedef float d_f32x2 __attribute__((ext_vector_type(2)));
 constexpr int kDnWaves = 4;                  // waves per workgroup
 constexpr uint32_t kDnSpan = 2048;           // elements per span: four table units of one row
 constexpr uint32_t kDnSlots = kDnSpan + 3 * 256;  // compacted x slots per wave: three arrays, each padded to 64 * E
+static_assert(kDnSlots * 2 >= 64 * 80 && (kDnSlots * 2) % 16 == 0, "the decode kernel re-uses a wave's slots as 64 rows of 80 bytes");
 constexpr uint32_t kDnLutBytes = 64 * 32 * 4;     // pair table: 64 code pairs x 32 lane copies
 
 enum : int { kDnDirect = 0, kDnAtomic = 1, kDnWorkspace = 2 };
@@ -300,6 +303,303 @@ k_gemv358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
           else ws[(size_t)k_first * P.out_f + row] = row_total;
       }
     }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Full decode to bf16 by the same route, for dense mixes: the codes of each level are dequantised where they lie
+// (dense, fixed positions) into three LDS arrays of weights, and every lane then gathers the weights of its 32
+// positions from the slots that the scatter above would have written to.  Spans are 2048 consecutive flat elements
+// (rows play no part in a decode); the last span and the last lane may be partial.
+// A lane's rows of the three arrays hold a number of codes that is twice an odd number, and the passes work in groups
+// of two pairs, so a lane's last group decodes one pair that is the next lane's first: both write the same value.
+// With group scales (GS: one fp16 scale per 2^group_shift >= 32 consecutive elements, so one per lane) the arrays
+// hold the integer values as bf16, exact, and the lane multiplies what it gathered by its scale.
+// ---------------------------------------------------------------------------------------------------------------
+template <bool GS>
+__global__ void __launch_bounds__(kWave *kDnWaves)
+k_decode358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, uint32_t n_spans, uint16_t *__restrict__ out,
+                  const uint16_t *__restrict__ group_scales, uint32_t group_shift) {
+    __shared__ __attribute__((aligned(16))) uint32_t lut[kDnLutBytes / 4];
+    __shared__ __attribute__((aligned(16))) uint16_t wc_all[kDnWaves][kDnSlots];
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const float scale = GS ? 1.0f : bf16_bits_to_f32(*P.scale);
+    const float m15 = -15.0f * scale, m127 = -127.0f * scale;
+    for (uint32_t e = tid; e < 64 * 32; e += kWave * kDnWaves) {
+        const uint32_t idx = e >> 5;
+        lut[e] = dn_pack(dequant((int)(idx & 7u) - 3, scale), dequant((int)(idx >> 3) - 3, scale));
+    }
+    __syncthreads();
+
+    uint16_t *const wc = wc_all[wave];
+    uint32_t *const wc32 = reinterpret_cast<uint32_t *>(wc);
+    const uint32_t lut_lane = (lane & 31u) << 2;
+    const uint32_t entries = n_units + 1;
+    const uint32_t *__restrict__ b1 = P.bm[0];
+    const __amdgpu_buffer_rsrc_t l1_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[0], 0, (int)(P.st_words[0] * 4u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t l2_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[1], 0, (int)(P.st_words[1] * 4u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t l3_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.last, 0, (int)((P.last_bytes + 3u) & ~3u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t b2_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[1], 0, (int)(P.bm_words[1] * 4u), 0x00020000);
+
+    // What a span needs from memory before any arithmetic: four table entries (scalars), the lane's bitmap word and
+    // its window of each code stream.  They are fetched one span ahead (the table entries two), so that a wave's
+    // chain table -> windows -> arithmetic does not wait on memory twice per span.
+    struct Ranks { uint32_t q1a, q1b, q2a, q2b; };
+    struct Loads { uint32_t w1; d_u32x4 l1a; uint32_t l1b; d_u32x4 l2a; d_u32x3 l2b; d_u32x4 l3a, l3b; d_u32x2 l3c; uint32_t group_scale; };
+    struct Shape { uint32_t p0, n_el, e1, e2, e3; };
+    // Codes of a level per lane: enough for all of them, and twice an odd number, so that the lanes' rows of the LDS
+    // array start an odd number of dwords apart (no two of 32 neighbouring lanes on one bank).  2, 6, ... 34.
+    auto codes_per_lane = [](uint32_t n) { return (((n + 63) / 64 + 1) & ~3u) + 2; };
+    auto table_of = [&](uint32_t s) {
+        const uint32_t u0 = 4 * s, u1 = min(u0 + 4, n_units);
+        return Ranks{(uint32_t)prefix[u0], (uint32_t)prefix[u1], (uint32_t)prefix[entries + u0], (uint32_t)prefix[entries + u1]};
+    };
+    auto shape_of = [&](uint32_t s, const Ranks &q) {
+        const uint32_t p0 = 4 * s * kFastChunk, n_el = min(kDnSpan, P.n - p0);
+        const uint32_t n1 = q.q1b - q.q1a, n2 = q.q2b - q.q2a, n3 = n_el - n1 - n2;
+        return Shape{p0, n_el, codes_per_lane(n1), codes_per_lane(n2), codes_per_lane(n3)};
+    };
+    auto fetch = [&](uint32_t s, const Ranks &q) {
+        const Shape g = shape_of(s, q);
+        Loads r;
+        r.w1 = 32 * lane < g.n_el ? b1[(g.p0 >> 5) + lane] : 0u;
+        r.group_scale = GS && 32 * lane < g.n_el ? group_scales[(g.p0 + 32 * lane) >> group_shift] : 0u;
+        {
+            const uint64_t bit = (uint64_t)(q.q1a + lane * g.e1) * 3u;
+            const uint32_t at = (uint32_t)(bit >> 5) * 4u;
+            r.l1a = __builtin_amdgcn_raw_buffer_load_b128(l1_rsrc, (int)at, 0, 0);
+            r.l1b = __builtin_amdgcn_raw_buffer_load_b32(l1_rsrc, (int)(at + 16u), 0, 0);
+        }
+        {
+            const uint64_t bit = (uint64_t)(q.q2a + lane * g.e2) * 5u;
+            const uint32_t at = (uint32_t)(bit >> 5) * 4u;
+            r.l2a = __builtin_amdgcn_raw_buffer_load_b128(l2_rsrc, (int)at, 0, 0);
+            r.l2b = __builtin_amdgcn_raw_buffer_load_b96(l2_rsrc, (int)(at + 16u), 0, 0);
+        }
+        {
+            const uint32_t at = (((g.p0 - q.q1a - q.q2a) + lane * g.e3) >> 2) * 4u;
+            r.l3a = __builtin_amdgcn_raw_buffer_load_b128(l3_rsrc, (int)at, 0, 0);
+            r.l3b = __builtin_amdgcn_raw_buffer_load_b128(l3_rsrc, (int)(at + 16u), 0, 0);
+            r.l3c = __builtin_amdgcn_raw_buffer_load_b64(l3_rsrc, (int)(at + 32u), 0, 0);
+        }
+        return r;
+    };
+
+    const uint32_t n_waves = gridDim.x * kDnWaves;
+    uint32_t s = blockIdx.x * kDnWaves + wave;
+    if (s >= n_spans) return;
+    const uint32_t last_span = n_spans - 1;
+    Ranks q_now = table_of(s);
+    Loads in_now = fetch(s, q_now);
+    Ranks q_next = table_of(min(s + n_waves, last_span));
+    for (; s < n_spans; s += n_waves) {
+        // the span after this one (or, at the end, the last span once more: loads that nobody uses)
+        const Loads in_next = fetch(min(s + n_waves, last_span), q_next);
+        const Ranks q_after = table_of(min(s + 2 * n_waves, last_span));
+        const Shape g = shape_of(s, q_now);
+        const uint32_t p0 = g.p0, n_el = g.n_el, e1 = g.e1, e2 = g.e2, e3 = g.e3;
+        const uint32_t q1a = q_now.q1a, q2a = q_now.q2a;
+        const uint32_t base2 = 64 * e1, base3 = base2 + 64 * e2;
+
+        // positions of this lane inside the span, and its bitmap word
+        const uint32_t n_here = 32 * lane < n_el ? min(32u, n_el - 32 * lane) : 0u;
+        const uint32_t here = (uint32_t)(0xFFFFFFFFull >> (32u - n_here));  // n_here = 0 gives an empty mask
+        const uint32_t w1 = in_now.w1 & here;
+
+        // ---- dequantise every level where its codes lie ----
+        {
+            const uint32_t sh = (uint32_t)((uint64_t)(q1a + lane * e1) * 3u) & 31u;
+            const d_u32x4 d = in_now.l1a;
+            const uint32_t c1w[4] = {__builtin_amdgcn_alignbit(d[1], d[0], sh), __builtin_amdgcn_alignbit(d[2], d[1], sh),
+                                     __builtin_amdgcn_alignbit(d[3], d[2], sh), __builtin_amdgcn_alignbit(in_now.l1b, d[3], sh)};
+            uint32_t *dst = wc32 + (lane * e1) / 2;
+#pragma unroll
+            for (int g = 0; g < 9; ++g) {
+                if (e1 > 4u * g) {
+                    asm volatile("");
+#pragma unroll
+                    for (int t = 2 * g; t < 2 * g + 2; ++t) {
+                        const int bt = 6 * t, ob = bt & 31, dd = bt >> 5;
+                        const uint32_t lo = c1w[dd];
+                        const uint32_t hi = dd < 3 ? c1w[dd + 1] : 0u;
+                        uint32_t a;
+                        if (ob > 26) a = __builtin_amdgcn_alignbit(hi, lo, ob - 7);
+                        else if (ob >= 7) a = lo >> (ob - 7);
+                        else a = lo << (7 - ob);
+                        dst[t] = lut[((a & 0x1F80u) | lut_lane) >> 2];
+                    }
+                }
+            }
+        }
+        {
+            const uint32_t sh = (uint32_t)((uint64_t)(q2a + lane * e2) * 5u) & 31u;
+            const uint32_t d[7] = {in_now.l2a[0], in_now.l2a[1], in_now.l2a[2], in_now.l2a[3],
+                                   in_now.l2b[0], in_now.l2b[1], in_now.l2b[2]};
+            uint32_t c2w[6];
+#pragma unroll
+            for (int j = 0; j < 6; ++j) c2w[j] = __builtin_amdgcn_alignbit(d[j + 1], d[j], sh);
+            uint32_t *dst = wc32 + (base2 + lane * e2) / 2;
+#pragma unroll
+            for (int g = 0; g < 9; ++g) {
+                if (e2 > 4u * g) {
+                    asm volatile("");
+#pragma unroll
+                    for (int t = 2 * g; t < 2 * g + 2; ++t) {
+                        uint32_t c[2];
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const int bt = 10 * t + 5 * h, ob = bt & 31, dd = bt >> 5;
+                            c[h] = ob <= 27 ? (c2w[dd] >> ob) & 31u
+                                            : __builtin_amdgcn_alignbit(dd < 5 ? c2w[dd + 1] : 0u, c2w[dd], ob) & 31u;
+                        }
+                        dst[t] = dn_pack(__fmaf_rn((float)c[0], scale, m15), __fmaf_rn((float)c[1], scale, m15));
+                    }
+                }
+            }
+        }
+        {
+            const uint32_t sh = (((p0 - q1a - q2a) + lane * e3) & 3u) * 8u;
+            const uint32_t d[10] = {in_now.l3a[0], in_now.l3a[1], in_now.l3a[2], in_now.l3a[3], in_now.l3b[0],
+                                    in_now.l3b[1], in_now.l3b[2], in_now.l3b[3], in_now.l3c[0], in_now.l3c[1]};
+            uint32_t c3w[9];
+#pragma unroll
+            for (int j = 0; j < 9; ++j) c3w[j] = __builtin_amdgcn_alignbit(d[j + 1], d[j], sh);
+            uint32_t *dst = wc32 + (base3 + lane * e3) / 2;
+#pragma unroll
+            for (int g = 0; g < 9; ++g) {
+                if (e3 > 4u * g) {
+                    asm volatile("");
+#pragma unroll
+                    for (int t = 2 * g; t < 2 * g + 2; ++t) {
+                        const uint32_t word = c3w[t >> 1];
+                        const uint32_t ca = (word >> (16 * (t & 1))) & 255u, cb = (word >> (16 * (t & 1) + 8)) & 255u;
+                        dst[t] = dn_pack(__fmaf_rn((float)ca, scale, m127), __fmaf_rn((float)cb, scale, m127));
+                    }
+                }
+            }
+        }
+
+        // ---- ranks: first slot of this lane in each array ----
+        const uint32_t cnt1 = (uint32_t)__popc(w1);
+        const uint32_t alive = n_here - cnt1;
+        const uint32_t packed = wave_scan_inclusive(cnt1 | (alive << 16));
+        const uint32_t first1 = (packed & 0xffffu) - cnt1;
+        const uint32_t first_a = (packed >> 16) - alive;
+        uint32_t bits2;
+        {
+            const uint32_t g = (p0 - q1a) + first_a;
+            const d_u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(b2_rsrc, (int)((g >> 5) * 4u), 0, 0);
+            bits2 = __builtin_amdgcn_alignbit(w[1], w[0], g & 31u) & (uint32_t)(0xFFFFFFFFull >> (32u - alive));
+        }
+        const uint32_t cnt2 = (uint32_t)__popc(bits2);
+        const uint32_t first2 = wave_scan_inclusive(cnt2) - cnt2;
+        const uint32_t first3 = first_a - first2;
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+
+        // ---- gather: the same walk as the scatter of the product kernel, reading instead of writing ----
+        uint32_t o[16];  // the lane's 32 weights, in position order
+        {
+            const uint32_t wc_half = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)wc >> 1;
+            const uint32_t low1 = (uint32_t)__popc(w1 & 0xffffu);
+            const uint32_t low_a = min(n_here, 16u) - low1;
+            const uint32_t low2 = (uint32_t)__popc(bits2 & ((1u << low_a) - 1u));
+            const uint32_t a1 = wc_half + first1, a2 = wc_half + base2 + first2, a3 = wc_half + base3 + first3;
+            dn_u16x2 s1 = __builtin_bit_cast(dn_u16x2, a1 | ((a1 + low1) << 16));
+            dn_u16x2 s2 = __builtin_bit_cast(dn_u16x2, a2 | ((a2 + low2) << 16));
+            dn_u16x2 s3 = __builtin_bit_cast(dn_u16x2, a3 | ((a3 + low_a - low2) << 16));
+            const dn_u16x2 flags = __builtin_bit_cast(dn_u16x2, (bits2 & 0xffffu) | ((bits2 >> low_a) << 16));
+            dn_u16x2 ja = {0, 0};
+            const dn_u16x2 one = {1, 1};
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const dn_u16x2 in1 = __builtin_bit_cast(dn_u16x2, (w1 >> t) & 0x00010001u);
+                const dn_u16x2 out1 = in1 ^ one;
+                const dn_u16x2 in2 = (flags >> ja) & out1;
+                const dn_u16x2 in3 = out1 ^ in2;
+                const dn_u16x2 at = in1 * (s1 - s3) + (in2 * (s2 - s3) + s3);
+                const uint32_t at32 = __builtin_bit_cast(uint32_t, at);
+                // positions past the end of the tensor walk on through the last array; what they read is not stored
+                const uint32_t va = *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>((uintptr_t)((at32 & 0xffffu) << 1));
+                const uint32_t vb = *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>((uintptr_t)((at32 >> 16) << 1));
+                if (t & 1) {
+                    o[t >> 1] |= va << 16;
+                    o[8 + (t >> 1)] |= vb << 16;
+                } else {
+                    o[t >> 1] = va;
+                    o[8 + (t >> 1)] = vb;
+                }
+                s1 += in1; s2 += in2; s3 += in3; ja += out1;
+            }
+        }
+        uint16_t *dst = out + (size_t)p0 + 32 * lane;
+        if (GS) {
+            const float sc = fp16_bits_to_f32((uint16_t)in_now.group_scale);
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+                o[j] = dn_pack(__uint_as_float(o[j] << 16) * sc, __uint_as_float(o[j] & 0xffff0000u) * sc);
+        }
+        if (n_el == kDnSpan) {
+            // Whole span: through LDS once more, so that a store instruction writes 1 KB of consecutive bytes
+            // (lane rows 80 bytes apart keep the 16-byte accesses of eight neighbouring lanes on distinct banks).
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            d_u32x4 *const rows = reinterpret_cast<d_u32x4 *>(wc);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) rows[lane * 5 + j] = d_u32x4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            d_u32x4 *const line = reinterpret_cast<d_u32x4 *>(out + (size_t)p0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) line[64 * j + lane] = rows[(16 * j + (lane >> 2)) * 5 + (lane & 3u)];
+        } else if (n_here == 32) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                reinterpret_cast<d_u32x4 *>(dst)[j] = d_u32x4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
+        } else {
+            for (uint32_t t = 0; t < n_here; ++t) {
+                uint32_t v = 0;
+#pragma unroll
+                for (int j = 0; j < 16; ++j) v = (t >> 1) == (uint32_t)j ? o[j] : v;
+                dst[t] = (uint16_t)((t & 1u) ? v >> 16 : v);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        in_now = in_next;
+        q_now = q_next;
+        q_next = q_after;
+    }
+}
+
+bool decode_dense358_supports(const Dev &P, uint32_t chunk, const int8_t *o8, const uint16_t *o16, GroupScales gs) {
+    if (gs.fp16 && (gs.group < 32 || (gs.group & (gs.group - 1)) != 0)) return false;  // one scale per lane, by a shift
+    return P.n_levels == 3 && P.bits[0] == 3 && P.bits[1] == 5 && P.bits[2] == 8 && chunk == kFastChunk && !o8 && o16 &&
+           ((uintptr_t)o16 & 15u) == 0 && ((uintptr_t)P.last & 3u) == 0 && P.n != 0;
+}
+
+int launch_decode_dense358(const Dev &P, const int32_t *prefix, uint16_t *o16, GroupScales gs, hipStream_t s) {
+    const uint32_t n_units = (P.n + kFastChunk - 1) / kFastChunk;
+    const uint32_t n_spans = (n_units + 3) / 4;
+    static const uint32_t resident = [] {
+        int dev = 0, n_cu = 256, per_cu = 0;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_decode358_dense<true>, kWave * kDnWaves, 0) != hipSuccess || per_cu < 1)
+            per_cu = 4;
+        return (uint32_t)n_cu * (uint32_t)per_cu;
+    }();
+    const uint32_t blocks = min(resident, (n_spans + kDnWaves - 1) / kDnWaves);
+    if (gs.fp16)
+        hipLaunchKernelGGL(k_decode358_dense<true>, dim3(blocks), dim3(kWave * kDnWaves), 0, s, P, prefix, n_units, n_spans, o16,
+                           gs.fp16, (uint32_t)__builtin_ctz(gs.group));
+    else
+        hipLaunchKernelGGL(k_decode358_dense<false>, dim3(blocks), dim3(kWave * kDnWaves), 0, s, P, prefix, n_units, n_spans, o16,
+                           (const uint16_t *)nullptr, 0u);
+    return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }
 
 bool gemv_dense358_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x) {

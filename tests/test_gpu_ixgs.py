@@ -32,10 +32,19 @@ def packed_from_ints(oracle, q, scales, out_f, in_f, group):
             "counts": e["counts"], "total_bytes": 0, "bits_per_weight": 0.0, "compression_vs_bf16": 0.0}
 
 
+@pytest.fixture(params=["by_mix", "0", "1"])
+def decoder(request, monkeypatch):
+    """Which of the two unit-512 decoders runs: chosen by the mix of tiers, or forced ("1": level by level where the
+    group size allows it, "0": the one that stages the streams)."""
+    if request.param != "by_mix":
+        monkeypatch.setenv("IXH_DECODE_DENSE", request.param)
+    return request.param
+
+
 @pytest.mark.parametrize("shape,group", [((512, 256), 64), ((1000, 640), 64), ((1, 1), 64), ((3, 11), 64), ((33, 1000), 64),
                                          ((300, 1031), 64), ((256, 4608), 64), ((128, 512), 8), ((128, 512), 32),
                                          ((64, 1536), 128), ((40, 100), 20), ((7, 513), 3), ((2048, 2048), 64)])
-def test_decode_matches_oracle(oracle, dev, shape, group):
+def test_decode_matches_oracle(oracle, dev, decoder, shape, group):
     from ixrun_amd import ixgs
 
     w = heavy_tail(shape, seed=1)
@@ -50,7 +59,7 @@ def test_decode_matches_oracle(oracle, dev, shape, group):
 
 @pytest.mark.parametrize("mix", ["all_tiers", "only_tier3", "only_tier2", "dense_mix"])
 @pytest.mark.parametrize("shape,group", [((64, 1536), 64), ((37, 1000), 64), ((5, 100), 10)])
-def test_decode_hand_built_tiers(oracle, dev, mix, shape, group):
+def test_decode_hand_built_tiers(oracle, dev, decoder, mix, shape, group):
     """Integers over the whole range [-127, 128], which the quantizer itself never emits."""
     from ixrun_amd import ixgs
 

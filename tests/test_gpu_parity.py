@@ -144,6 +144,31 @@ def test_decode_bf16_only(oracle, dev, kind, shape, level_bits):
     assert torch.all(o16[p["N"]:] == 7.0)  # nothing written past the end
 
 
+@pytest.mark.parametrize("decoder", ["0", "1"])
+@pytest.mark.parametrize("kind", KINDS + ["all_l3", "zeros"])
+@pytest.mark.parametrize("shape", [(1, 1), (1, 31), (1, 512), (3, 171), (5, 413), (33, 1000), (64, 1536), (300, 1031),
+                                   (256, 4608), (17, 2048), (1, 2049)])
+def test_decode_358_both_decoders(oracle, dev, monkeypatch, kind, shape, decoder):
+    """(3,5,8) to bf16 at unit 512 through each of the two decoders, whatever the mix of levels would choose:
+    "1" forces the level-by-level decoder (partial last lane, partial last span, tensors smaller than a lane),
+    "0" the one that stages the streams."""
+    monkeypatch.setenv("IXH_DECODE_DENSE", decoder)
+    if kind == "all_l3":
+        g = torch.Generator("cpu").manual_seed(shape[1])
+        w = ((torch.randint(0, 2, shape, generator=g) * 2 - 1) * (0.25 + 0.5 * torch.rand(shape, generator=g))).bfloat16()
+        p = quantize(w, (3, 5, 8))
+    elif kind == "zeros":
+        p = quantize(torch.zeros(shape, dtype=torch.bfloat16), (3, 5, 8))
+    else:
+        p = make_packed(kind, *shape, (3, 5, 8))
+    dp = device_packed(p, dev)
+    table = dp.prefix_build(512)
+    o16 = torch.full((p["N"] + 64,), 7.0, dtype=torch.bfloat16, device=dev)
+    dp.decode(table, 512, out_bf16=o16[: p["N"]])
+    assert np.array_equal(bf16_bits(o16[: p["N"]]).reshape(shape), oracle.decode_packed_bf16(p)), (kind, shape, decoder)
+    assert torch.all(o16[p["N"]:] == 7.0)  # nothing written past the end
+
+
 @pytest.mark.parametrize("level_bits", [(3, 4, 5, 6, 8), (2, 8), (4, 8), (1, 2, 3, 4, 5, 6, 7, 8), (3, 3, 8)])
 def test_decode_other_level_schemes(oracle, dev, level_bits):
     from ixrun_amd.triton_kernels import decode_weight_triton, decode_int8
