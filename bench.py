@@ -296,6 +296,8 @@ def main():
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of hipGraph replays")
     ap.add_argument("--unfused", action="store_true",
                     help="many-row workloads: decode the bf16 weight to HBM and call the library GEMM instead")
+    ap.add_argument("--tune-gemm", action="store_true",
+                    help="with --unfused: let the library GEMM of the many-row path be chosen by measurement")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 256 MiB device copies (known traffic) so that counter runs can be scaled")
     args = ap.parse_args()
@@ -323,6 +325,9 @@ def main():
     chained = args.workload.startswith("graph64")
     copies = args.copies or (64 if chained else max(2, -(-600_000_000 // packed["total_bytes"])))
     layers = [StreamingLinear(packed) for _ in range(copies)]
+    if args.tune_gemm:
+        from ixrun_amd import gemm_tuning
+        gemm_tuning.enable()
     if args.unfused:
         shared = torch.empty(packed["N"], dtype=torch.bfloat16, device=dev)
         for sl in layers:
@@ -435,6 +440,8 @@ def main():
                     "that feeds the matrix cores, not by MFMA issue",
         }
         out["path"] = "decode to HBM + library GEMM" if args.unfused else "fused decode + MFMA (ixh_gemm)"
+        if args.unfused and args.tune_gemm:
+            out["path"] += ", GEMM kernel chosen by measurement (torch.cuda.tunable)"
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(weight, x_host, level_bits)
         out["cpu_baseline"]["speedup_vs_cpu"] = out["value"] / out["cpu_baseline"]["value"]

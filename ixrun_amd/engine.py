@@ -19,7 +19,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from . import _lib
+from . import _lib, gemm_tuning
 from .config import TRITON_BLOCK
 from .fused import FUSED_TILE, _pick_split, pick_unit, shared_workspace
 from .linear import _set_parent_child, iter_quantizable_linears
@@ -156,7 +156,7 @@ class StreamingLinear(nn.Module):
                 return y
         w = self._decode()
         bias = self._bias.to(x.dtype) if self._bias is not None else None
-        return F.linear(x, w.to(x.dtype) if w.dtype != x.dtype else w, bias)
+        return gemm_tuning.linear(x, w.to(x.dtype) if w.dtype != x.dtype else w, bias)
 
 
 class GraphLinear(nn.Module):
@@ -177,7 +177,7 @@ class GraphLinear(nn.Module):
     def forward(self, x):
         w = self._w_buf[: self.N].view(self.out_features, self.in_features)
         bias = self._bias.to(x.dtype) if self._bias is not None else None
-        return F.linear(x, w, bias)
+        return gemm_tuning.linear(x, w, bias)
 
 
 class ResourceScheduler:

@@ -4,6 +4,7 @@ file, graph.  Outputs are compared with the same model run on plain int8-dequant
 weights, the reference's own equivalence claim (tests/test_int8_equivalence.py:29-33)."""
 import copy
 
+import numpy as np
 import pytest
 import torch
 import torch.nn as nn
@@ -104,3 +105,36 @@ def test_five_level_streaming_linear():
         x = torch.randn(rows, 768, generator=torch.Generator().manual_seed(rows)).bfloat16().cuda()
         want = torch.nn.functional.linear(x.float().cpu(), decode_to_weight(p).float())
         assert close(sl(x).cpu(), want)
+
+
+def test_tuned_library_gemm_on_the_many_row_path(oracle):
+    """Decode + library GEMM with the GEMM kernel chosen by measurement: same result to the tolerance of the
+    many-row path (rel-L2 <= 1e-3 against the fp64 product of the dequantised weights), signature remembered,
+    tuning off again afterwards."""
+    import torch.cuda.tunable as tunable
+    from ixrun_amd import gemm_tuning
+    from ixrun_amd.engine import StreamingLinear
+    from ixrun_amd.quantize import int8x_quantize
+    from helpers import student_t_weight
+
+    dev = torch.device("cuda:0")
+    w = student_t_weight(256, 1024, seed=11)
+    p = int8x_quantize(w, (3, 5, 8))
+    layer = StreamingLinear(p)
+    layer._gemm_ok = False
+    layer._set_shared_buf(torch.empty(p["N"], dtype=torch.bfloat16, device=dev))
+    x = torch.randn(96, 1024, generator=torch.Generator("cpu").manual_seed(3)).bfloat16()
+    w_deq = oracle.bf16_bits_to_f32(oracle.decode_packed_bf16(p)).astype(np.float64).reshape(256, 1024)
+    want = torch.from_numpy(x.double().numpy() @ w_deq.T).bfloat16().double().numpy()  # the exact product, as bf16
+    plain = layer(x.to(dev)).float().cpu().numpy()
+    gemm_tuning.enable(max_ms=50)
+    try:
+        tuned = layer(x.to(dev)).float().cpu().numpy()
+        again = layer(x.to(dev)).float().cpu().numpy()
+        assert (96, 256, 1024, torch.bfloat16, False) in gemm_tuning.tuned_shapes()
+        assert not tunable.tuning_is_enabled()
+    finally:
+        gemm_tuning.disable()
+    for got in (plain, tuned, again):
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-3
+    assert np.array_equal(tuned, again)
