@@ -109,15 +109,21 @@ static int decode_any(const IxhPacked *packed, const int32_t *prefix, int64_t ch
     if (d.n == 0) return IXH_OK;
     if (!prefix) { set_error("prefix is NULL"); return IXH_EINVAL; }
     if (!out_i8 && !out_bf16) { set_error("both outputs are NULL"); return IXH_EINVAL; }
-    static const bool no_staged = getenv("IXH_DECODE_GENERIC") != nullptr;  // measurement switches
-    const char *dense_env = getenv("IXH_DECODE_DENSE");  // read per call so that tests can force either decoder
-    const int dense_mode = dense_env ? atoi(dense_env) : -1;
-    // (3,5,8) with many elements above level 1: the level-by-level decoder (see ixh_dense358.hip)
+    // Which decoder: by the tensor, unless IXH_DECODE_KERNEL names one (rows | dense | staged | generic; read per call,
+    // so that tests and measurements can take each of them; a named kernel that does not support the call is skipped).
+    const char *want = getenv("IXH_DECODE_KERNEL");
+    auto allowed = [&](const char *name) { return !want || !*want || strcmp(want, name) == 0; };
+    const bool forced = want && *want;
+    // level 1 holds at least 97 % of the elements (from the size of its stream)
     const bool mostly_l1 = (uint64_t)d.st_words[0] * 32u / 3u >= (uint64_t)d.n / 100u * 97u;
-    if (!no_staged && dense_mode != 0 && (dense_mode == 1 || !mostly_l1) &&
-        decode_dense358_supports(d, (uint32_t)chunk, out_i8, out_bf16, gs))
+    if (allowed("rows") && (forced || mostly_l1) && !gs.fp16 && decode_rows358_supports(d, (uint32_t)chunk, out_i8, out_bf16))
+        // (3,5,8), almost all level 1, whole unit-quads: the row-block decoder (ixh_decode_rows358.hip)
+        rc = launch_decode_rows358(d, prefix, out_bf16, (hipStream_t)stream);
+    else if (allowed("dense") && (forced || !mostly_l1) && decode_dense358_supports(d, (uint32_t)chunk, out_i8, out_bf16, gs))
+        // (3,5,8) with many elements above level 1: the level-by-level decoder (ixh_dense358.hip)
         rc = launch_decode_dense358(d, prefix, out_bf16, gs, (hipStream_t)stream);
-    else if (!no_staged && decode_staged_supports(d, (uint32_t)chunk, out_i8, out_bf16, gs))
+    else if ((allowed("staged") || allowed("rows") || allowed("dense")) &&
+             decode_staged_supports(d, (uint32_t)chunk, out_i8, out_bf16, gs))
         rc = launch_decode_staged(d, prefix, out_bf16, gs, (hipStream_t)stream);
     else
         rc = launch_decode(d, prefix, (uint32_t)chunk, out_i8, out_bf16, gs, (hipStream_t)stream);

@@ -18,6 +18,8 @@ int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x,
 bool gemv_dense358_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x);
 int launch_gemv_dense358(const Dev &P, const int32_t *prefix, const uint16_t *x, uint16_t *y, float *y32, float *ws,
                          bool atomic, hipStream_t s);
+bool decode_rows358_supports(const Dev &P, uint32_t chunk, const int8_t *o8, const uint16_t *o16);
+int launch_decode_rows358(const Dev &P, const int32_t *prefix, uint16_t *o16, hipStream_t s);
 bool decode_dense358_supports(const Dev &P, uint32_t chunk, const int8_t *o8, const uint16_t *o16, GroupScales gs);
 int launch_decode_dense358(const Dev &P, const int32_t *prefix, uint16_t *o16, GroupScales gs, hipStream_t s);
 int launch_reduce_chunks(const float *ws, uint32_t n_chunks, int m, uint32_t out_f, uint16_t *y, int64_t ldy,

@@ -32,12 +32,12 @@ def packed_from_ints(oracle, q, scales, out_f, in_f, group):
             "counts": e["counts"], "total_bytes": 0, "bits_per_weight": 0.0, "compression_vs_bf16": 0.0}
 
 
-@pytest.fixture(params=["by_mix", "0", "1"])
+@pytest.fixture(params=["by_mix", "staged", "dense"])
 def decoder(request, monkeypatch):
-    """Which of the two unit-512 decoders runs: chosen by the mix of tiers, or forced ("1": level by level where the
-    group size allows it, "0": the one that stages the streams)."""
+    """Which of the two unit-512 decoders runs: chosen by the mix of tiers, or forced (level by level where the
+    group size allows it, or the one that stages the streams)."""
     if request.param != "by_mix":
-        monkeypatch.setenv("IXH_DECODE_DENSE", request.param)
+        monkeypatch.setenv("IXH_DECODE_KERNEL", request.param)
     return request.param
 
 

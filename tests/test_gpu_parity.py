@@ -144,15 +144,17 @@ def test_decode_bf16_only(oracle, dev, kind, shape, level_bits):
     assert torch.all(o16[p["N"]:] == 7.0)  # nothing written past the end
 
 
-@pytest.mark.parametrize("decoder", ["0", "1"])
+@pytest.mark.parametrize("decoder", ["staged", "dense", "rows"])
 @pytest.mark.parametrize("kind", KINDS + ["all_l3", "zeros"])
 @pytest.mark.parametrize("shape", [(1, 1), (1, 31), (1, 512), (3, 171), (5, 413), (33, 1000), (64, 1536), (300, 1031),
-                                   (256, 4608), (17, 2048), (1, 2049)])
-def test_decode_358_both_decoders(oracle, dev, monkeypatch, kind, shape, decoder):
-    """(3,5,8) to bf16 at unit 512 through each of the two decoders, whatever the mix of levels would choose:
-    "1" forces the level-by-level decoder (partial last lane, partial last span, tensors smaller than a lane),
-    "0" the one that stages the streams."""
-    monkeypatch.setenv("IXH_DECODE_DENSE", decoder)
+                                   (256, 4608), (17, 2048), (1, 2049), (4, 512), (8, 512), (52, 512), (200, 1024),
+                                   (1000, 2048), (2600, 1024)])
+def test_decode_358_each_decoder(oracle, dev, monkeypatch, kind, shape, decoder):
+    """(3,5,8) to bf16 at unit 512 through each of the three decoders, whatever the mix of levels would choose:
+    the level-by-level one (partial last lane, partial last span, tensors smaller than a lane), the one that
+    stages the streams, and the row-block one (whole unit-quads only: other sizes fall through to the staged one;
+    with dense mixes its record queue is resolved every few units)."""
+    monkeypatch.setenv("IXH_DECODE_KERNEL", decoder)
     if kind == "all_l3":
         g = torch.Generator("cpu").manual_seed(shape[1])
         w = ((torch.randint(0, 2, shape, generator=g) * 2 - 1) * (0.25 + 0.5 * torch.rand(shape, generator=g))).bfloat16()
