@@ -117,7 +117,7 @@ static int decode_any(const IxhPacked *packed, const int32_t *prefix, int64_t ch
     // level 1 holds at least 97 % of the elements (from the size of its stream)
     const bool mostly_l1 = (uint64_t)d.st_words[0] * 32u / 3u >= (uint64_t)d.n / 100u * 97u;
     if (allowed("rows") && (forced || mostly_l1) && !gs.fp16 && decode_rows358_supports(d, (uint32_t)chunk, out_i8, out_bf16))
-        // (3,5,8), almost all level 1, whole unit-quads: the row-block decoder (ixh_decode_rows358.hip)
+        // first level of 3 bits, almost all level 1, whole unit-quads: the row-block decoder (ixh_decode_rows358.hip)
         rc = launch_decode_rows358(d, prefix, out_bf16, (hipStream_t)stream);
     else if (allowed("dense") && (forced || !mostly_l1) && decode_dense358_supports(d, (uint32_t)chunk, out_i8, out_bf16, gs))
         // (3,5,8) with many elements above level 1: the level-by-level decoder (ixh_dense358.hip)

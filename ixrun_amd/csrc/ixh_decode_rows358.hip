@@ -1,5 +1,6 @@
-// (3,5,8) full decode to bf16 for tensors that are almost all level 1, built like the row-block product kernel
-// (ixh_rows358.hip) with the dot products taken out and the weights written instead.
+// Full decode to bf16 for tensors that are almost all level 1, for (3,5,8) and any other scheme whose first level has
+// 3 bits: built like the row-block product kernel (ixh_rows358.hip) with the dot products taken out and the weights
+// written instead.
 //
 // Work split.  The tensor is a flat run of 512-element units; four consecutive units are a unit-quad.  A workgroup
 // owns a contiguous run of unit-quads, its waves take them in turn; each 16-lane DPP row of a wave takes one unit of
@@ -210,6 +211,66 @@ __device__ __forceinline__ void dr_resolve(const Dev &P, const DrSide &sv, uint3
     }
 }
 
+// The same for any scheme whose first level has 3 bits: an element above level 1 is followed down the nested
+// bitmaps (level i: rank among the elements that are in no level below i), every rank counted from the unit's start,
+// where the table holds it; all reads from global memory (these elements are rare in the tensors this kernel gets).
+__device__ __forceinline__ void dr_resolve_any(const Dev &P, const int32_t *__restrict__ prefix, uint32_t entries,
+                                               uint32_t tq1_addr, uint32_t unit0, const uint4 *__restrict__ queue,
+                                               uint32_t count, uint16_t *__restrict__ out, float scale, uint32_t lane) {
+    auto one = [&](const uint4 rec, uint32_t nth, uint32_t e) {
+        const uint32_t unit = rec.z;
+        uint32_t r = rec.y + nth;                                                           // rank at level i
+        uint32_t ru = unit * kFastChunk - dr_lds_u32(tq1_addr + (unit - unit0) * 4);        // the unit's first rank there
+        int v = 0;
+        bool found = false;
+        for (int i = 1; i + 1 < P.n_levels; ++i) {
+            const uint32_t *__restrict__ bm = P.bm[i];
+            const uint32_t words = P.bm_words[i];
+            const uint32_t qu = (uint32_t)prefix[(size_t)i * entries + unit];  // level-i elements before the unit
+            const uint32_t wf = ru >> 5, wl = min(r >> 5, wf + 17u);
+            const uint32_t first_mask = ~0u << (ru & 31);
+            uint32_t cnt = 0;
+            for (uint32_t w = wf; w < wl; ++w) {
+                uint32_t bits = w < words ? bm[w] : 0u;
+                if (w == wf) bits &= first_mask;
+                cnt += __popc(bits);
+            }
+            const uint32_t bits = wl < words ? bm[wl] : 0u;
+            uint32_t low = (1u << (r & 31)) - 1u;
+            if (wl == wf) low &= first_mask;
+            cnt += __popc(bits & low);
+            if ((bits >> (r & 31)) & 1u) {
+                const uint32_t nb = (uint32_t)P.bits[i];
+                const uint64_t bitpos = (uint64_t)(qu + cnt) * nb;
+                const uint32_t wi = (uint32_t)(bitpos >> 5), sh = (uint32_t)bitpos & 31u;
+                const uint32_t lo = wi < P.st_words[i] ? P.st[i][wi] : 0u;
+                const uint32_t hi = (sh + nb > 32 && wi + 1 < P.st_words[i]) ? P.st[i][wi + 1] : 0u;
+                v = (int)((uint32_t)((((uint64_t)hi << 32) | lo) >> sh) & ((1u << nb) - 1u)) - threshold_of((int)nb);
+                found = true;
+                break;
+            }
+            r -= qu + cnt;
+            ru -= qu;
+        }
+        if (!found) v = r < P.last_bytes ? (int)P.last[r] - 127 : 0;
+        out[(size_t)unit * kFastChunk + rec.w + e] = (uint16_t)f32_to_bf16_bits((float)v * scale);
+    };
+    dr_wait_vmem<0>();
+    for (uint32_t base = 0; base < count; base += kWave) {
+        const uint32_t idx = base + lane;
+        uint4 rec = make_uint4(0, 0, 0, 0);
+        if (idx < count) rec = queue[idx];
+        uint32_t zeros = rec.x, nth = 0;
+        while (zeros != 0) {
+            const uint32_t e = (uint32_t)__builtin_ctz(zeros);
+            zeros &= zeros - 1;
+            one(rec, nth++, e);
+        }
+    }
+}
+
+// ANY: any scheme whose first level has 3 bits (else: (3,5,8), with the small-share staging of the other streams)
+template <bool ANY>
 __global__ void __launch_bounds__(kDrWaves *kWave)
 k_decode358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_quads, uint32_t quads_per_wg, uint32_t flags,
                  uint16_t *__restrict__ out) {
@@ -245,7 +306,7 @@ k_decode358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_quads, ui
     const uint32_t entries = n_quads * 4 + 1;
     for (uint32_t i = tid; i <= units_here; i += blockDim.x) {
         tq1[i] = (uint32_t)prefix[unit0 + i];
-        tq2[i] = (uint32_t)prefix[entries + unit0 + i];
+        if (!ANY) tq2[i] = (uint32_t)prefix[entries + unit0 + i];
     }
     const float scale = bf16_bits_to_f32(*P.scale);
     for (uint32_t i = tid; i < 64 * 32; i += blockDim.x) {
@@ -279,7 +340,8 @@ k_decode358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_quads, ui
     // (every wave copies all of it: same bytes to the same place, and a wave's own loads complete in order, before
     // the first unit it waits for, so no barrier is needed)
     DrSide sv;
-    {
+    sv.staged = false;
+    if (!ANY) {
         const uint32_t q1b = tq1[0], q2b = tq2[0], q1e = tq1[units_here], q2e = tq2[units_here];
         const uint32_t nl1b = unit0 * kFastChunk - q1b, nl1e = (unit0 + units_here) * kFastChunk - q1e;
         sv.base = L.side;
@@ -377,7 +439,8 @@ k_decode358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_quads, ui
     };
 
     auto resolve = [&](uint32_t count) {
-        if (sv.staged) dr_resolve<true>(P, sv, tq1_addr, tq2_addr, unit0, queue, count, tasks, out, scale, lane);
+        if (ANY) dr_resolve_any(P, prefix, entries, tq1_addr, unit0, queue, count, out, scale, lane);
+        else if (sv.staged) dr_resolve<true>(P, sv, tq1_addr, tq2_addr, unit0, queue, count, tasks, out, scale, lane);
         else dr_resolve<false>(P, sv, tq1_addr, tq2_addr, unit0, queue, count, tasks, out, scale, lane);
     };
 
@@ -454,7 +517,7 @@ k_decode358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_quads, ui
 }
 
 bool decode_rows358_supports(const Dev &P, uint32_t chunk, const int8_t *o8, const uint16_t *o16) {
-    return P.n_levels == 3 && P.bits[0] == 3 && P.bits[1] == 5 && P.bits[2] == 8 && chunk == kFastChunk && !o8 && o16 &&
+    return P.n_levels >= 2 && P.bits[0] == 3 && chunk == kFastChunk && !o8 && o16 &&
            ((uintptr_t)o16 & 15u) == 0 && P.n != 0 && P.n % (4 * kFastChunk) == 0 && P.n < (1u << 30);
 }
 
@@ -472,14 +535,21 @@ int launch_decode_rows358(const Dev &P, const int32_t *prefix, uint16_t *o16, hi
     const size_t lds = dr_layout(quads).total;
     static bool raised = false;
     if (!raised) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(k_decode358_rows), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                160 * 1024) != hipSuccess)
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(k_decode358_rows<false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess ||
+            hipFuncSetAttribute(reinterpret_cast<const void *>(k_decode358_rows<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
             return IXH_EUNSUPPORTED;
         raised = true;
     }
     if (lds > 160 * 1024) return IXH_EUNSUPPORTED;
     const uint32_t flags = ((uintptr_t)P.last & 3u) == 0 ? 1u : 0u;
-    hipLaunchKernelGGL(k_decode358_rows, dim3(groups), dim3(kDrWaves * kWave), lds, s, P, prefix, n_quads, quads, flags, o16);
+    if (P.n_levels == 3 && P.bits[1] == 5)
+        hipLaunchKernelGGL(k_decode358_rows<false>, dim3(groups), dim3(kDrWaves * kWave), lds, s, P, prefix, n_quads, quads,
+                           flags, o16);
+    else
+        hipLaunchKernelGGL(k_decode358_rows<true>, dim3(groups), dim3(kDrWaves * kWave), lds, s, P, prefix, n_quads, quads,
+                           flags, o16);
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }
 

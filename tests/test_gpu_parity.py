@@ -171,6 +171,23 @@ def test_decode_358_each_decoder(oracle, dev, monkeypatch, kind, shape, decoder)
     assert torch.all(o16[p["N"]:] == 7.0)  # nothing written past the end
 
 
+@pytest.mark.parametrize("level_bits", [(3, 4, 5, 6, 8), (3, 8), (3, 3, 8), (3, 4, 8), (3, 5, 6, 7, 8), (3, 4, 5, 6, 7, 8)])
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("shape", [(8, 512), (64, 1536), (1000, 2048)])
+def test_decode_row_block_decoder_other_schemes(oracle, dev, monkeypatch, kind, shape, level_bits):
+    """The row-block decoder takes every scheme whose first level has 3 bits; its elements above level 1 are followed
+    down the nested bitmaps one by one.  Forced here for every mix (it is chosen only for tensors that are almost all
+    level 1)."""
+    monkeypatch.setenv("IXH_DECODE_KERNEL", "rows")
+    p = make_packed(kind, *shape, level_bits)
+    dp = device_packed(p, dev)
+    table = dp.prefix_build(512)
+    o16 = torch.full((p["N"] + 64,), 7.0, dtype=torch.bfloat16, device=dev)
+    dp.decode(table, 512, out_bf16=o16[: p["N"]])
+    assert np.array_equal(bf16_bits(o16[: p["N"]]).reshape(shape), oracle.decode_packed_bf16(p)), (kind, shape, level_bits)
+    assert torch.all(o16[p["N"]:] == 7.0)
+
+
 @pytest.mark.parametrize("level_bits", [(3, 4, 5, 6, 8), (2, 8), (4, 8), (1, 2, 3, 4, 5, 6, 7, 8), (3, 3, 8)])
 def test_decode_other_level_schemes(oracle, dev, level_bits):
     from ixrun_amd.triton_kernels import decode_weight_triton, decode_int8
