@@ -37,7 +37,7 @@ MEASURED_TRAFFIC_BYTES = {
     "prefill_5120x5120_m512_five_level": 50297.9 * 2.0 * 1024 + 30720.0 * 1024,
     "attn_proj_5120x5120_m1_student_t": 7118.0 * 2.0 * 1024 + 16.0 * 1024,
     "gate_up_17408x5120_m4_student_t": 23193.0 * 2.0 * 1024 + 181.0 * 1024,
-    "decode_5120x17408_student_t": 25672.0 * 2.0 * 1024 + 174080.0 * 1024,
+    "decode_5120x17408_student_t": 23268.0 * 2.0 * 1024 + 179524.0 * 1024,
     "decode_5120x17408_calibrated": 36308.0 * 2.0 * 1024 + 174080.0 * 1024,
     "decode_gs_5120x17408_student_t": 33559.0 * 2.0 * 1024 + 174080.0 * 1024,
     # all kernels of one encode step together (absmax, count, scans, clear, pack)
