@@ -138,3 +138,27 @@ def test_tuned_library_gemm_on_the_many_row_path(oracle):
     for got in (plain, tuned, again):
         assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-3
     assert np.array_equal(tuned, again)
+
+
+@pytest.mark.parametrize("rows", [8, 9, 16])
+def test_row_count_policy_with_a_decode_buffer(oracle, rows):
+    """Up to 8 rows the fused kernel, from 9 on decode + GEMM when the layer has a decode buffer (without one the
+    fused kernel serves up to 16): all within the many-row tolerance of the exact product."""
+    from ixrun_amd.engine import StreamingLinear
+    from ixrun_amd.quantize import int8x_quantize
+    from helpers import student_t_weight
+
+    dev = torch.device("cuda:0")
+    p = int8x_quantize(student_t_weight(128, 2048, seed=5), (3, 5, 8))
+    x = torch.randn(rows, 2048, generator=torch.Generator("cpu").manual_seed(rows)).bfloat16()
+    w_deq = oracle.bf16_bits_to_f32(oracle.decode_packed_bf16(p)).astype(np.float64).reshape(128, 2048)
+    want = torch.from_numpy(x.double().numpy() @ w_deq.T).bfloat16().double().numpy()
+    plain = StreamingLinear(p)
+    buffered = StreamingLinear(p)
+    buf = torch.full((p["N"],), 9.0, dtype=torch.bfloat16, device=dev)
+    buffered._set_shared_buf(buf)
+    for layer in (plain, buffered):
+        got = layer(x.to(dev)).float().cpu().numpy()
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-3
+    decoded = bool((buf != 9.0).any())  # the buffer was written iff the pair path ran
+    assert decoded == (rows > 8)
