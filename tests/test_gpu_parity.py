@@ -384,10 +384,26 @@ def test_full_size_layers(oracle, dev, shape, m):
     x = activations(m, in_f, seed=1)
     y = sl(x.to(dev))
     w_bits = oracle.dequant_bf16(q_want, oracle.packed_to_numpy(p)["scale_bits"]).reshape(out_f, in_f)
+    # the bf16 decode as the library chooses it for this tensor (the row-block decoder: > 97 % level 1)
+    o16 = torch.zeros(p["N"], dtype=torch.bfloat16, device=dev)
+    sl._dp.decode(sl._table, sl._unit, out_bf16=o16)
+    assert np.array_equal(bf16_bits(o16).reshape(out_f, in_f), w_bits)
+    del o16
     y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
     err = check_outputs(bf16_bits(y), y64, f"full {shape} m={m}")
     print(f"{shape} m={m}: rel-L2 {err:.2e}, fractions {[round(c / p['N'], 5) for c in p['counts']]}, "
           f"packed {p['total_bytes']} B")
+
+
+def test_full_size_five_level_decode(oracle, dev):
+    """5120 x 17408 Student-t in the five-level scheme: the bf16 decode (row-block decoder, elements above level 1
+    followed down four bitmaps) equals the oracle's, every element."""
+    p = quantize(student_t_weight(5120, 17408, seed=0), (3, 4, 5, 6, 8))
+    dp = device_packed(p, dev)
+    table = dp.prefix_build(512)
+    o16 = torch.zeros(p["N"], dtype=torch.bfloat16, device=dev)
+    dp.decode(table, 512, out_bf16=o16)
+    assert np.array_equal(bf16_bits(o16), oracle.decode_packed_bf16(p).reshape(-1))
 
 
 def test_full_size_calibrated_layer(oracle, dev):
