@@ -99,8 +99,12 @@ int ixh_prefix_build(const IxhPacked *packed, int64_t chunk, int32_t *prefix, ix
  * _ix_decode_kernel / decode_weight_triton (ixrun/triton_kernels.py:68-177,
  * :224-259) and StreamingLinear._decode (ixrun/engine.py:109-133), for any
  * level scheme.  prefix/chunk: a table from ixh_prefix_build; any chunk > 0.
- * Fastest with chunk = 512, bf16 output only and a 16-byte aligned out_bf16
- * (the streams are then staged through on-chip memory).
+ * Fastest with chunk = 512, bf16 output only and a 16-byte aligned out_bf16:
+ * then one of three kernels that stage the streams through on-chip memory runs,
+ * chosen from the tensor (a first level of 3 bits that holds 97 % or more of the
+ * elements, with out_f * in_f a multiple of 2048: the row-block decoder; other
+ * (3,5,8) tensors: the level-by-level decoder; any other scheme: the staged
+ * decoder).  All kernels write the same bytes.
  */
 int ixh_decode(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, int8_t *out_i8,
                uint16_t *out_bf16, ixh_stream_t stream);
@@ -114,8 +118,8 @@ int ixh_decode(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, in
  * tensors (ixgs/kernels.py:107-118, three int32 per weight) are replaced by the same
  * chunked rank table as ixh_decode.  packed->scale is not read and may be NULL; the codes
  * are offset by 3 / 15 / 127 exactly as in the per-tensor format, so values up to +128
- * (ixgs/quantize.py:63) decode correctly.  Fastest with chunk = 512, group_size a multiple
- * of 8 and a 16-byte aligned out_bf16.
+ * (ixgs/quantize.py:63) decode correctly.  Fastest with chunk = 512, group_size a power of
+ * two from 32 up (a multiple of 8 otherwise) and a 16-byte aligned out_bf16.
  */
 int ixh_decode_gs(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, const uint16_t *group_scales,
                   int64_t group_size, uint16_t *out_bf16, ixh_stream_t stream);
