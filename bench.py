@@ -53,6 +53,9 @@ WORKLOADS = {
     "gate_up_17408x5120_m4_student_t": (17408, 5120, 4, "student_t"),
     "gate_up_17408x5120_m8_student_t": (17408, 5120, 8, "student_t"),
     "gate_up_17408x5120_m16_student_t": (17408, 5120, 16, "student_t"),
+    "gate_up_17408x5120_m2_calibrated": (17408, 5120, 2, "calibrated"),
+    "gate_up_17408x5120_m4_calibrated": (17408, 5120, 4, "calibrated"),
+    "gate_up_17408x5120_m8_calibrated": (17408, 5120, 8, "calibrated"),
     # 64 distinct 5120x5120 layers chained (each output feeds the next layer), one hipGraph: us per layer
     "graph64_5120x5120_m1_student_t": (5120, 5120, 1, "student_t"),
     # many activation rows: decode into LDS tiles + bf16 MFMA, five-level scheme

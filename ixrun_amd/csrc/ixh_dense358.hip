@@ -306,35 +306,54 @@ k_gemv358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// Full decode to bf16 by the same route, for dense mixes: the codes of each level are dequantised where they lie
-// (dense, fixed positions) into three LDS arrays of weights, and every lane then gathers the weights of its 32
-// positions from the slots that the scatter above would have written to.  Spans are 2048 consecutive flat elements
-// (rows play no part in a decode); the last span and the last lane may be partial.
+// The weights of a span in position order, by the same route turned round (for dense mixes): the codes of each level
+// are dequantised where they lie (dense, fixed positions) into three LDS arrays of weights, and every lane then
+// gathers the weights of its 32 positions from the slots that the scatter above would have written to.
+// dn_walk_spans does this for every span that `spans` deals to the wave and hands the lane's 16 packed pairs to
+// `sink` (the full decode stores them, the several-row product multiplies them with its activations).
 // A lane's rows of the three arrays hold a number of codes that is twice an odd number, and the passes work in groups
 // of two pairs, so a lane's last group decodes one pair that is the next lane's first: both write the same value.
 // With group scales (GS: one fp16 scale per 2^group_shift >= 32 consecutive elements, so one per lane) the arrays
 // hold the integer values as bf16, exact, and the lane multiplies what it gathered by its scale.
 // ---------------------------------------------------------------------------------------------------------------
-template <bool GS>
-__global__ void __launch_bounds__(kWave *kDnWaves)
-k_decode358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, uint32_t n_spans, uint16_t *__restrict__ out,
-                  const uint16_t *__restrict__ group_scales, uint32_t group_shift) {
-    __shared__ __attribute__((aligned(16))) uint32_t lut[kDnLutBytes / 4];
-    __shared__ __attribute__((aligned(16))) uint16_t wc_all[kDnWaves][kDnSlots];
-    const uint32_t tid = threadIdx.x, lane = tid & 63;
-    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const float scale = GS ? 1.0f : bf16_bits_to_f32(*P.scale);
-    const float m15 = -15.0f * scale, m127 = -127.0f * scale;
-    for (uint32_t e = tid; e < 64 * 32; e += kWave * kDnWaves) {
-        const uint32_t idx = e >> 5;
-        lut[e] = dn_pack(dequant((int)(idx & 7u) - 3, scale), dequant((int)(idx >> 3) - 3, scale));
-    }
-    __syncthreads();
+struct DnSpan {
+    uint32_t p0, n_el;   // first flat element, elements (a multiple of 32 except at the tensor's end)
+    uint32_t u0, u1;     // rank-table entries at its start and end
+    uint32_t a, b, c;    // the enumerator's own: span index, or row / span of the row / item
+};
 
-    uint16_t *const wc = wc_all[wave];
+// flat spans of 2048 elements, dealt to the waves of the launch in turn
+struct DnFlatSpans {
+    uint32_t n_units, n_spans, n, first, stride;
+    __device__ __forceinline__ DnSpan at(uint32_t s) const {
+        DnSpan sp;
+        sp.u0 = 4 * s;
+        sp.u1 = min(sp.u0 + 4, n_units);
+        sp.p0 = sp.u0 * kFastChunk;
+        sp.n_el = min(kDnSpan, n - sp.p0);
+        sp.a = s; sp.b = 0; sp.c = 0;
+        return sp;
+    }
+    __device__ __forceinline__ bool first_span(DnSpan &sp) const {
+        if (first >= n_spans) return false;
+        sp = at(first);
+        return true;
+    }
+    __device__ __forceinline__ bool next(const DnSpan &cur, DnSpan &nx) const {
+        if (cur.a + stride >= n_spans) return false;
+        nx = at(cur.a + stride);
+        return true;
+    }
+};
+
+template <bool GS, class Spans, class Sink>
+__device__ __forceinline__ void dn_walk_spans(const Dev &P, const int32_t *__restrict__ prefix, uint32_t entries,
+                                              const uint16_t *__restrict__ group_scales, uint32_t group_shift,
+                                              const uint32_t *lut, uint16_t *wc, float scale, uint32_t lane,
+                                              const Spans &spans, Sink &sink) {
+    const float m15 = -15.0f * scale, m127 = -127.0f * scale;
     uint32_t *const wc32 = reinterpret_cast<uint32_t *>(wc);
     const uint32_t lut_lane = (lane & 31u) << 2;
-    const uint32_t entries = n_units + 1;
     const uint32_t *__restrict__ b1 = P.bm[0];
     const __amdgpu_buffer_rsrc_t l1_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void *)P.st[0], 0, (int)(P.st_words[0] * 4u), 0x00020000);
@@ -354,17 +373,17 @@ k_decode358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, u
     // Codes of a level per lane: enough for all of them, and twice an odd number, so that the lanes' rows of the LDS
     // array start an odd number of dwords apart (no two of 32 neighbouring lanes on one bank).  2, 6, ... 34.
     auto codes_per_lane = [](uint32_t n) { return (((n + 63) / 64 + 1) & ~3u) + 2; };
-    auto table_of = [&](uint32_t s) {
-        const uint32_t u0 = 4 * s, u1 = min(u0 + 4, n_units);
-        return Ranks{(uint32_t)prefix[u0], (uint32_t)prefix[u1], (uint32_t)prefix[entries + u0], (uint32_t)prefix[entries + u1]};
+    auto table_of = [&](const DnSpan &sp) {
+        return Ranks{(uint32_t)prefix[sp.u0], (uint32_t)prefix[sp.u1], (uint32_t)prefix[entries + sp.u0],
+                     (uint32_t)prefix[entries + sp.u1]};
     };
-    auto shape_of = [&](uint32_t s, const Ranks &q) {
-        const uint32_t p0 = 4 * s * kFastChunk, n_el = min(kDnSpan, P.n - p0);
+    auto shape_of = [&](const DnSpan &sp, const Ranks &q) {
+        const uint32_t p0 = sp.p0, n_el = sp.n_el;
         const uint32_t n1 = q.q1b - q.q1a, n2 = q.q2b - q.q2a, n3 = n_el - n1 - n2;
         return Shape{p0, n_el, codes_per_lane(n1), codes_per_lane(n2), codes_per_lane(n3)};
     };
-    auto fetch = [&](uint32_t s, const Ranks &q) {
-        const Shape g = shape_of(s, q);
+    auto fetch = [&](const DnSpan &sp, const Ranks &q) {
+        const Shape g = shape_of(sp, q);
         Loads r;
         r.w1 = 32 * lane < g.n_el ? b1[(g.p0 >> 5) + lane] : 0u;
         r.group_scale = GS && 32 * lane < g.n_el ? group_scales[(g.p0 + 32 * lane) >> group_shift] : 0u;
@@ -389,18 +408,21 @@ k_decode358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, u
         return r;
     };
 
-    const uint32_t n_waves = gridDim.x * kDnWaves;
-    uint32_t s = blockIdx.x * kDnWaves + wave;
-    if (s >= n_spans) return;
-    const uint32_t last_span = n_spans - 1;
-    Ranks q_now = table_of(s);
-    Loads in_now = fetch(s, q_now);
-    Ranks q_next = table_of(min(s + n_waves, last_span));
-    for (; s < n_spans; s += n_waves) {
-        // the span after this one (or, at the end, the last span once more: loads that nobody uses)
-        const Loads in_next = fetch(min(s + n_waves, last_span), q_next);
-        const Ranks q_after = table_of(min(s + 2 * n_waves, last_span));
-        const Shape g = shape_of(s, q_now);
+
+    DnSpan sp_now, sp_next, sp_after;
+    if (!spans.first_span(sp_now)) return;
+    bool has_next = spans.next(sp_now, sp_next);
+    if (!has_next) sp_next = sp_now;  // at the end the last span is fetched once more: loads that nobody uses
+    bool has_after = has_next && spans.next(sp_next, sp_after);
+    if (!has_after) sp_after = sp_next;
+    Ranks q_now = table_of(sp_now);
+    Loads in_now = fetch(sp_now, q_now);
+    Ranks q_next = table_of(sp_next);
+    for (;;) {
+        const Loads in_next = fetch(sp_next, q_next);
+        const Ranks q_after = table_of(sp_after);
+        sink.begin(sp_now);
+        const Shape g = shape_of(sp_now, q_now);
         const uint32_t p0 = g.p0, n_el = g.n_el, e1 = g.e1, e2 = g.e2, e3 = g.e3;
         const uint32_t q1a = q_now.q1a, q2a = q_now.q2a;
         const uint32_t base2 = 64 * e1, base3 = base2 + 64 * e2;
@@ -536,13 +558,36 @@ k_decode358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, u
                 s1 += in1; s2 += in2; s3 += in3; ja += out1;
             }
         }
-        uint16_t *dst = out + (size_t)p0 + 32 * lane;
         if (GS) {
             const float sc = fp16_bits_to_f32((uint16_t)in_now.group_scale);
 #pragma unroll
             for (int j = 0; j < 16; ++j)
                 o[j] = dn_pack(__uint_as_float(o[j] << 16) * sc, __uint_as_float(o[j] & 0xffff0000u) * sc);
         }
+        sink.end(sp_now, o, n_here);
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (!has_next) break;
+        sp_now = sp_next;
+        in_now = in_next;
+        q_now = q_next;
+        q_next = q_after;
+        sp_next = sp_after;
+        has_next = has_after;
+        has_after = has_next && spans.next(sp_next, sp_after);
+        if (!has_after) sp_after = sp_next;
+    }
+}
+
+// the full decode's end of a span: the lane's 64 bytes to their place in the output
+struct DnStoreSink {
+    uint16_t *__restrict__ out;
+    uint16_t *wc;
+    uint32_t lane;
+    __device__ __forceinline__ void begin(const DnSpan &) {}
+    __device__ __forceinline__ void end(const DnSpan &sp, const uint32_t (&o)[16], uint32_t n_here) {
+        const uint32_t p0 = sp.p0, n_el = sp.n_el;
+        uint16_t *dst = out + (size_t)p0 + 32 * lane;
         if (n_el == kDnSpan) {
             // Whole span: through LDS once more, so that a store instruction writes 1 KB of consecutive bytes
             // (lane rows 80 bytes apart keep the 16-byte accesses of eight neighbouring lanes on distinct banks).
@@ -568,12 +613,187 @@ k_decode358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, u
                 dst[t] = (uint16_t)((t & 1u) ? v >> 16 : v);
             }
         }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        in_now = in_next;
-        q_now = q_next;
-        q_next = q_after;
     }
+};
+
+template <bool GS>
+__global__ void __launch_bounds__(kWave *kDnWaves, 5)  // five waves per SIMD: what the LDS allows
+k_decode358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, uint32_t n_spans, uint16_t *__restrict__ out,
+                  const uint16_t *__restrict__ group_scales, uint32_t group_shift) {
+    __shared__ __attribute__((aligned(16))) uint32_t lut[kDnLutBytes / 4];
+    __shared__ __attribute__((aligned(16))) uint16_t wc_all[kDnWaves][kDnSlots];
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const float scale = GS ? 1.0f : bf16_bits_to_f32(*P.scale);
+    for (uint32_t e = tid; e < 64 * 32; e += kWave * kDnWaves) {
+        const uint32_t idx = e >> 5;
+        lut[e] = dn_pack(dequant((int)(idx & 7u) - 3, scale), dequant((int)(idx >> 3) - 3, scale));
+    }
+    __syncthreads();
+    const DnFlatSpans spans{n_units, n_spans, P.n, blockIdx.x * kDnWaves + wave, gridDim.x * kDnWaves};
+    DnStoreSink sink{out, wc_all[wave], lane};
+    dn_walk_spans<GS>(P, prefix, n_units + 1, group_scales, group_shift, lut, wc_all[wave], scale, lane, spans, sink);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Product with 2..4 activation rows for dense mixes: the span walker above with a sink that multiplies.  (With one
+// row it is cheaper to move the activations to the codes, k_gemv358_dense; with several rows the weights are
+// brought to position order once and meet every row's activations there.)
+// ---------------------------------------------------------------------------------------------------------------
+// spans of up to four units of one row; an item of the deal is a whole row (by_rows) or one span
+struct DnRowSpans {
+    uint32_t n_chunks, spans_per_row, n_items, first, stride, stride_rows, stride_spans;  // stride = rows * spans_per_row + spans
+    bool by_rows;
+    __device__ __forceinline__ DnSpan at(uint32_t row, uint32_t k, uint32_t item) const {
+        DnSpan sp;
+        const uint32_t nb = min(4u, n_chunks - 4 * k);
+        sp.u0 = row * n_chunks + 4 * k;
+        sp.u1 = sp.u0 + nb;
+        sp.p0 = sp.u0 * kFastChunk;
+        sp.n_el = nb * kFastChunk;
+        sp.a = row; sp.b = k; sp.c = item;
+        return sp;
+    }
+    __device__ __forceinline__ bool first_span(DnSpan &sp) const {
+        if (first >= n_items) return false;
+        sp = by_rows ? at(first, 0, first) : at(first / spans_per_row, first % spans_per_row, first);
+        return true;
+    }
+    __device__ __forceinline__ bool next(const DnSpan &cur, DnSpan &nx) const {
+        if (by_rows) {
+            if (cur.b + 1 < spans_per_row) { nx = at(cur.a, cur.b + 1, cur.c); return true; }
+            if (cur.a + stride >= n_items) return false;
+            nx = at(cur.a + stride, 0, cur.a + stride);
+            return true;
+        }
+        if (cur.c + stride >= n_items) return false;
+        uint32_t row = cur.a + stride_rows, k = cur.b + stride_spans;
+        if (k >= spans_per_row) { k -= spans_per_row; ++row; }
+        nx = at(row, k, cur.c + stride);
+        return true;
+    }
+};
+
+template <int MT>
+struct DnDotSink {
+    const uint16_t *__restrict__ x;
+    int64_t ldx;
+    int m;
+    uint16_t *__restrict__ y;
+    int64_t ldy;
+    float *__restrict__ ws;
+    uint32_t out_f, spans_per_row, lane;
+    bool by_rows;
+    uint32_t xr[MT][16];
+    float row_total[MT];  // meaningful in lane 63
+
+    // the lane's activations for this span, requested before the span's arithmetic starts
+    __device__ __forceinline__ void begin(const DnSpan &sp) {
+        const bool valid = 32 * lane < sp.n_el;
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            if (valid && j < m) {
+                const uint4 *xp = reinterpret_cast<const uint4 *>(x + (int64_t)j * ldx + (size_t)sp.b * kDnSpan + 32 * lane);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const uint4 v = xp[t];
+                    xr[j][4 * t] = v.x; xr[j][4 * t + 1] = v.y; xr[j][4 * t + 2] = v.z; xr[j][4 * t + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 16; ++t) xr[j][t] = 0u;  // lanes past the row's end gathered stale weights
+            }
+        }
+    }
+    __device__ __forceinline__ void end(const DnSpan &sp, const uint32_t (&o)[16], uint32_t) {
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+            for (int t = 0; t < 16; t += 2) {
+                a0 = dn_dot2(o[t], xr[j][t], a0);
+                a1 = dn_dot2(o[t + 1], xr[j][t + 1], a1);
+            }
+            const float total = dn_wave_sum(a0 + a1);
+            if (by_rows) {
+                row_total[j] = (sp.b == 0 ? 0.0f : row_total[j]) + total;
+                if (sp.b + 1 == spans_per_row && lane == 63 && j < m)
+                    y[(int64_t)j * ldy + sp.a] = (uint16_t)f32_to_bf16_bits(row_total[j]);
+            } else if (lane == 63 && j < m) {
+                ws[((size_t)sp.b * m + j) * out_f + sp.a] = total;
+            }
+        }
+    }
+};
+
+template <int MT>
+__global__ void __launch_bounds__(kWave *kDnWaves)
+k_gemv358_dense_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t spans_per_row, uint32_t n_items,
+                     const uint16_t *__restrict__ x, int m, int64_t ldx, uint16_t *__restrict__ y, int64_t ldy,
+                     float *__restrict__ ws, bool by_rows) {
+    __shared__ __attribute__((aligned(16))) uint32_t lut[kDnLutBytes / 4];
+    __shared__ __attribute__((aligned(16))) uint16_t wc_all[kDnWaves][kDnSlots];
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const float scale = bf16_bits_to_f32(*P.scale);
+    for (uint32_t e = tid; e < 64 * 32; e += kWave * kDnWaves) {
+        const uint32_t idx = e >> 5;
+        lut[e] = dn_pack(dequant((int)(idx & 7u) - 3, scale), dequant((int)(idx >> 3) - 3, scale));
+    }
+    // Lanes past a row's end gather from wherever their walk leads, inside the wave's arrays; their activations are
+    // zero, so what they find only has to be finite: start from zeros (later contents are weights).
+    for (uint32_t j = lane; j < kDnSlots / 8; j += kWave) reinterpret_cast<d_u32x4 *>(wc_all[wave])[j] = d_u32x4{0, 0, 0, 0};
+    __syncthreads();
+    const uint32_t stride = gridDim.x * kDnWaves;
+    const DnRowSpans spans{n_chunks, spans_per_row, n_items, blockIdx.x * kDnWaves + wave, stride, stride / spans_per_row,
+                           stride % spans_per_row, by_rows};
+    DnDotSink<MT> sink;
+    sink.x = x; sink.ldx = ldx; sink.m = m; sink.y = y; sink.ldy = ldy; sink.ws = ws;
+    sink.out_f = P.out_f; sink.spans_per_row = spans_per_row; sink.lane = lane; sink.by_rows = by_rows;
+#pragma unroll
+    for (int j = 0; j < MT; ++j) sink.row_total[j] = 0.0f;
+    dn_walk_spans<false>(P, prefix, P.out_f * n_chunks + 1, nullptr, 0u, lut, wc_all[wave], scale, lane, spans, sink);
+}
+
+bool gemv_dense358_rows_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x, int64_t ldx) {
+    return P.n_levels == 3 && P.bits[0] == 3 && P.bits[1] == 5 && P.bits[2] == 8 && chunk == kFastChunk && m >= 2 && m <= 4 &&
+           P.in_f % kFastChunk == 0 && P.in_f != 0 && ((uintptr_t)x & 15u) == 0 && (ldx & 7) == 0 &&
+           ((uintptr_t)P.last & 3u) == 0;
+}
+
+template <int MT>
+static int launch_dense_rows(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
+                             int64_t ldy, float *ws, hipStream_t s) {
+    const uint32_t n_chunks = P.in_f / kFastChunk;
+    const uint32_t spans_per_row = (n_chunks + 3) / 4;
+    const uint32_t n_spans = P.out_f * spans_per_row;
+    if (n_spans == 0) return IXH_OK;
+    static const uint32_t resident = [] {
+        int dev = 0, n_cu = 256, per_cu = 0;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_dense_rows<MT>, kWave * kDnWaves, 0) != hipSuccess ||
+            per_cu < 1)
+            per_cu = 3;
+        return (uint32_t)n_cu * (uint32_t)per_cu;
+    }();
+    // whole rows per wave when they spread over the resident waves within 12 % (one launch, no workspace); otherwise
+    // spans are dealt out and a second kernel adds a row's partial sums in span order
+    const uint32_t waves_res = resident * kDnWaves;
+    const uint32_t rounds = (P.out_f + waves_res - 1) / waves_res;
+    const bool by_rows = spans_per_row == 1 || (uint64_t)rounds * waves_res * 100u <= (uint64_t)P.out_f * 112u;
+    const uint32_t n_items = by_rows ? P.out_f : n_spans;
+    const uint32_t blocks = min(resident, (n_items + kDnWaves - 1) / kDnWaves);
+    hipLaunchKernelGGL(k_gemv358_dense_rows<MT>, dim3(blocks), dim3(kWave * kDnWaves), 0, s, P, prefix, n_chunks, spans_per_row,
+                       n_items, x, m, ldx, y, ldy, ws, by_rows);
+    if (hipGetLastError() != hipSuccess) return IXH_ELAUNCH;
+    if (!by_rows) return launch_reduce_chunks(ws, spans_per_row, m, P.out_f, y, ldy, s);
+    return IXH_OK;
+}
+
+int launch_gemv_dense358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
+                              int64_t ldy, float *ws, hipStream_t s) {
+    return m <= 2 ? launch_dense_rows<2>(P, prefix, x, m, ldx, y, ldy, ws, s)
+                  : launch_dense_rows<4>(P, prefix, x, m, ldx, y, ldy, ws, s);
 }
 
 bool decode_dense358_supports(const Dev &P, uint32_t chunk, const int8_t *o8, const uint16_t *o16, GroupScales gs) {
