@@ -221,7 +221,7 @@ int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, cons
         rc = launch_gemv_dense358(d, prefix, x, y, y32, (float *)workspace, atomic, (hipStream_t)stream);
     if (rc == IXH_EUNSUPPORTED && !atomic && !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED)) &&
         (!mostly_l1 || (flags & IXH_GEMV_DENSE)) && gemv_dense358_rows_supports(d, (uint32_t)chunk, m, x, ldx))
-        // (3,5,8), 2..4 activation rows, many elements above level 1: weights gathered to position order per span
+        // (3,5,8), 2..8 activation rows, many elements above level 1: weights gathered to position order per span
         rc = launch_gemv_dense358_rows(d, prefix, x, m, ldx, y, ldy, (float *)workspace, (hipStream_t)stream);
     if (rc == IXH_EUNSUPPORTED && !(flags & IXH_GEMV_FORCE_GENERIC) && gemv_staged_supports(d, (uint32_t)chunk, x, ldx))
         // any scheme, any mix, whole 512-element units: streams staged in LDS, eight elements per lane

@@ -636,7 +636,7 @@ k_decode358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, u
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// Product with 2..4 activation rows for dense mixes: the span walker above with a sink that multiplies.  (With one
+// Product with 2..8 activation rows for dense mixes (more than four: in two passes over the gathered weights): the span walker above with a sink that multiplies.  (With one
 // row it is cheaper to move the activations to the codes, k_gemv358_dense; with several rows the weights are
 // brought to position order once and meet every row's activations there.)
 // ---------------------------------------------------------------------------------------------------------------
@@ -685,15 +685,16 @@ struct DnDotSink {
     uint32_t out_f, spans_per_row, lane;
     bool by_rows;
     uint32_t xr[MT][16];
-    float row_total[MT];  // meaningful in lane 63
+    float row_total[2 * MT];  // meaningful in lane 63
 
-    // the lane's activations for this span, requested before the span's arithmetic starts
-    __device__ __forceinline__ void begin(const DnSpan &sp) {
+    // the lane's activations of rows j0 .. j0 + MT - 1 for this span
+    __device__ __forceinline__ void load_x(const DnSpan &sp, int j0) {
         const bool valid = 32 * lane < sp.n_el;
 #pragma unroll
         for (int j = 0; j < MT; ++j) {
-            if (valid && j < m) {
-                const uint4 *xp = reinterpret_cast<const uint4 *>(x + (int64_t)j * ldx + (size_t)sp.b * kDnSpan + 32 * lane);
+            if (valid && j0 + j < m) {
+                const uint4 *xp =
+                    reinterpret_cast<const uint4 *>(x + (int64_t)(j0 + j) * ldx + (size_t)sp.b * kDnSpan + 32 * lane);
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     const uint4 v = xp[t];
@@ -705,7 +706,17 @@ struct DnDotSink {
             }
         }
     }
+    // the first MT rows are requested before the span's arithmetic starts; rows MT .. 2 MT - 1 (if any) take their
+    // place after the first rows' products
+    __device__ __forceinline__ void begin(const DnSpan &sp) { load_x(sp, 0); }
     __device__ __forceinline__ void end(const DnSpan &sp, const uint32_t (&o)[16], uint32_t) {
+        dots(sp, o, 0);
+        if (m > MT) {
+            load_x(sp, MT);
+            dots(sp, o, MT);
+        }
+    }
+    __device__ __forceinline__ void dots(const DnSpan &sp, const uint32_t (&o)[16], int j0) {
 #pragma unroll
         for (int j = 0; j < MT; ++j) {
             float a0 = 0.0f, a1 = 0.0f;
@@ -716,18 +727,19 @@ struct DnDotSink {
             }
             const float total = dn_wave_sum(a0 + a1);
             if (by_rows) {
-                row_total[j] = (sp.b == 0 ? 0.0f : row_total[j]) + total;
-                if (sp.b + 1 == spans_per_row && lane == 63 && j < m)
-                    y[(int64_t)j * ldy + sp.a] = (uint16_t)f32_to_bf16_bits(row_total[j]);
-            } else if (lane == 63 && j < m) {
-                ws[((size_t)sp.b * m + j) * out_f + sp.a] = total;
+                float &sum = j0 == 0 ? row_total[j] : row_total[MT + j];
+                sum = (sp.b == 0 ? 0.0f : sum) + total;
+                if (sp.b + 1 == spans_per_row && lane == 63 && j0 + j < m)
+                    y[(int64_t)(j0 + j) * ldy + sp.a] = (uint16_t)f32_to_bf16_bits(sum);
+            } else if (lane == 63 && j0 + j < m) {
+                ws[((size_t)sp.b * m + j0 + j) * out_f + sp.a] = total;
             }
         }
     }
 };
 
 template <int MT>
-__global__ void __launch_bounds__(kWave *kDnWaves)
+__global__ void __launch_bounds__(kWave *kDnWaves, MT == 4 ? 3 : 4)  // waves per SIMD that the registers should allow
 k_gemv358_dense_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t spans_per_row, uint32_t n_items,
                      const uint16_t *__restrict__ x, int m, int64_t ldx, uint16_t *__restrict__ y, int64_t ldy,
                      float *__restrict__ ws, bool by_rows) {
@@ -751,12 +763,12 @@ k_gemv358_dense_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunk
     sink.x = x; sink.ldx = ldx; sink.m = m; sink.y = y; sink.ldy = ldy; sink.ws = ws;
     sink.out_f = P.out_f; sink.spans_per_row = spans_per_row; sink.lane = lane; sink.by_rows = by_rows;
 #pragma unroll
-    for (int j = 0; j < MT; ++j) sink.row_total[j] = 0.0f;
+    for (int j = 0; j < 2 * MT; ++j) sink.row_total[j] = 0.0f;
     dn_walk_spans<false>(P, prefix, P.out_f * n_chunks + 1, nullptr, 0u, lut, wc_all[wave], scale, lane, spans, sink);
 }
 
 bool gemv_dense358_rows_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x, int64_t ldx) {
-    return P.n_levels == 3 && P.bits[0] == 3 && P.bits[1] == 5 && P.bits[2] == 8 && chunk == kFastChunk && m >= 2 && m <= 4 &&
+    return P.n_levels == 3 && P.bits[0] == 3 && P.bits[1] == 5 && P.bits[2] == 8 && chunk == kFastChunk && m >= 2 && m <= 8 &&
            P.in_f % kFastChunk == 0 && P.in_f != 0 && ((uintptr_t)x & 15u) == 0 && (ldx & 7) == 0 &&
            ((uintptr_t)P.last & 3u) == 0;
 }

@@ -232,7 +232,7 @@ def run_gemv(dp, chunk, x, m, dev, flags=0, atomic=False):
 
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("shape", [(64, 512), (37, 1024), (130, 1536), (256, 4608)])
-@pytest.mark.parametrize("m", [1, 2, 3, 4, 8, 9, 13, 16])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 7, 8, 9, 13, 16])
 def test_gemv_fast_and_general(oracle, dev, kind, shape, m):
     from ixrun_amd import _lib
 
@@ -247,7 +247,7 @@ def test_gemv_fast_and_general(oracle, dev, kind, shape, m):
                                  (0, in_f, False), (0, 256, True)]:
         y = run_gemv(dp, chunk, x, m, dev, flags=flags, atomic=atomic)
         check_outputs(y, y64, f"{kind} {shape} m={m} flags={flags} chunk={chunk} atomic={atomic}")
-    if m <= 4:  # the level-by-level kernels (one row; 2..4 rows), forced also for the mixes they are not built for
+    if m <= 8:  # the level-by-level kernels (one row; 2..8 rows), forced also for the mixes they are not built for
         for atomic in (False, True):
             y = run_gemv(dp, 512, x, m, dev, flags=_lib.IXH_GEMV_DENSE, atomic=atomic)
             check_outputs(y, y64, f"{kind} {shape} m={m} level-by-level kernel atomic={atomic}")
@@ -267,7 +267,7 @@ def test_gemv_wide_rows(oracle, dev, kind, shape):
     for m in (1, 2, 4, 7):
         x = activations(m, in_f, seed=m)
         y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
-        for flags in (0, _lib.IXH_GEMV_FORCE_358, _lib.IXH_GEMV_COLUMN_KERNEL) + ((_lib.IXH_GEMV_DENSE,) if m <= 4 else ()):
+        for flags in (0, _lib.IXH_GEMV_FORCE_358, _lib.IXH_GEMV_COLUMN_KERNEL) + ((_lib.IXH_GEMV_DENSE,) if m <= 8 else ()):
             check_outputs(run_gemv(dp, 512, x, m, dev, flags=flags), y64, f"{kind} {shape} m={m} flags={flags}")
 
 
