@@ -28,9 +28,12 @@ from .quantize import int8x_quantize, portable_packed, quantize_for_deploy
 __all__ = ["Int8XEngine", "StreamingLinear", "GraphLinear", "ResourceScheduler"]
 
 MAX_FUSED_ROWS = 16  # activation rows served by the fused decode+GEMV kernel
-# With a decode buffer at hand, more rows than this go through decode + library GEMM: on 17408 x 5120 that pair takes
-# 75 us at any M up to 32, the fused kernel 70 us at M = 8 but 118 / 155 us at M = 12 / 16 (it runs four rows a pass).
+# With a decode buffer at hand, more rows than this go through decode + library GEMM.  Tensors that are almost all
+# level 1 (17408 x 5120): the pair takes 75 us at any M up to 32, the fused kernel 70 us at M = 8 but 118 / 155 us at
+# M = 12 / 16 (it runs four rows a pass).  Dense mixes (55 / 40 / 5 %): the pair takes 92 us, the fused kernels 75 / 93 /
+# 131 us at M = 2 / 4 / 8.
 MAX_FUSED_ROWS_WITH_BUFFER = 8
+MAX_FUSED_ROWS_WITH_BUFFER_DENSE = 4
 # More rows than that: with a shared decode buffer the layer decodes into it and calls the library GEMM
 # (5120 x 5120 five-level on MI355X: 60 us at 32 rows, 84 us at 512); without one it runs the fused
 # decode+GEMM, which keeps the bf16 weight out of HBM altogether but is slower (84 us and 194 us): its
@@ -126,7 +129,12 @@ class StreamingLinear(nn.Module):
 
     def forward(self, x):
         rows = x.numel() // self.in_features if self.in_features else 0
-        fused_rows = MAX_FUSED_ROWS if self._w_buf is None else MAX_FUSED_ROWS_WITH_BUFFER
+        if self._w_buf is None:
+            fused_rows = MAX_FUSED_ROWS
+        elif self.counts[0] * 100 >= self.N * 97:
+            fused_rows = MAX_FUSED_ROWS_WITH_BUFFER
+        else:
+            fused_rows = MAX_FUSED_ROWS_WITH_BUFFER_DENSE
         if (self._use_fused and x.dtype == torch.bfloat16 and x.is_cuda and 1 <= rows <= fused_rows
                 and x.shape[-1] == self.in_features):
             x2 = x.reshape(rows, self.in_features)

@@ -140,16 +140,22 @@ def test_tuned_library_gemm_on_the_many_row_path(oracle):
     assert np.array_equal(tuned, again)
 
 
-@pytest.mark.parametrize("rows", [8, 9, 16])
-def test_row_count_policy_with_a_decode_buffer(oracle, rows):
-    """Up to 8 rows the fused kernel, from 9 on decode + GEMM when the layer has a decode buffer (without one the
-    fused kernel serves up to 16): all within the many-row tolerance of the exact product."""
+@pytest.mark.parametrize("rows,dense", [(8, False), (9, False), (16, False), (4, True), (5, True)])
+def test_row_count_policy_with_a_decode_buffer(oracle, rows, dense):
+    """Up to 8 rows the fused kernel (4 for dense level mixes), beyond that decode + GEMM when the layer has a decode
+    buffer (without one the fused kernel serves up to 16): all within the many-row tolerance of the exact product."""
     from ixrun_amd.engine import StreamingLinear
     from ixrun_amd.quantize import int8x_quantize
     from helpers import student_t_weight
 
     dev = torch.device("cuda:0")
-    p = int8x_quantize(student_t_weight(128, 2048, seed=5), (3, 5, 8))
+    from helpers import calibrated_weight, int8_mix, packed_from_int8
+
+    if dense:  # 55 / 40 / 5 %
+        p = int8x_quantize(calibrated_weight(128, 2048, seed=5)[0], (3, 5, 8))
+    else:      # 99.8 % level 1
+        p = packed_from_int8(int8_mix("rare_other", 128 * 2048, seed=5), 128, 2048)
+    assert (p["counts"][0] * 100 >= p["N"] * 97) == (not dense)
     x = torch.randn(rows, 2048, generator=torch.Generator("cpu").manual_seed(rows)).bfloat16()
     w_deq = oracle.bf16_bits_to_f32(oracle.decode_packed_bf16(p)).astype(np.float64).reshape(128, 2048)
     want = torch.from_numpy(x.double().numpy() @ w_deq.T).bfloat16().double().numpy()
@@ -161,4 +167,4 @@ def test_row_count_policy_with_a_decode_buffer(oracle, rows):
         got = layer(x.to(dev)).float().cpu().numpy()
         assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-3
     decoded = bool((buf != 9.0).any())  # the buffer was written iff the pair path ran
-    assert decoded == (rows > 8)
+    assert decoded == (rows > (4 if dense else 8))
