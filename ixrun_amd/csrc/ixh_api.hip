@@ -200,7 +200,13 @@ int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, cons
     const bool fast = !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED | IXH_GEMV_DENSE)) && is_358(d) &&
                       fast358_supports(d, (uint32_t)chunk, m) &&
                       (mostly_l1 || (flags & (IXH_GEMV_COLUMN_KERNEL | IXH_GEMV_FORCE_358)));
-    if (fast && !atomic && !(flags & IXH_GEMV_COLUMN_KERNEL)) {
+    // any other scheme whose first level has 3 bits, almost all level 1: the row-block kernel with the resolver that
+    // walks the nested bitmaps (the column-block kernel is (3,5,8) only, so 5..8 rows go on to the any-scheme kernel)
+    const bool fast_any = !fast && !is_358(d) && d.n_levels >= 2 && d.bits[0] == 3 &&
+                          !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED | IXH_GEMV_DENSE | IXH_GEMV_COLUMN_KERNEL)) &&
+                          fast358_supports(d, (uint32_t)chunk, m) && (mostly_l1 || (flags & IXH_GEMV_FORCE_358)) &&
+                          (m <= 4 || m > 8);
+    if ((fast || fast_any) && !atomic && !(flags & IXH_GEMV_COLUMN_KERNEL)) {
         if (m <= 4) {
             rc = launch_gemv_358_rows(d, prefix, x, m, ldx, y, ldy, (hipStream_t)stream);
         } else if (m > 8) {

@@ -160,14 +160,50 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
 // STAGED: the workgroup's share of bitmap 1 and of the 5-bit / 8-bit streams is in LDS; that version reads
 // no global memory at all (the activations come from the wave's LDS copy), so nothing in it waits for the
 // copies the wave has in flight: a load from global memory returns behind all of them.
-template <int MT, bool STAGED>
+// ANY: any scheme whose first level has 3 bits: the element is followed down the nested bitmaps (level i: rank among
+// the elements in no level below i), every rank counted from the unit's start, where the table holds it (read
+// from global memory; tq2 and the staged side streams are not used).
+template <int MT, bool STAGED, bool ANY = false>
 __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, uint32_t tq1_addr, uint32_t tq2_addr,
                                              uint32_t unit0, const uint4 *__restrict__ queue, uint32_t count,
                                              uint32_t rowacc_addr, uint16_t *__restrict__ tasks,
                                              uint32_t xs_addr, uint32_t xs_row, uint32_t k_first,
-                                             int m, float scale, uint32_t lane) {
+                                             int m, float scale, uint32_t lane,
+                                             const int32_t *__restrict__ prefix = nullptr, uint32_t entries = 0) {
     const uint32_t *__restrict__ b2 = P.bm[1];
     const uint32_t b2_words = P.bm_words[1];
+    // value of the element at rank r of bitmap 1's domain, unit `unit`, any scheme
+    auto value_any = [&](uint32_t unit, uint32_t r) {
+        uint32_t ru = unit * kFastChunk - lds_u32(tq1_addr + (unit - unit0) * 4);  // the unit's first rank at level i
+        for (int i = 1; i + 1 < P.n_levels; ++i) {
+            const uint32_t *__restrict__ bm = P.bm[i];
+            const uint32_t words = P.bm_words[i];
+            const uint32_t qu = (uint32_t)prefix[(size_t)i * entries + unit];  // level-i elements before the unit
+            const uint32_t wf = ru >> 5, wl = min(r >> 5, wf + 17u);
+            const uint32_t first_mask = ~0u << (ru & 31);
+            uint32_t cnt = 0;
+            for (uint32_t w = wf; w < wl; ++w) {
+                uint32_t bits = w < words ? bm[w] : 0u;
+                if (w == wf) bits &= first_mask;
+                cnt += __popc(bits);
+            }
+            const uint32_t bits = wl < words ? bm[wl] : 0u;
+            uint32_t low = (1u << (r & 31)) - 1u;
+            if (wl == wf) low &= first_mask;
+            cnt += __popc(bits & low);
+            if ((bits >> (r & 31)) & 1u) {
+                const uint32_t nb = (uint32_t)P.bits[i];
+                const uint64_t bitpos = (uint64_t)(qu + cnt) * nb;
+                const uint32_t wi = (uint32_t)(bitpos >> 5), sh = (uint32_t)bitpos & 31u;
+                const uint32_t lo = wi < P.st_words[i] ? P.st[i][wi] : 0u;
+                const uint32_t hi = (sh + nb > 32 && wi + 1 < P.st_words[i]) ? P.st[i][wi + 1] : 0u;
+                return (int)((uint32_t)((((uint64_t)hi << 32) | lo) >> sh) & ((1u << nb) - 1u)) - threshold_of((int)nb);
+            }
+            r -= qu + cnt;
+            ru -= qu;
+        }
+        return r < P.last_bytes ? (int)P.last[r] - 127 : 0;
+    };
     // element `e` (bit of the record's word), the nth element above level 1 of its record
     auto one = [&](const uint4 rec, uint32_t nth, uint32_t e) {
         const uint32_t r0_lane = rec.y, unit = rec.z;
@@ -175,6 +211,13 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
         uint32_t xe[MT];  // the activations this element meets
 #pragma unroll
         for (int j = 0; j < MT; ++j) xe[j] = lds_u16(xs_addr + ((uint32_t)j * xs_row + k0 - k_first + e) * 2u);
+        if (ANY) {
+            const float w = dequant(value_any(unit, r0_lane + nth), scale);
+#pragma unroll
+            for (int j = 0; j < MT; ++j)
+                if (j < m) lds_add_f32_raw(rowacc_addr + (slot * MT + j) * 4, bf16_bits_to_f32(xe[j]) * w);
+            return;
+        }
         const uint32_t r0u = unit * kFastChunk - lds_u32(tq1_addr + (unit - unit0) * 4);
         const uint32_t q2u = lds_u32(tq2_addr + (unit - unit0) * 4);
         const uint32_t wf = r0u >> 5;
@@ -257,7 +300,7 @@ __device__ __forceinline__ void set_wave_priority(uint32_t p) {
     else __builtin_amdgcn_s_setprio(2);
 }
 
-template <int MT, int C>
+template <int MT, int C, bool ANY = false>
 __global__ void __launch_bounds__(kRMaxWaves * kWave)
 k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t quads_per_wg_arg, uint32_t flags,
                const uint16_t *__restrict__ x, int m, int64_t ldx, uint16_t *__restrict__ y, int64_t ldy
@@ -313,7 +356,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     if (!(dbg & 16))
         for (uint32_t i = tid; i <= rows_here * n_chunks; i += blockDim.x) {
             tq1[i] = (uint32_t)prefix[unit0 + i];
-            tq2[i] = (uint32_t)prefix[entries + unit0 + i];
+            if (!ANY) tq2[i] = (uint32_t)prefix[entries + unit0 + i];
         }
     const float scale = bf16_bits_to_f32(*P.scale);
     if (!(dbg & 8))
@@ -382,7 +425,8 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     // DMAs all of it (same bytes to the same place, so no barrier is needed: a wave's own loads
     // complete in order, before the first unit it waits for).
     SideView sv;
-    {
+    sv.staged = false;
+    if (!ANY) {
         const uint32_t n_local = rows_here * n_chunks;
         const uint32_t q1b = tq1[0], q2b = tq2[0], q1e = tq1[n_local], q2e = tq2[n_local];
         const uint32_t nl1b = row0 * P.in_f - q1b, nl1e = (row0 + rows_here) * P.in_f - q1e;
@@ -500,7 +544,10 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     const uint32_t rowacc_addr = (uint32_t)(uintptr_t)(lds_ptr_t)rowacc;
     auto resolve = [&]() {
         if (dbg & 128) {
-        } else if (sv.staged)
+        } else if (ANY)
+            resolve_rows<MT, false, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks, xs_addr,
+                                          C * kFastChunk, col0 * kFastChunk, m, scale, lane, prefix, entries);
+        else if (sv.staged)
             resolve_rows<MT, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks, xs_addr,
                                    C * kFastChunk, col0 * kFastChunk, m, scale, lane);
         else
@@ -642,7 +689,7 @@ static int env_int(const char *name) {
 
 constexpr size_t kLdsLimit = 160 * 1024;
 
-template <int MT, int C>
+template <int MT, int C, bool ANY>
 static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, const uint16_t *x, int m,
                        int64_t ldx, uint16_t *y, int64_t ldy, hipStream_t s) {
     static const int forced_quads = env_int("IXH_QUADS_PER_WG");
@@ -653,7 +700,7 @@ static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, c
     int per_cu = per_cu_cache[waves];
     if (per_cu == 0) {
         const size_t probe = rows_layout(min(16u, P.out_f), n_chunks, waves, MT, C).total;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rows<MT, C>, (int)(waves * kWave), probe) !=
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rows<MT, C, ANY>, (int)(waves * kWave), probe) !=
                 hipSuccess || per_cu < 1)
             per_cu = -1;
         per_cu_cache[waves] = per_cu;
@@ -679,7 +726,7 @@ static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, c
     if (lds > 64 * 1024) {
         static bool raised = false;  // per instantiation
         if (!raised) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_rows<MT, C>),
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_rows<MT, C, ANY>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit) != hipSuccess)
                 return IXH_EUNSUPPORTED;
             raised = true;
@@ -688,10 +735,10 @@ static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, c
 #ifdef IXH_VARIANTS
     static const int dbg = env_int("IXH_DBG");
     if (!g_trace) (void)hipMalloc(&g_trace, 4096 * 8 * 8);
-    hipLaunchKernelGGL((k_gemv358_rows<MT, C>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks,
+    hipLaunchKernelGGL((k_gemv358_rows<MT, C, ANY>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks,
                        quads | ((uint32_t)dbg << 16), flags, x, m, ldx, y, ldy, g_trace);
 #else
-    hipLaunchKernelGGL((k_gemv358_rows<MT, C>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks, quads,
+    hipLaunchKernelGGL((k_gemv358_rows<MT, C, ANY>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks, quads,
                        flags, x, m, ldx, y, ldy);
 #endif
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
@@ -701,12 +748,15 @@ static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, c
 // full workgroup; IXH_EUNSUPPORTED sends the caller to the column kernel.
 int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
                          int64_t ldy, hipStream_t s) {
+    const bool any = !(P.n_levels == 3 && P.bits[1] == 5);  // not (3,5,8): the resolver that walks the nested bitmaps
     if (((uintptr_t)x & 15u) != 0 || (m > 1 && (ldx & 7) != 0)) return IXH_EUNSUPPORTED;
     const uint32_t n_chunks = P.in_f / kFastChunk;
     const uint32_t c = (n_chunks + kRMaxWaves - 1) / kRMaxWaves;  // blocks per wave: a workgroup has at most kRMaxWaves waves
     const int mt = m == 1 ? 1 : (m == 2 ? 2 : (m <= 4 ? 4 : 0));
 #define IXH_ROWS(MTV, CV) \
-    if (mt == MTV && c == CV) return launch_rows<MTV, CV>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
+    if (mt == MTV && c == CV)                                                                  \
+        return any ? launch_rows<MTV, CV, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s)     \
+                   : launch_rows<MTV, CV, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
     IXH_ROWS(1, 1) IXH_ROWS(1, 2) IXH_ROWS(1, 3) IXH_ROWS(1, 4)
     IXH_ROWS(2, 1) IXH_ROWS(2, 2)
     IXH_ROWS(4, 1)

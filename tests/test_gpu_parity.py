@@ -291,6 +291,26 @@ def test_gemv_staged(oracle, dev, kind, shape, level_bits):
             check_outputs(y, y64, f"{kind} {shape} {level_bits} m={m} atomic={atomic}")
 
 
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("shape", [(64, 512), (37, 1024), (130, 1536), (24, 8704), (9, 25600)])
+@pytest.mark.parametrize("level_bits", [(3, 4, 5, 6, 8), (3, 8), (3, 3, 8), (3, 5, 6, 7, 8)])
+def test_gemv_row_block_kernel_other_schemes(oracle, dev, kind, shape, level_bits):
+    """The row-block kernel takes every scheme whose first level has 3 bits (its elements above level 1 are followed
+    down the nested bitmaps): chosen by itself for tensors that are almost all level 1, forced here for every mix;
+    1..4 rows in one launch, 9..16 rows four at a time."""
+    from ixrun_amd import _lib
+
+    out_f, in_f = shape
+    p = make_packed(kind, out_f, in_f, level_bits)
+    dp = device_packed(p, dev)
+    w_bits = oracle.decode_packed_bf16(p)
+    for m in (1, 2, 4, 9, 16):
+        x = activations(m, in_f, seed=m)
+        y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
+        for flags in (0, _lib.IXH_GEMV_FORCE_358):
+            check_outputs(run_gemv(dp, 512, x, m, dev, flags=flags), y64, f"{kind} {shape} {level_bits} m={m} flags={flags}")
+
+
 @pytest.mark.parametrize("shape,level_bits,chunk", [((40, 96), (3, 4, 5, 6, 8), 32), ((33, 100), (3, 5, 8), 50),
                                                     ((64, 1024), (3, 4, 5, 6, 8), 512), ((9, 7), (2, 8), 7)])
 def test_gemv_general_shapes_and_schemes(oracle, dev, shape, level_bits, chunk):
