@@ -386,32 +386,21 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
 
     const uint32_t col0 = wave * C;
 
-    // this lane's activations: C blocks x MT rows x 16 packed bf16 pairs
-    uint32_t xr[C][MT][16];
+    // The wave's activations (C blocks x MT rows x 512 bf16) go to its LDS area by LDS-DMA, 1 KB per instruction, and
+    // from there into registers once the first copies have landed: one request per byte of x and wave (the four
+    // 16-lane rows need the same bytes), and nothing waits for x before the ring's first copies are on their way.
+    {
+        const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)x, 0, (int)((((int64_t)(m - 1) * ldx + P.in_f) * 2)), 0x00020000);
 #pragma unroll
-    for (int cc = 0; cc < C; ++cc) {
-        const uint32_t col = min(col0 + cc, n_chunks - 1);
+        for (int cc = 0; cc < C; ++cc) {
+            const uint32_t col = min(col0 + cc, n_chunks - 1);
 #pragma unroll
-        for (int j = 0; j < MT; ++j) {
-            if (j < m && !(dbg & 32)) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const uint4 v = reinterpret_cast<const uint4 *>(x + (int64_t)j * ldx + col * kFastChunk + li * 32)[t];
-                    xr[cc][j][4 * t] = v.x; xr[cc][j][4 * t + 1] = v.y;
-                    xr[cc][j][4 * t + 2] = v.z; xr[cc][j][4 * t + 3] = v.w;
-                }
-            } else {
-#pragma unroll
-                for (int t = 0; t < 16; ++t) xr[cc][j][t] = 0u;
-            }
-            // The wave's LDS copy.  All four 16-lane rows write (the same values to the same place) on purpose:
-            // a store under a lane condition would leave the loads above "possibly pending" on the path around
-            // it, and the compiler would then wait for them inside the main loop, where the wait also covers
-            // the copies in flight.
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-                *reinterpret_cast<u32x4 *>(xs + (j * C + cc) * (kFastChunk / 2) + li * 16 + 4 * t) =
-                    u32x4{xr[cc][j][4 * t], xr[cc][j][4 * t + 1], xr[cc][j][4 * t + 2], xr[cc][j][4 * t + 3]};
+            for (int j = 0; j < MT; ++j)
+                if (j < m && !(dbg & 32))
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                        x_rsrc, (lds_ptr_t)(xs + (j * C + cc) * (kFastChunk / 2)), 16,
+                        (int)(((int64_t)j * ldx + col * kFastChunk) * 2 + lane * 16), 0, 0, 0);
         }
     }
 
@@ -562,6 +551,26 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     if (n_units >= (uint32_t)kRStages) wait_vmem<2 * (kRStages - 1)>();
     else wait_vmem<0>();
     IXH_STAMP(2);
+
+    // this lane's activations: C blocks x MT rows x 16 packed bf16 pairs
+    uint32_t xr[C][MT][16];
+#pragma unroll
+    for (int cc = 0; cc < C; ++cc)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            if (j < m && !(dbg & 32)) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const u32x4 v = lds_u128((uint32_t)(uintptr_t)(lds_ptr_t)xs +
+                                             (((uint32_t)(j * C + cc) * (kFastChunk / 2) + li * 16 + 4 * t) * 4u));
+                    xr[cc][j][4 * t] = v.x; xr[cc][j][4 * t + 1] = v.y;
+                    xr[cc][j][4 * t + 2] = v.z; xr[cc][j][4 * t + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 16; ++t) xr[cc][j][t] = 0u;
+            }
+        }
 
     uint32_t lrn_step = min(quarter, rows_here - 1) * n_chunks;  // local row * n_chunks of the current step
     bool valid_step = quarter < rows_here;
