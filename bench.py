@@ -50,6 +50,8 @@ WORKLOADS = {
     "down_proj_5120x17408_m1_calibrated": (5120, 17408, 1, "calibrated"),
     "down_proj_5120x17408_m1_five_level": (5120, 17408, 1, "student_t", (3, 4, 5, 6, 8)),
     "attn_proj_5120x5120_m1_five_level": (5120, 5120, 1, "student_t", (3, 4, 5, 6, 8)),
+    "attn_proj_5120x5120_m1_calibrated": (5120, 5120, 1, "calibrated"),
+    "graph64_5120x5120_m1_calibrated": (5120, 5120, 1, "calibrated"),
     "attn_proj_5120x5120_m1_student_t": (5120, 5120, 1, "student_t"),
     "gate_up_17408x5120_m2_student_t": (17408, 5120, 2, "student_t"),
     "gate_up_17408x5120_m4_student_t": (17408, 5120, 4, "student_t"),
