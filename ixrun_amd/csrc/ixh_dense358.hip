@@ -108,6 +108,14 @@ k_gemv358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
       const uint32_t k_end = by_rows ? spans_per_row : k_first + 1u;
       float row_total = 0.0f;  // meaningful in lane 63
       for (uint32_t k = k_first; k < k_end; ++k) {
+        // The waves that share a SIMD take turns at the issue priority, one span each: all of them start their rows
+        // together, and this keeps them from meeting at the same phase (scatter, dense passes) span after span.
+        {
+            const uint32_t turn = (wave + k) % 3u;  // s_setprio takes an immediate
+            if (turn == 0) __builtin_amdgcn_s_setprio(0);
+            else if (turn == 1) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(2);
+        }
         const uint32_t c0 = 4 * k, nb = min(4u, n_chunks - c0);
         const uint32_t u0 = row * n_chunks + c0;
         const uint32_t n_el = nb * kFastChunk, p0 = u0 * kFastChunk;
