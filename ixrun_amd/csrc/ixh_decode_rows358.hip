@@ -458,6 +458,13 @@ k_decode358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_quads, ui
     const uint32_t rd_addr = tile_addr + (quarter * 16u + (li >> 2)) * 80u + (li & 3u) * 16u;
 
     for (uint32_t i = 0; i < n_mine; ++i) {
+        // the waves that share a SIMD (wave, wave + 4, wave + 8) take turns at the issue priority, one unit-quad each
+        {
+            const uint32_t pr = ((wave >> 2) + i) % 3u;  // s_setprio takes an immediate
+            if (pr == 0) __builtin_amdgcn_s_setprio(0);
+            else if (pr == 1) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(2);
+        }
         // Room for a full wave of records.  Only the records of units whose rows are stored may be resolved: the
         // current unit's (at most 64, at the queue's end) move to its front.
         if (qcount > kDrQueue - kWave) {

@@ -358,7 +358,7 @@ template <bool GS, class Spans, class Sink>
 __device__ __forceinline__ void dn_walk_spans(const Dev &P, const int32_t *__restrict__ prefix, uint32_t entries,
                                               const uint16_t *__restrict__ group_scales, uint32_t group_shift,
                                               const uint32_t *lut, uint16_t *wc, float scale, uint32_t lane,
-                                              const Spans &spans, Sink &sink) {
+                                              const Spans &spans, Sink &sink, uint32_t wave_turn) {
     const float m15 = -15.0f * scale, m127 = -127.0f * scale;
     uint32_t *const wc32 = reinterpret_cast<uint32_t *>(wc);
     const uint32_t lut_lane = (lane & 31u) << 2;
@@ -426,7 +426,15 @@ __device__ __forceinline__ void dn_walk_spans(const Dev &P, const int32_t *__res
     Ranks q_now = table_of(sp_now);
     Loads in_now = fetch(sp_now, q_now);
     Ranks q_next = table_of(sp_next);
-    for (;;) {
+    for (uint32_t turn = wave_turn;; ++turn) {
+        // the waves that share a SIMD take turns at the issue priority, one span each, so that they do not meet at the
+        // same phase (dequantise, gather, store or multiply) span after span
+        {
+            const uint32_t pr = turn % 3u;  // s_setprio takes an immediate
+            if (pr == 0) __builtin_amdgcn_s_setprio(0);
+            else if (pr == 1) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(2);
+        }
         const Loads in_next = fetch(sp_next, q_next);
         const Ranks q_after = table_of(sp_after);
         sink.begin(sp_now);
@@ -640,7 +648,7 @@ k_decode358_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, u
     __syncthreads();
     const DnFlatSpans spans{n_units, n_spans, P.n, blockIdx.x * kDnWaves + wave, gridDim.x * kDnWaves};
     DnStoreSink sink{out, wc_all[wave], lane};
-    dn_walk_spans<GS>(P, prefix, n_units + 1, group_scales, group_shift, lut, wc_all[wave], scale, lane, spans, sink);
+    dn_walk_spans<GS>(P, prefix, n_units + 1, group_scales, group_shift, lut, wc_all[wave], scale, lane, spans, sink, wave);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -772,7 +780,7 @@ k_gemv358_dense_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunk
     sink.out_f = P.out_f; sink.spans_per_row = spans_per_row; sink.lane = lane; sink.by_rows = by_rows;
 #pragma unroll
     for (int j = 0; j < 2 * MT; ++j) sink.row_total[j] = 0.0f;
-    dn_walk_spans<false>(P, prefix, P.out_f * n_chunks + 1, nullptr, 0u, lut, wc_all[wave], scale, lane, spans, sink);
+    dn_walk_spans<false>(P, prefix, P.out_f * n_chunks + 1, nullptr, 0u, lut, wc_all[wave], scale, lane, spans, sink, wave);
 }
 
 bool gemv_dense358_rows_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x, int64_t ldx) {
