@@ -163,7 +163,9 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
 // ANY: any scheme whose first level has 3 bits: the element is followed down the nested bitmaps (level i: rank among
 // the elements in no level below i), every rank counted from the unit's start, where the table holds it (read
 // from global memory; tq2 and the staged side streams are not used).
-template <int MT, bool STAGED, bool ANY = false>
+// XSW: the activations are the workgroup's shared, swizzled copy of the whole x row (one activation row): 16-byte
+// piece p of the 64 bytes that lane l of a 16-lane row owns in a column block sits at piece p * 16 + l of the block.
+template <int MT, bool STAGED, bool ANY = false, bool XSW = false>
 __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, uint32_t tq1_addr, uint32_t tq2_addr,
                                              uint32_t unit0, const uint4 *__restrict__ queue, uint32_t count,
                                              uint32_t rowacc_addr, uint16_t *__restrict__ tasks,
@@ -206,11 +208,20 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
     };
     // element `e` (bit of the record's word), the nth element above level 1 of its record
     auto one = [&](const uint4 rec, uint32_t nth, uint32_t e) {
-        const uint32_t r0_lane = rec.y, unit = rec.z;
-        const uint32_t slot = rec.w >> 16, k0 = rec.w & 0xFFFFu;
+        uint32_t r0_lane = rec.y, unit = rec.z, k0 = rec.w & 0xFFFFu;
+        const uint32_t slot = rec.w >> 16;
+        if (XSW) {  // the shared-x kernel's records: rank offset in the unit, local unit, column block << 4 | lane
+            const uint32_t in_unit = (rec.w & 15u) * 32u;
+            unit = unit0 + rec.z;
+            r0_lane = unit * kFastChunk + in_unit - (lds_u32(tq1_addr + rec.z * 4) + rec.y);
+            k0 = ((rec.w >> 4) & 0xFFFu) * kFastChunk + in_unit;
+        }
         uint32_t xe[MT];  // the activations this element meets
 #pragma unroll
-        for (int j = 0; j < MT; ++j) xe[j] = lds_u16(xs_addr + ((uint32_t)j * xs_row + k0 - k_first + e) * 2u);
+        for (int j = 0; j < MT; ++j)
+            xe[j] = XSW ? lds_u16(xs_addr + (k0 >> 9) * (kFastChunk * 2) + (((e >> 3) * 16u + ((k0 >> 5) & 15u)) * 16u) +
+                                  (e & 7u) * 2u)
+                        : lds_u16(xs_addr + ((uint32_t)j * xs_row + k0 - k_first + e) * 2u);
         if (ANY) {
             const float w = dequant(value_any(unit, r0_lane + nth), scale);
 #pragma unroll
@@ -681,6 +692,340 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
 }
 
 // ---------------------------------------------------------------------------
+// One activation row, x shared by the workgroup
+// ---------------------------------------------------------------------------
+// Same decode as k_gemv358_rows, different work split.  There a wave owns column blocks and keeps their activations
+// in registers, which ties the number of waves to the number of column blocks (12 waves, three per SIMD, for 34
+// blocks) and makes every wave walk 15 unit-quads one after the other.  Here the whole activation row sits in LDS
+// once per workgroup (swizzled, so that the 16 lanes of a row read consecutive 16-byte pieces), the workgroup's
+// unit-quads are dealt round-robin to as many waves as LDS allows (16: four per SIMD), and a wave reads the 64
+// activation bytes of a lane afresh for every unit-quad (four ds_read_b128).  The chain of dependent steps a wave
+// walks is a quarter shorter and a SIMD has one more wave to issue from.
+constexpr int kXMaxWaves = 16;
+
+__host__ __device__ constexpr uint32_t wave_lds_bytes_x() {
+    return kRStages * kRStageBytes + kRQueue * 16 + kRSlots * 4 + kRTasks * 2;
+}
+
+struct RowsXLds {
+    uint32_t tq1, tq2, side, xs, waves, total;
+};
+
+__host__ __device__ inline RowsXLds rowsx_layout(uint32_t rows_cap, uint32_t n_chunks, uint32_t n_waves) {
+    RowsXLds L;
+    const uint32_t tbl = ((rows_cap * n_chunks + 1u + 3u) & ~3u) * 4u;
+    L.tq1 = kRLutBytes + kRSpliceBytes;
+    L.tq2 = L.tq1 + tbl;
+    L.side = L.tq2 + tbl;
+    L.xs = L.side + kRSideBytes;
+    L.waves = L.xs + n_chunks * kFastChunk * 2;
+    L.total = L.waves + n_waves * wave_lds_bytes_x();
+    return L;
+}
+
+template <bool ANY>
+__global__ void __launch_bounds__(kXMaxWaves * kWave)
+k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t quads_per_wg, uint32_t flags,
+                const uint16_t *__restrict__ x, uint16_t *__restrict__ y) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t n_waves = blockDim.x >> 6;
+    const uint32_t quarter = lane >> 4, li = lane & 15;
+
+    const uint32_t n_quads = (P.out_f + 3) >> 2;
+    const uint32_t quad0 = blockIdx.x * quads_per_wg;
+    const uint32_t n_steps = min(quads_per_wg, n_quads - quad0);
+    const uint32_t row0 = quad0 * 4;
+    const uint32_t rows_here = min(n_steps * 4, P.out_f - row0);
+    const RowsXLds L = rowsx_layout(min(quads_per_wg * 4, P.out_f), n_chunks, n_waves);
+
+    // the pair table is addressed with (index bits | lane bits): it must sit at LDS address 0
+    if ((uint32_t)(uintptr_t)(lds_ptr_t)smem != 0) {
+        for (uint32_t t = tid; t < rows_here; t += blockDim.x) y[row0 + t] = 0x7FC0;  // NaN
+        return;
+    }
+    uint32_t *const lut = reinterpret_cast<uint32_t *>(smem);            // [64][32]
+    uint4 *const splice = reinterpret_cast<uint4 *>(smem + kRLutBytes);  // [33][2]
+    uint32_t *const tq1 = reinterpret_cast<uint32_t *>(smem + L.tq1);
+    uint32_t *const tq2 = reinterpret_cast<uint32_t *>(smem + L.tq2);
+    uint8_t *const wave_base = smem + L.waves + wave * wave_lds_bytes_x();
+    uint8_t *const ring = wave_base;
+    uint4 *const queue = reinterpret_cast<uint4 *>(wave_base + kRStages * kRStageBytes);
+    float *const rowacc = reinterpret_cast<float *>(wave_base + kRStages * kRStageBytes + kRQueue * 16);
+    uint16_t *const tasks = reinterpret_cast<uint16_t *>(rowacc + kRSlots);
+
+    // ---- the activation row: needs nothing but the arguments, so it is requested first.  Lane (t, l) of the copy
+    // fetches piece l * 4 + t of the block and the hardware puts it at piece t * 16 + l.
+    {
+        const __amdgpu_buffer_rsrc_t x_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, (int)(P.in_f * 2u), 0x00020000);
+        for (uint32_t col = wave; col < n_chunks; col += n_waves)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (lds_ptr_t)(smem + L.xs + col * (kFastChunk * 2)), 16,
+                                                     (int)(col * (kFastChunk * 2) + (li * 4u + quarter) * 16u), 0, 0,
+                                                     0);
+    }
+
+    // ---- workgroup set-up: table slices, pair table, splice masks ----
+    const uint32_t unit0 = row0 * n_chunks;
+    const uint32_t entries = P.out_f * n_chunks + 1;
+    for (uint32_t i = tid; i <= rows_here * n_chunks; i += blockDim.x) {
+        tq1[i] = (uint32_t)prefix[unit0 + i];
+        if (!ANY) tq2[i] = (uint32_t)prefix[entries + unit0 + i];
+    }
+    const float scale = bf16_bits_to_f32(*P.scale);
+    for (uint32_t i = tid; i < 64 * 32; i += blockDim.x) {
+        const int c0 = (i >> 5) & 7, c1 = i >> 8;
+        const uint32_t w0 = c0 < 7 ? f32_to_bf16_bits((float)(c0 - 3) * scale) : 0u;
+        const uint32_t w1 = c1 < 7 ? f32_to_bf16_bits((float)(c1 - 3) * scale) : 0u;
+        lut[i] = w0 | (w1 << 16);
+    }
+    if (tid <= 32) {
+        const uint32_t pos = 3 * tid;
+        uint32_t lm[3], f[3];
+#pragma unroll
+        for (int d = 0; d < 3; ++d) {
+            const uint32_t base = 32u * d;
+            lm[d] = pos <= base ? 0u : (pos >= base + 32 ? ~0u : (1u << (pos - base)) - 1u);
+            f[d] = (pos + 3 <= base || pos >= base + 32) ? 0u : (pos >= base ? 7u << (pos - base) : 7u >> (base - pos));
+        }
+        splice[2 * tid] = make_uint4(lm[0], lm[1], lm[2], 0u);
+        splice[2 * tid + 1] = make_uint4(f[0], f[1], f[2], 0u);
+    }
+    for (uint32_t j = lane; j < kRSlots; j += kWave) rowacc[j] = 0.0f;
+    wait_vmem<0>();  // this wave's pieces of x are in LDS
+    __syncthreads();
+
+    const __amdgpu_buffer_rsrc_t b1_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[0], 0, (int)(P.bm_words[0] * 4u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t l1_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[0], 0, (int)(P.st_words[0] * 4u), 0x00020000);
+
+    // ---- this workgroup's share of bitmap 1 and of the 5-bit / 8-bit streams (as in k_gemv358_rows) ----
+    SideView sv;
+    sv.staged = false;
+    if (!ANY) {
+        const uint32_t n_local = rows_here * n_chunks;
+        const uint32_t q1b = tq1[0], q2b = tq2[0], q1e = tq1[n_local], q2e = tq2[n_local];
+        const uint32_t nl1b = row0 * P.in_f - q1b, nl1e = (row0 + rows_here) * P.in_f - q1e;
+        sv.base = L.side;
+        sv.b2w0 = nl1b >> 5;
+        sv.l2w0 = (uint32_t)(((uint64_t)q2b * 5u) >> 5);
+        sv.l3w0 = (nl1b - q2b) >> 2;
+        const uint32_t n_b2 = ((nl1e + 31) >> 5) - sv.b2w0;
+        const uint32_t n_l2 = (uint32_t)((((uint64_t)q2e * 5u) + 31) >> 5) - sv.l2w0;
+        const uint32_t n_l3 = ((nl1e - q2e + 3) >> 2) - sv.l3w0;
+        sv.staged = (flags & kFlagStageSide) && n_b2 < 256 && n_l2 < 511 && n_l3 <= 256;
+        if (sv.staged) {
+            const __amdgpu_buffer_rsrc_t b2_rsrc =
+                __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[1], 0, (int)(P.bm_words[1] * 4u), 0x00020000);
+            const __amdgpu_buffer_rsrc_t l2_rsrc =
+                __builtin_amdgcn_make_buffer_rsrc((void *)P.st[1], 0, (int)(P.st_words[1] * 4u), 0x00020000);
+            const __amdgpu_buffer_rsrc_t l3_rsrc =
+                __builtin_amdgcn_make_buffer_rsrc((void *)P.last, 0, (int)((P.last_bytes + 3u) & ~3u), 0x00020000);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(b2_rsrc, (lds_ptr_t)(smem + L.side + kRSideB2), 16,
+                                                     (int)(sv.b2w0 * 4 + lane * 16), 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(l2_rsrc, (lds_ptr_t)(smem + L.side + kRSideL2), 16,
+                                                     (int)(sv.l2w0 * 4 + lane * 16), 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(l2_rsrc, (lds_ptr_t)(smem + L.side + kRSideL2 + 1024), 16,
+                                                     (int)(sv.l2w0 * 4 + 1024 + lane * 16), 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(l3_rsrc, (lds_ptr_t)(smem + L.side + kRSideL3), 16,
+                                                     (int)(sv.l3w0 * 4 + lane * 16), 0, 0, 0);
+        }
+    }
+
+    const uint32_t lut_lane = (lane & 31u) << 2;
+    const uint32_t splice_addr = kRLutBytes;
+    const uint32_t tq1_addr = L.tq1, tq2_addr = L.tq2;
+    const uint32_t ring_addr = (uint32_t)(uintptr_t)(lds_ptr_t)ring;
+    const uint32_t xs_addr = L.xs;
+    const uint32_t rowacc_addr = (uint32_t)(uintptr_t)(lds_ptr_t)rowacc;
+
+    // The workgroup's unit-quads in walk order are u = step * n_chunks + col; this wave takes u = wave, wave +
+    // n_waves, ...  A cursor is the (step, col) of one of them and moves on by n_waves.
+    const uint32_t n_total = n_steps * n_chunks;
+    const uint32_t n_mine = wave < n_total ? (n_total - wave + n_waves - 1) / n_waves : 0u;
+    const uint32_t dq = n_waves / n_chunks, dr = n_waves - dq * n_chunks;
+    struct Cur {
+        uint32_t step, col;
+    };
+    auto advance = [&](Cur &c) {
+        c.step += dq;
+        c.col += dr;
+        if (c.col >= n_chunks) {
+            c.col -= n_chunks;
+            ++c.step;
+        }
+    };
+    Cur c_issue = {wave / n_chunks, wave % n_chunks};
+    Cur c_now = c_issue, c_next = c_issue;
+    advance(c_next);
+
+    uint32_t st_issue = 0;  // ring stage the next copy goes to
+    auto issue = [&]() {
+        const uint32_t lrn = __umul24(min(4 * c_issue.step + quarter, rows_here - 1), n_chunks);
+        const uint32_t q1u = lds_u32(tq1_addr + (lrn + c_issue.col) * 4);
+        const uint32_t unit = unit0 + lrn + c_issue.col;
+        uint8_t *stage = ring + st_issue * kRStageBytes;
+        asm volatile("" ::: "memory");
+        if (li < 13)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(l1_rsrc, (lds_ptr_t)stage, 16,
+                                                     (int)(((q1u * 3u) >> 5) * 4u + li * 16u), 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(b1_rsrc, (lds_ptr_t)(stage + 1024), 4, (int)((unit * 16u + li) * 4u),
+                                                 0, 0, 0);
+        st_issue = st_issue + 1 == (uint32_t)kRStages ? 0u : st_issue + 1;
+        advance(c_issue);
+    };
+
+    uint32_t qcount = 0;  // wave-uniform
+
+    auto splice_once = [&](uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &zrem) {
+        const uint32_t e = zrem != 0 ? (uint32_t)__builtin_ctz(zrem) : 32u;
+        zrem &= zrem - 1;
+        const u32x4 lm = lds_u128(splice_addr + e * 32), fm = lds_u128(splice_addr + e * 32 + 16);
+        const uint32_t s0 = w0 << 3;
+        const uint32_t s1 = __builtin_amdgcn_alignbit(w1, w0, 29);
+        const uint32_t s2 = __builtin_amdgcn_alignbit(w2, w1, 29);
+        w0 = (w0 & lm.x) | (s0 & ~lm.x);
+        w1 = (w1 & lm.y) | (s1 & ~lm.y);
+        w2 = (w2 & lm.z) | (s2 & ~lm.z);
+        w0 = (w0 & ~fm.x) | (kZeroCodes0 & fm.x);
+        w1 = (w1 & ~fm.y) | (kZeroCodes1 & fm.y);
+        w2 = (w2 & ~fm.z) | (kZeroCodes2 & fm.z);
+    };
+
+    // Code window of the unit-quad at cursor c, whose data is in ring stage `st`, spliced once.  A row quad that
+    // reaches past the workgroup's last row repeats that row: its sums go to row slots nobody reads.
+    // A lane with elements above level 1 leaves a record: {their bitmap bits, the lane's rank offset inside the
+    // unit, the unit's index in the workgroup's table slice, row slot << 16 | column block << 4 | lane of the row}.
+    const uint32_t rec_lane = (quarter << 16) | li;
+    auto open_window = [&](uint32_t st, const Cur &c, uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &zrem) {
+        const uint32_t lu = __umul24(min(4 * c.step + quarter, rows_here - 1), n_chunks) + c.col;
+        const uint32_t stage = ring_addr + st * kRStageBytes;
+        const uint32_t word = lds_u32(stage + 1024 + lane * 4);
+        const uint32_t q1u = lds_u32(tq1_addr + lu * 4);
+        const uint32_t cnt = __popc(word);
+        const uint32_t excl = row_scan(cnt) - cnt;
+        const uint32_t off = __umul24(excl, 3u) + ((q1u * 3u) & 31u);
+        const uint32_t wa = stage + quarter * 256 + (off >> 5) * 4;
+        const uint32_t d0 = lds_u32(wa), d1 = lds_u32(wa + 4), d2 = lds_u32(wa + 8), d3 = lds_u32(wa + 12);
+        w0 = __builtin_amdgcn_alignbit(d1, d0, off);
+        w1 = __builtin_amdgcn_alignbit(d2, d1, off);
+        w2 = __builtin_amdgcn_alignbit(d3, d2, off);
+        const uint32_t zeros = ~word;
+        const uint64_t any = __ballot(zeros != 0);
+        if (zeros != 0)
+            push_record(queue, qcount + lanes_below(any),
+                        make_uint4(zeros, excl, lu, rec_lane + ((c.step << 18) | (c.col << 4))));
+        qcount += (uint32_t)__popcll(any);
+        zrem = zeros;
+        splice_once(w0, w1, w2, zrem);
+    };
+
+    auto resolve = [&]() {
+        if (ANY)
+            resolve_rows<1, false, true, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
+                                               xs_addr, 0, 0, 1, scale, lane, prefix, entries);
+        else if (sv.staged)
+            resolve_rows<1, true, false, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
+                                               xs_addr, 0, 0, 1, scale, lane);
+        else
+            resolve_rows<1, false, false, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
+                                                xs_addr, 0, 0, 1, scale, lane);
+        qcount = 0;
+    };
+
+    if (n_mine > 0) {
+        const uint32_t n_pre = min((uint32_t)kRStages, n_mine);
+        for (uint32_t i = 0; i < n_pre; ++i) issue();
+        if (n_mine >= (uint32_t)kRStages) wait_vmem<2 * (kRStages - 1)>();
+        else wait_vmem<0>();
+
+        uint32_t cw0, cw1, cw2, czrem;
+        open_window(0, c_now, cw0, cw1, cw2, czrem);
+        while (__ballot(czrem != 0) != 0) splice_once(cw0, cw1, cw2, czrem);
+        uint32_t st_now = 0;  // ring stage of the unit-quad whose window is open
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+
+        for (uint32_t i = 0; i < n_mine; ++i) {
+            // the waves that share a SIMD take turns at the issue priority (see k_gemv358_rows)
+            __builtin_amdgcn_s_setprio(0);
+            const uint32_t turn = ((wave >> 2) + i) & 3u;
+            if (turn == 1) __builtin_amdgcn_s_setprio(1);
+            else if (turn == 2) __builtin_amdgcn_s_setprio(2);
+            else if (turn == 3) __builtin_amdgcn_s_setprio(3);
+
+            if (qcount > kRQueue - kWave) resolve();  // keep room for a full wave of records
+            // refill the stage whose window was read last time (it is st_issue); make unit i+1 readable
+            if (i + kRStages < n_mine) {
+                issue();
+                wait_vmem<2 * (kRStages - 1)>();
+            } else {
+                wait_vmem<0>();
+            }
+
+            // this lane's 16 activation pairs of the column block
+            uint32_t xr[16];
+            {
+                const uint32_t xa = xs_addr + c_now.col * (kFastChunk * 2) + li * 16u;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const u32x4 v = lds_u128(xa + (uint32_t)t * 256u);
+                    xr[4 * t] = v.x; xr[4 * t + 1] = v.y; xr[4 * t + 2] = v.z; xr[4 * t + 3] = v.w;
+                }
+            }
+
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const int bit = 6 * t, ob = bit & 31, d = bit >> 5;
+                const uint32_t lo = d == 0 ? cw0 : (d == 1 ? cw1 : cw2);
+                const uint32_t hi = d == 0 ? cw1 : cw2;
+                uint32_t a;  // pair index at bits 12..7
+                if (ob > 26) a = __builtin_amdgcn_alignbit(hi, lo, ob - 7);
+                else if (ob >= 7) a = lo >> (ob - 7);
+                else a = lo << (7 - ob);
+                const uint32_t wp = lds_u32((a & 0x1F80u) | lut_lane);
+                acc[t % 4] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, wp),
+                                                             __builtin_bit_cast(bf16x2, xr[t]), acc[t % 4], false);
+            }
+
+            // window of this wave's next unit-quad
+            const uint32_t st_next = st_now + 1 == (uint32_t)kRStages ? 0u : st_now + 1;
+            const bool more = i + 1 < n_mine;
+            if (more) {
+                uint32_t nzrem;
+                open_window(st_next, c_next, cw0, cw1, cw2, nzrem);
+                while (__ballot(nzrem != 0) != 0) splice_once(cw0, cw1, cw2, nzrem);
+            }
+
+            // the lane's sum stays in its register while the wave's next unit-quad is in the same row quad
+            if (!more || c_next.step != c_now.step) {
+                const float total = row_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
+                if (li == 15) rowacc[4 * c_now.step + quarter] += total;
+                acc[0] = acc[1] = acc[2] = acc[3] = 0.0f;
+            }
+
+            st_now = st_next;
+            c_now = c_next;
+            advance(c_next);
+        }
+        __builtin_amdgcn_s_setprio(0);
+        resolve();
+    }
+    __syncthreads();
+
+    // ---- add the waves' row sums in wave order, write bf16 ----
+    const uint32_t first_acc = L.waves + kRStages * kRStageBytes + kRQueue * 16;
+    for (uint32_t t = tid; t < rows_here; t += blockDim.x) {
+        float sum = 0.0f;
+        for (uint32_t w = 0; w < n_waves; ++w)
+            sum += *reinterpret_cast<const float *>(smem + first_acc + w * wave_lds_bytes_x() + t * 4);
+        y[row0 + t] = (uint16_t)f32_to_bf16_bits(sum);
+    }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 #ifdef IXH_VARIANTS
@@ -753,6 +1098,58 @@ static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, c
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }
 
+// The shared-x kernel for one activation row: as many waves as LDS allows (16, 12 or 8); IXH_EUNSUPPORTED when the
+// activation row does not fit beside them.
+template <bool ANY>
+static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, const uint16_t *x, uint16_t *y,
+                        hipStream_t s) {
+    const uint32_t n_quads = (P.out_f + 3) / 4;
+    static const int n_cu = [] {
+        int dev = 0, v = 256;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
+        return v;
+    }();
+    static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_rowsx<ANY>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                   (int)kLdsLimit) == hipSuccess;  // per instantiation
+    if (!raised) return IXH_EUNSUPPORTED;
+    // the last answer is kept: a model asks for the same few shapes over and over
+    static uint32_t k_chunks = 0, k_out = 0, k_waves = 0, k_quads = 0;
+    if (k_chunks != n_chunks || k_out != P.out_f) {
+        uint32_t waves = 0, quads = 0;
+        for (uint32_t w : {16u, 12u, 8u}) {
+            const size_t probe = rowsx_layout(min(16u, P.out_f), n_chunks, w).total;
+            int per_cu = 0;
+            if (probe > kLdsLimit ||
+                hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rowsx<ANY>, (int)(w * kWave), probe) !=
+                    hipSuccess || per_cu < 1)
+                continue;
+            // whole rounds of resident workgroups, each with a contiguous run of at most 16 row quads
+            const uint32_t resident = (uint32_t)n_cu * (uint32_t)per_cu;
+            const uint32_t rounds = (n_quads + resident * (kRSlots / 4) - 1) / (resident * (kRSlots / 4));
+            uint32_t q = (n_quads + rounds * resident - 1) / (rounds * resident);
+            q = max(1u, min(q, kRSlots / 4));
+            if (rowsx_layout(min(q * 4, P.out_f), n_chunks, w).total > kLdsLimit) continue;
+            waves = w;
+            quads = q;
+            break;
+        }
+        k_chunks = n_chunks;
+        k_out = P.out_f;
+        k_waves = waves;
+        k_quads = quads;
+    }
+    if (k_waves == 0) return IXH_EUNSUPPORTED;
+    const uint32_t waves = k_waves, quads = k_quads;
+    const uint32_t groups = (n_quads + quads - 1) / quads;
+    uint32_t flags = 0;
+    if (((uintptr_t)P.last & 3u) == 0) flags |= kFlagStageSide;
+    const size_t lds = rowsx_layout(min(quads * 4, P.out_f), n_chunks, waves).total;
+    hipLaunchKernelGGL((k_gemv358_rowsx<ANY>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks, quads,
+                       flags, x, y);
+    return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
+}
+
 // Row-block kernel for the shapes whose x slices fit the register budget of a
 // full workgroup; IXH_EUNSUPPORTED sends the caller to the column kernel.
 int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
@@ -760,6 +1157,11 @@ int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x,
     const bool any = !(P.n_levels == 3 && P.bits[1] == 5);  // not (3,5,8): the resolver that walks the nested bitmaps
     if (((uintptr_t)x & 15u) != 0 || (m > 1 && (ldx & 7) != 0)) return IXH_EUNSUPPORTED;
     const uint32_t n_chunks = P.in_f / kFastChunk;
+    static const int shared_x = getenv("IXH_GEMV_SHARED_X") ? atoi(getenv("IXH_GEMV_SHARED_X")) : 1;
+    if (m == 1 && shared_x && P.in_f <= 65536u) {
+        const int rc = any ? launch_rowsx<true>(P, prefix, n_chunks, x, y, s) : launch_rowsx<false>(P, prefix, n_chunks, x, y, s);
+        if (rc != IXH_EUNSUPPORTED) return rc;
+    }
     const uint32_t c = (n_chunks + kRMaxWaves - 1) / kRMaxWaves;  // blocks per wave: a workgroup has at most kRMaxWaves waves
     const int mt = m == 1 ? 1 : (m == 2 ? 2 : (m <= 4 ? 4 : 0));
 #define IXH_ROWS(MTV, CV) \
