@@ -210,10 +210,11 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
     auto one = [&](const uint4 rec, uint32_t nth, uint32_t e) {
         uint32_t r0_lane = rec.y, unit = rec.z, k0 = rec.w & 0xFFFFu;
         const uint32_t slot = rec.w >> 16;
-        if (XSW) {  // the shared-x kernel's records: rank offset in the unit, local unit, column block << 4 | lane
+        if (XSW) {  // the shared-x kernel's records: rank offset in the unit, LDS address of the unit's table
+                    // entry, column block << 4 | lane
             const uint32_t in_unit = (rec.w & 15u) * 32u;
-            unit = unit0 + rec.z;
-            r0_lane = unit * kFastChunk + in_unit - (lds_u32(tq1_addr + rec.z * 4) + rec.y);
+            unit = unit0 + ((rec.z - tq1_addr) >> 2);
+            r0_lane = unit * kFastChunk + in_unit - (lds_u32(rec.z) + rec.y);
             k0 = ((rec.w >> 4) & 0xFFFu) * kFastChunk + in_unit;
         }
         uint32_t xe[MT];  // the activations this element meets
@@ -843,12 +844,14 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     const uint32_t rowacc_addr = (uint32_t)(uintptr_t)(lds_ptr_t)rowacc;
 
     // The workgroup's unit-quads in walk order are u = step * n_chunks + col; this wave takes u = wave, wave +
-    // n_waves, ...  A cursor is the (step, col) of one of them and moves on by n_waves.
+    // n_waves, ...  A cursor is the (step, col) of one of them and moves on by n_waves.  su = 4 * step * n_chunks +
+    // col: the index of the lane's unit in the workgroup's table slice is su + quarter * n_chunks (out_f is a
+    // multiple of four here, so every row quad is whole), which leaves one addition per address to the lanes.
     const uint32_t n_total = n_steps * n_chunks;
     const uint32_t n_mine = wave < n_total ? (n_total - wave + n_waves - 1) / n_waves : 0u;
     const uint32_t dq = n_waves / n_chunks, dr = n_waves - dq * n_chunks;
     struct Cur {
-        uint32_t step, col;
+        uint32_t step, col, su;
     };
     auto advance = [&](Cur &c) {
         c.step += dq;
@@ -857,23 +860,27 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
             c.col -= n_chunks;
             ++c.step;
         }
+        c.su = 4 * c.step * n_chunks + c.col;
     };
-    Cur c_issue = {wave / n_chunks, wave % n_chunks};
+    Cur c_issue = {wave / n_chunks, wave % n_chunks, 0};
+    c_issue.su = 4 * c_issue.step * n_chunks + c_issue.col;
     Cur c_now = c_issue, c_next = c_issue;
     advance(c_next);
+    const uint32_t tq1_lane = tq1_addr + quarter * n_chunks * 4;    // LDS address of the lane's row's entries
+    const uint32_t b1_lane = (quarter * n_chunks * 16u + li) * 4u;  // bitmap 0: byte offset of the lane's word
+    const uint32_t l1_lane = li * 16u;
+    const uint32_t xs_lane = xs_addr + li * 16u;
 
     uint32_t st_issue = 0;  // ring stage the next copy goes to
     auto issue = [&]() {
-        const uint32_t lrn = __umul24(min(4 * c_issue.step + quarter, rows_here - 1), n_chunks);
-        const uint32_t q1u = lds_u32(tq1_addr + (lrn + c_issue.col) * 4);
-        const uint32_t unit = unit0 + lrn + c_issue.col;
+        const uint32_t q1u = lds_u32(tq1_lane + c_issue.su * 4);
         uint8_t *stage = ring + st_issue * kRStageBytes;
         asm volatile("" ::: "memory");
         if (li < 13)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(l1_rsrc, (lds_ptr_t)stage, 16,
-                                                     (int)(((q1u * 3u) >> 5) * 4u + li * 16u), 0, 0, 0);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(b1_rsrc, (lds_ptr_t)(stage + 1024), 4, (int)((unit * 16u + li) * 4u),
-                                                 0, 0, 0);
+                                                     (int)(((q1u * 3u) >> 5) * 4u + l1_lane), 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(b1_rsrc, (lds_ptr_t)(stage + 1024), 4, (int)b1_lane,
+                                                 (int)((unit0 + c_issue.su) * 64u), 0, 0);
         st_issue = st_issue + 1 == (uint32_t)kRStages ? 0u : st_issue + 1;
         advance(c_issue);
     };
@@ -895,16 +902,15 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         w2 = (w2 & ~fm.z) | (kZeroCodes2 & fm.z);
     };
 
-    // Code window of the unit-quad at cursor c, whose data is in ring stage `st`, spliced once.  A row quad that
-    // reaches past the workgroup's last row repeats that row: its sums go to row slots nobody reads.
+    // Code window of the unit-quad at cursor c, whose data is in ring stage `st`, spliced once.
     // A lane with elements above level 1 leaves a record: {their bitmap bits, the lane's rank offset inside the
-    // unit, the unit's index in the workgroup's table slice, row slot << 16 | column block << 4 | lane of the row}.
+    // unit, the LDS address of the unit's table entry, row slot << 16 | column block << 4 | lane of the row}.
     const uint32_t rec_lane = (quarter << 16) | li;
     auto open_window = [&](uint32_t st, const Cur &c, uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &zrem) {
-        const uint32_t lu = __umul24(min(4 * c.step + quarter, rows_here - 1), n_chunks) + c.col;
+        const uint32_t ta = tq1_lane + c.su * 4;
         const uint32_t stage = ring_addr + st * kRStageBytes;
         const uint32_t word = lds_u32(stage + 1024 + lane * 4);
-        const uint32_t q1u = lds_u32(tq1_addr + lu * 4);
+        const uint32_t q1u = lds_u32(ta);
         const uint32_t cnt = __popc(word);
         const uint32_t excl = row_scan(cnt) - cnt;
         const uint32_t off = __umul24(excl, 3u) + ((q1u * 3u) & 31u);
@@ -917,7 +923,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         const uint64_t any = __ballot(zeros != 0);
         if (zeros != 0)
             push_record(queue, qcount + lanes_below(any),
-                        make_uint4(zeros, excl, lu, rec_lane + ((c.step << 18) | (c.col << 4))));
+                        make_uint4(zeros, excl, ta, rec_lane + ((c.step << 18) | (c.col << 4))));
         qcount += (uint32_t)__popcll(any);
         zrem = zeros;
         splice_once(w0, w1, w2, zrem);
@@ -968,7 +974,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
             // this lane's 16 activation pairs of the column block
             uint32_t xr[16];
             {
-                const uint32_t xa = xs_addr + c_now.col * (kFastChunk * 2) + li * 16u;
+                const uint32_t xa = xs_lane + c_now.col * (kFastChunk * 2);
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     const u32x4 v = lds_u128(xa + (uint32_t)t * 256u);
@@ -1158,7 +1164,7 @@ int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x,
     if (((uintptr_t)x & 15u) != 0 || (m > 1 && (ldx & 7) != 0)) return IXH_EUNSUPPORTED;
     const uint32_t n_chunks = P.in_f / kFastChunk;
     static const int shared_x = getenv("IXH_GEMV_SHARED_X") ? atoi(getenv("IXH_GEMV_SHARED_X")) : 1;
-    if (m == 1 && shared_x && P.in_f <= 65536u) {
+    if (m == 1 && shared_x && P.in_f <= 65536u && P.out_f % 4u == 0) {
         const int rc = any ? launch_rowsx<true>(P, prefix, n_chunks, x, y, s) : launch_rowsx<false>(P, prefix, n_chunks, x, y, s);
         if (rc != IXH_EUNSUPPORTED) return rc;
     }
