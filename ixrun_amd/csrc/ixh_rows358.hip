@@ -30,6 +30,11 @@
 //
 // Reduction.  Lanes sum over the wave's C blocks, rows over their 16 lanes
 // (DPP), waves through LDS after one barrier, in wave order.
+//
+// Two kernels share this decode: k_gemv358_rows (a wave owns column blocks, x in
+// registers) and k_gemv358_rowsx further down (x in LDS once per workgroup, the
+// unit-quads dealt to 16 waves), which serves the shapes whose row count is a
+// multiple of four.
 #include <stdlib.h>
 
 #include "ixh_fast358.h"
@@ -163,7 +168,7 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
 // ANY: any scheme whose first level has 3 bits: the element is followed down the nested bitmaps (level i: rank among
 // the elements in no level below i), every rank counted from the unit's start, where the table holds it (read
 // from global memory; tq2 and the staged side streams are not used).
-// XSW: the activations are the workgroup's shared, swizzled copy of the whole x row (one activation row): 16-byte
+// XSW: the activations are the workgroup's shared, swizzled copy of the whole x rows (xs_row bytes apart): 16-byte
 // piece p of the 64 bytes that lane l of a 16-lane row owns in a column block sits at piece p * 16 + l of the block.
 template <int MT, bool STAGED, bool ANY = false, bool XSW = false>
 __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, uint32_t tq1_addr, uint32_t tq2_addr,
@@ -220,8 +225,8 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
         uint32_t xe[MT];  // the activations this element meets
 #pragma unroll
         for (int j = 0; j < MT; ++j)
-            xe[j] = XSW ? lds_u16(xs_addr + (k0 >> 9) * (kFastChunk * 2) + (((e >> 3) * 16u + ((k0 >> 5) & 15u)) * 16u) +
-                                  (e & 7u) * 2u)
+            xe[j] = XSW ? lds_u16(xs_addr + (uint32_t)j * xs_row + (k0 >> 9) * (kFastChunk * 2) +
+                                  (((e >> 3) * 16u + ((k0 >> 5) & 15u)) * 16u) + (e & 7u) * 2u)
                         : lds_u16(xs_addr + ((uint32_t)j * xs_row + k0 - k_first + e) * 2u);
         if (ANY) {
             const float w = dequant(value_any(unit, r0_lane + nth), scale);
@@ -470,7 +475,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
 
     // ---- producer: LDS-DMA of unit-quad i into ring stage i % kRStages ----
     uint32_t i_step = 0, i_cc = 0;                            // (step, block) of the next unit to issue
-    uint32_t i_lrn = min(quarter, rows_here - 1) * n_chunks;  // its local row * n_chunks, per lane
+    uint32_t i_lrn = __umul24(min(quarter, rows_here - 1), n_chunks);  // its local row * n_chunks, per lane
     auto issue = [&](uint32_t i) {
         const uint32_t col = min(col0 + i_cc, n_chunks - 1);
         const uint32_t q1u = lds_u32(tq1_addr + (i_lrn + col) * 4);
@@ -485,7 +490,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
         if (++i_cc == C) {
             i_cc = 0;
             ++i_step;
-            i_lrn = min(4 * i_step + quarter, rows_here - 1) * n_chunks;
+            i_lrn = __umul24(min(4 * i_step + quarter, rows_here - 1), n_chunks);
         }
     };
 
@@ -517,7 +522,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
         const uint32_t q1u = lds_u32(tq1_addr + (lrn + col) * 4);
         const uint32_t c = __popc(word);
         const uint32_t excl = row_scan(c) - c;
-        const uint32_t off = excl * 3u + ((q1u * 3u) & 31u);  // bit offset inside the staged stream piece
+        const uint32_t off = __umul24(excl, 3u) + ((q1u * 3u) & 31u);  // bit offset inside the staged stream piece
         const uint32_t wa = stage + quarter * 256 + (off >> 5) * 4;
         const uint32_t d0 = lds_u32(wa), d1 = lds_u32(wa + 4), d2 = lds_u32(wa + 8), d3 = lds_u32(wa + 12);
         w0 = __builtin_amdgcn_alignbit(d1, d0, off);
@@ -584,7 +589,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
             }
         }
 
-    uint32_t lrn_step = min(quarter, rows_here - 1) * n_chunks;  // local row * n_chunks of the current step
+    uint32_t lrn_step = __umul24(min(quarter, rows_here - 1), n_chunks);  // local row * n_chunks of the current step
     bool valid_step = quarter < rows_here;
     uint32_t cw0, cw1, cw2, czrem;
     open_window(0, quarter, lrn_step, valid_step, 0, cw0, cw1, cw2, czrem);
@@ -602,7 +607,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
         for (int j = 0; j < MT; ++j)
 #pragma unroll
             for (int a = 0; a < NA; ++a) acc[j][a] = 0.0f;
-        const uint32_t lrn_next = min(4 * (step + 1) + quarter, rows_here - 1) * n_chunks;
+        const uint32_t lrn_next = __umul24(min(4 * (step + 1) + quarter, rows_here - 1), n_chunks);
         const bool valid_next = 4 * (step + 1) + quarter < rows_here;
 
 #pragma unroll
@@ -693,41 +698,44 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
 }
 
 // ---------------------------------------------------------------------------
-// One activation row, x shared by the workgroup
+// Up to four activation rows, x shared by the workgroup
 // ---------------------------------------------------------------------------
 // Same decode as k_gemv358_rows, different work split.  There a wave owns column blocks and keeps their activations
 // in registers, which ties the number of waves to the number of column blocks (12 waves, three per SIMD, for 34
-// blocks) and makes every wave walk 15 unit-quads one after the other.  Here the whole activation row sits in LDS
-// once per workgroup (swizzled, so that the 16 lanes of a row read consecutive 16-byte pieces), the workgroup's
-// unit-quads are dealt round-robin to as many waves as LDS allows (16: four per SIMD), and a wave reads the 64
-// activation bytes of a lane afresh for every unit-quad (four ds_read_b128).  The chain of dependent steps a wave
-// walks is a quarter shorter and a SIMD has one more wave to issue from.
+// blocks; 10 waves for 10 blocks) and makes every wave walk all row quads of its blocks one after the other.  Here
+// the activation rows sit in LDS once per workgroup (swizzled, so that the 16 lanes of a row read consecutive
+// 16-byte pieces), the workgroup's unit-quads are dealt round-robin to as many waves as LDS allows (16: four per
+// SIMD), and a wave reads the 64 activation bytes of a lane afresh for every unit-quad (four ds_read_b128 per
+// activation row).  Neighbouring waves work on neighbouring column blocks of the same row quad, so what a
+// workgroup has in flight is contiguous in every row.  Every row quad is whole (out_f % 4 == 0; other shapes stay
+// with k_gemv358_rows), which leaves the lanes one addition per table or bitmap address: a lane constant plus the
+// scalar index of the unit-quad.
 constexpr int kXMaxWaves = 16;
 
-__host__ __device__ constexpr uint32_t wave_lds_bytes_x() {
-    return kRStages * kRStageBytes + kRQueue * 16 + kRSlots * 4 + kRTasks * 2;
+__host__ __device__ constexpr uint32_t wave_lds_bytes_x(int mt) {
+    return kRStages * kRStageBytes + kRQueue * 16 + kRSlots * mt * 4 + kRTasks * 2;
 }
 
 struct RowsXLds {
     uint32_t tq1, tq2, side, xs, waves, total;
 };
 
-__host__ __device__ inline RowsXLds rowsx_layout(uint32_t rows_cap, uint32_t n_chunks, uint32_t n_waves) {
+__host__ __device__ inline RowsXLds rowsx_layout(uint32_t rows_cap, uint32_t n_chunks, uint32_t n_waves, int mt) {
     RowsXLds L;
     const uint32_t tbl = ((rows_cap * n_chunks + 1u + 3u) & ~3u) * 4u;
     L.tq1 = kRLutBytes + kRSpliceBytes;
     L.tq2 = L.tq1 + tbl;
     L.side = L.tq2 + tbl;
     L.xs = L.side + kRSideBytes;
-    L.waves = L.xs + n_chunks * kFastChunk * 2;
-    L.total = L.waves + n_waves * wave_lds_bytes_x();
+    L.waves = L.xs + (uint32_t)mt * n_chunks * kFastChunk * 2;
+    L.total = L.waves + n_waves * wave_lds_bytes_x(mt);
     return L;
 }
 
-template <bool ANY>
+template <int MT, bool ANY>
 __global__ void __launch_bounds__(kXMaxWaves * kWave)
 k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t quads_per_wg, uint32_t flags,
-                const uint16_t *__restrict__ x, uint16_t *__restrict__ y) {
+                const uint16_t *__restrict__ x, int m, int64_t ldx, uint16_t *__restrict__ y, int64_t ldy) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
@@ -740,32 +748,35 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     const uint32_t n_steps = min(quads_per_wg, n_quads - quad0);
     const uint32_t row0 = quad0 * 4;
     const uint32_t rows_here = min(n_steps * 4, P.out_f - row0);
-    const RowsXLds L = rowsx_layout(min(quads_per_wg * 4, P.out_f), n_chunks, n_waves);
+    const RowsXLds L = rowsx_layout(min(quads_per_wg * 4, P.out_f), n_chunks, n_waves, MT);
 
     // the pair table is addressed with (index bits | lane bits): it must sit at LDS address 0
     if ((uint32_t)(uintptr_t)(lds_ptr_t)smem != 0) {
-        for (uint32_t t = tid; t < rows_here; t += blockDim.x) y[row0 + t] = 0x7FC0;  // NaN
+        for (uint32_t t = tid; t < rows_here * MT; t += blockDim.x)
+            if ((int)(t % MT) < m) y[(int64_t)(t % MT) * ldy + row0 + t / MT] = 0x7FC0;  // NaN
         return;
     }
     uint32_t *const lut = reinterpret_cast<uint32_t *>(smem);            // [64][32]
     uint4 *const splice = reinterpret_cast<uint4 *>(smem + kRLutBytes);  // [33][2]
     uint32_t *const tq1 = reinterpret_cast<uint32_t *>(smem + L.tq1);
     uint32_t *const tq2 = reinterpret_cast<uint32_t *>(smem + L.tq2);
-    uint8_t *const wave_base = smem + L.waves + wave * wave_lds_bytes_x();
+    uint8_t *const wave_base = smem + L.waves + wave * wave_lds_bytes_x(MT);
     uint8_t *const ring = wave_base;
     uint4 *const queue = reinterpret_cast<uint4 *>(wave_base + kRStages * kRStageBytes);
     float *const rowacc = reinterpret_cast<float *>(wave_base + kRStages * kRStageBytes + kRQueue * 16);
-    uint16_t *const tasks = reinterpret_cast<uint16_t *>(rowacc + kRSlots);
+    uint16_t *const tasks = reinterpret_cast<uint16_t *>(rowacc + kRSlots * MT);
 
     // ---- the activation row: needs nothing but the arguments, so it is requested first.  Lane (t, l) of the copy
     // fetches piece l * 4 + t of the block and the hardware puts it at piece t * 16 + l.
     {
-        const __amdgpu_buffer_rsrc_t x_rsrc =
-            __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, (int)(P.in_f * 2u), 0x00020000);
-        for (uint32_t col = wave; col < n_chunks; col += n_waves)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (lds_ptr_t)(smem + L.xs + col * (kFastChunk * 2)), 16,
-                                                     (int)(col * (kFastChunk * 2) + (li * 4u + quarter) * 16u), 0, 0,
-                                                     0);
+        const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)x, 0, (int)((((int64_t)(m - 1) * ldx + P.in_f) * 2)), 0x00020000);
+        for (uint32_t t = wave; t < (uint32_t)m * n_chunks; t += n_waves) {
+            const uint32_t j = t / n_chunks, col = t - j * n_chunks;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                x_rsrc, (lds_ptr_t)(smem + L.xs + (j * n_chunks + col) * (kFastChunk * 2)), 16,
+                (int)(((int64_t)j * ldx + col * kFastChunk) * 2 + (li * 4u + quarter) * 16u), 0, 0, 0);
+        }
     }
 
     // ---- workgroup set-up: table slices, pair table, splice masks ----
@@ -794,7 +805,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         splice[2 * tid] = make_uint4(lm[0], lm[1], lm[2], 0u);
         splice[2 * tid + 1] = make_uint4(f[0], f[1], f[2], 0u);
     }
-    for (uint32_t j = lane; j < kRSlots; j += kWave) rowacc[j] = 0.0f;
+    for (uint32_t j = lane; j < kRSlots * MT; j += kWave) rowacc[j] = 0.0f;
     wait_vmem<0>();  // this wave's pieces of x are in LDS
     __syncthreads();
 
@@ -840,7 +851,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     const uint32_t splice_addr = kRLutBytes;
     const uint32_t tq1_addr = L.tq1, tq2_addr = L.tq2;
     const uint32_t ring_addr = (uint32_t)(uintptr_t)(lds_ptr_t)ring;
-    const uint32_t xs_addr = L.xs;
+    const uint32_t xs_addr = L.xs, xs_row = n_chunks * (kFastChunk * 2);  // bytes between activation rows
     const uint32_t rowacc_addr = (uint32_t)(uintptr_t)(lds_ptr_t)rowacc;
 
     // The workgroup's unit-quads in walk order are u = step * n_chunks + col; this wave takes u = wave, wave +
@@ -931,14 +942,14 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
     auto resolve = [&]() {
         if (ANY)
-            resolve_rows<1, false, true, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
-                                               xs_addr, 0, 0, 1, scale, lane, prefix, entries);
+            resolve_rows<MT, false, true, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
+                                               xs_addr, xs_row, 0, m, scale, lane, prefix, entries);
         else if (sv.staged)
-            resolve_rows<1, true, false, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
-                                               xs_addr, 0, 0, 1, scale, lane);
+            resolve_rows<MT, true, false, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
+                                               xs_addr, xs_row, 0, m, scale, lane);
         else
-            resolve_rows<1, false, false, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
-                                                xs_addr, 0, 0, 1, scale, lane);
+            resolve_rows<MT, false, false, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
+                                                xs_addr, xs_row, 0, m, scale, lane);
         qcount = 0;
     };
 
@@ -952,7 +963,12 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         open_window(0, c_now, cw0, cw1, cw2, czrem);
         while (__ballot(czrem != 0) != 0) splice_once(cw0, cw1, cw2, czrem);
         uint32_t st_now = 0;  // ring stage of the unit-quad whose window is open
-        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        constexpr int NA = MT == 1 ? 4 : (MT == 2 ? 2 : 1);  // independent accumulators per activation row
+        float acc[MT][NA];
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+#pragma unroll
+            for (int a = 0; a < NA; ++a) acc[j][a] = 0.0f;
 
         for (uint32_t i = 0; i < n_mine; ++i) {
             // the waves that share a SIMD take turns at the issue priority (see k_gemv358_rows)
@@ -971,14 +987,15 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
                 wait_vmem<0>();
             }
 
-            // this lane's 16 activation pairs of the column block
-            uint32_t xr[16];
-            {
-                const uint32_t xa = xs_lane + c_now.col * (kFastChunk * 2);
+            // this lane's 16 activation pairs of the column block, per activation row
+            uint32_t xr[MT][16];
+#pragma unroll
+            for (int j = 0; j < MT; ++j) {
+                const uint32_t xa = xs_lane + (uint32_t)j * xs_row + c_now.col * (kFastChunk * 2);
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     const u32x4 v = lds_u128(xa + (uint32_t)t * 256u);
-                    xr[4 * t] = v.x; xr[4 * t + 1] = v.y; xr[4 * t + 2] = v.z; xr[4 * t + 3] = v.w;
+                    xr[j][4 * t] = v.x; xr[j][4 * t + 1] = v.y; xr[j][4 * t + 2] = v.z; xr[j][4 * t + 3] = v.w;
                 }
             }
 
@@ -992,8 +1009,10 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
                 else if (ob >= 7) a = lo >> (ob - 7);
                 else a = lo << (7 - ob);
                 const uint32_t wp = lds_u32((a & 0x1F80u) | lut_lane);
-                acc[t % 4] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, wp),
-                                                             __builtin_bit_cast(bf16x2, xr[t]), acc[t % 4], false);
+#pragma unroll
+                for (int j = 0; j < MT; ++j)
+                    acc[j][t % NA] = __builtin_amdgcn_fdot2_f32_bf16(
+                        __builtin_bit_cast(bf16x2, wp), __builtin_bit_cast(bf16x2, xr[j][t]), acc[j][t % NA], false);
             }
 
             // window of this wave's next unit-quad
@@ -1007,9 +1026,16 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
             // the lane's sum stays in its register while the wave's next unit-quad is in the same row quad
             if (!more || c_next.step != c_now.step) {
-                const float total = row_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
-                if (li == 15) rowacc[4 * c_now.step + quarter] += total;
-                acc[0] = acc[1] = acc[2] = acc[3] = 0.0f;
+#pragma unroll
+                for (int j = 0; j < MT; ++j) {
+                    float sum = acc[j][0];
+#pragma unroll
+                    for (int a = 1; a < NA; ++a) sum += acc[j][a];
+                    const float total = row_sum(sum);
+                    if (li == 15) rowacc[(4 * c_now.step + quarter) * MT + j] += total;
+#pragma unroll
+                    for (int a = 0; a < NA; ++a) acc[j][a] = 0.0f;
+                }
             }
 
             st_now = st_next;
@@ -1023,11 +1049,13 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
     // ---- add the waves' row sums in wave order, write bf16 ----
     const uint32_t first_acc = L.waves + kRStages * kRStageBytes + kRQueue * 16;
-    for (uint32_t t = tid; t < rows_here; t += blockDim.x) {
+    for (uint32_t t = tid; t < rows_here * MT; t += blockDim.x) {
+        const uint32_t slot = t / MT, j = t - slot * MT;
+        if ((int)j >= m) continue;
         float sum = 0.0f;
         for (uint32_t w = 0; w < n_waves; ++w)
-            sum += *reinterpret_cast<const float *>(smem + first_acc + w * wave_lds_bytes_x() + t * 4);
-        y[row0 + t] = (uint16_t)f32_to_bf16_bits(sum);
+            sum += *reinterpret_cast<const float *>(smem + first_acc + w * wave_lds_bytes_x(MT) + t * 4);
+        y[(int64_t)j * ldy + row0 + slot] = (uint16_t)f32_to_bf16_bits(sum);
     }
 }
 
@@ -1104,18 +1132,18 @@ static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, c
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }
 
-// The shared-x kernel for one activation row: as many waves as LDS allows (16, 12 or 8); IXH_EUNSUPPORTED when the
-// activation row does not fit beside them.
-template <bool ANY>
-static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, const uint16_t *x, uint16_t *y,
-                        hipStream_t s) {
+// The shared-x kernel: as many waves as LDS allows (16, 12 or 8); IXH_EUNSUPPORTED when the activation rows do not
+// fit beside them.
+template <int MT, bool ANY>
+static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, const uint16_t *x, int m, int64_t ldx,
+                        uint16_t *y, int64_t ldy, hipStream_t s) {
     const uint32_t n_quads = (P.out_f + 3) / 4;
     static const int n_cu = [] {
         int dev = 0, v = 256;
         if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
         return v;
     }();
-    static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_rowsx<ANY>),
+    static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_rowsx<MT, ANY>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize,
                                                    (int)kLdsLimit) == hipSuccess;  // per instantiation
     if (!raised) return IXH_EUNSUPPORTED;
@@ -1124,10 +1152,10 @@ static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
     if (k_chunks != n_chunks || k_out != P.out_f) {
         uint32_t waves = 0, quads = 0;
         for (uint32_t w : {16u, 12u, 8u}) {
-            const size_t probe = rowsx_layout(min(16u, P.out_f), n_chunks, w).total;
+            const size_t probe = rowsx_layout(min(16u, P.out_f), n_chunks, w, MT).total;
             int per_cu = 0;
             if (probe > kLdsLimit ||
-                hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rowsx<ANY>, (int)(w * kWave), probe) !=
+                hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rowsx<MT, ANY>, (int)(w * kWave), probe) !=
                     hipSuccess || per_cu < 1)
                 continue;
             // whole rounds of resident workgroups, each with a contiguous run of at most 16 row quads
@@ -1135,7 +1163,7 @@ static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
             const uint32_t rounds = (n_quads + resident * (kRSlots / 4) - 1) / (resident * (kRSlots / 4));
             uint32_t q = (n_quads + rounds * resident - 1) / (rounds * resident);
             q = max(1u, min(q, kRSlots / 4));
-            if (rowsx_layout(min(q * 4, P.out_f), n_chunks, w).total > kLdsLimit) continue;
+            if (rowsx_layout(min(q * 4, P.out_f), n_chunks, w, MT).total > kLdsLimit) continue;
             waves = w;
             quads = q;
             break;
@@ -1150,9 +1178,9 @@ static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
     const uint32_t groups = (n_quads + quads - 1) / quads;
     uint32_t flags = 0;
     if (((uintptr_t)P.last & 3u) == 0) flags |= kFlagStageSide;
-    const size_t lds = rowsx_layout(min(quads * 4, P.out_f), n_chunks, waves).total;
-    hipLaunchKernelGGL((k_gemv358_rowsx<ANY>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks, quads,
-                       flags, x, y);
+    const size_t lds = rowsx_layout(min(quads * 4, P.out_f), n_chunks, waves, MT).total;
+    hipLaunchKernelGGL((k_gemv358_rowsx<MT, ANY>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks, quads,
+                       flags, x, m, ldx, y, ldy);
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }
 
@@ -1163,9 +1191,14 @@ int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x,
     const bool any = !(P.n_levels == 3 && P.bits[1] == 5);  // not (3,5,8): the resolver that walks the nested bitmaps
     if (((uintptr_t)x & 15u) != 0 || (m > 1 && (ldx & 7) != 0)) return IXH_EUNSUPPORTED;
     const uint32_t n_chunks = P.in_f / kFastChunk;
-    static const int shared_x = getenv("IXH_GEMV_SHARED_X") ? atoi(getenv("IXH_GEMV_SHARED_X")) : 1;
-    if (m == 1 && shared_x && P.in_f <= 65536u && P.out_f % 4u == 0) {
-        const int rc = any ? launch_rowsx<true>(P, prefix, n_chunks, x, y, s) : launch_rowsx<false>(P, prefix, n_chunks, x, y, s);
+    static const int shared_x = getenv("IXH_GEMV_SHARED_X") ? atoi(getenv("IXH_GEMV_SHARED_X")) : 4;
+    // IXH_GEMV_SHARED_X (development): 0 = never the shared-x kernel, 1 = for one activation row only, 2 = up to
+    // two rows, 4 = up to four (default)
+    if (shared_x && P.in_f <= 65536u && P.out_f % 4u == 0 && (m == 1 || (m == 2 && shared_x >= 2) || (m <= 4 && shared_x >= 4))) {
+        int rc;
+        if (m == 1) rc = any ? launch_rowsx<1, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s) : launch_rowsx<1, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
+        else if (m == 2) rc = any ? launch_rowsx<2, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s) : launch_rowsx<2, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
+        else rc = any ? launch_rowsx<4, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s) : launch_rowsx<4, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
         if (rc != IXH_EUNSUPPORTED) return rc;
     }
     const uint32_t c = (n_chunks + kRMaxWaves - 1) / kRMaxWaves;  // blocks per wave: a workgroup has at most kRMaxWaves waves
