@@ -204,18 +204,21 @@ int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, cons
     // walks the nested bitmaps (the column-block kernel is (3,5,8) only, so 5..8 rows go on to the any-scheme kernel)
     const bool fast_any = !fast && !is_358(d) && d.n_levels >= 2 && d.bits[0] == 3 &&
                           !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED | IXH_GEMV_DENSE | IXH_GEMV_COLUMN_KERNEL)) &&
-                          fast358_supports(d, (uint32_t)chunk, m) && (mostly_l1 || (flags & IXH_GEMV_FORCE_358)) &&
-                          (m <= 4 || m > 8);
+                          fast358_supports(d, (uint32_t)chunk, m) && (mostly_l1 || (flags & IXH_GEMV_FORCE_358));
     if ((fast || fast_any) && !atomic && !(flags & IXH_GEMV_COLUMN_KERNEL)) {
-        if (m <= 4) {
+        if (m <= 8) {
+            // up to four rows: one of the row-block kernels; five to eight: the shared-x row-block kernel where the
+            // activation rows fit in LDS, else (IXH_EUNSUPPORTED) the column-block kernel below
             rc = launch_gemv_358_rows(d, prefix, x, m, ldx, y, ldy, (hipStream_t)stream);
-        } else if (m > 8) {
-            // 9..16 rows: the row-block kernel four rows at a time beats the column-block kernel's 16-row version
-            // (3 or 4 launches of 40 us against 175 us on 17408 x 5120); 5..8 rows stay with the column-block kernel
-            rc = IXH_OK;
-            for (int j = 0; j < m && rc == IXH_OK; j += 4)
-                rc = launch_gemv_358_rows(d, prefix, x + (int64_t)j * ldx, m - j < 4 ? m - j : 4, ldx,
-                                          y + (int64_t)j * ldy, ldy, (hipStream_t)stream);
+        } else {
+            // 9..16 rows: the row-block kernels eight or four rows at a time beat the column-block kernel's 16-row
+            // version (175 us on 17408 x 5120)
+            for (int group = 8; group >= 4 && rc == IXH_EUNSUPPORTED; group -= 4) {
+                rc = IXH_OK;
+                for (int j = 0; j < m && rc == IXH_OK; j += group)
+                    rc = launch_gemv_358_rows(d, prefix, x + (int64_t)j * ldx, m - j < group ? m - j : group, ldx,
+                                              y + (int64_t)j * ldy, ldy, (hipStream_t)stream);
+            }
         }
     }
     if (fast && rc == IXH_EUNSUPPORTED)

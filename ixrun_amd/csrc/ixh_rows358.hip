@@ -712,8 +712,9 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
 // scalar index of the unit-quad.
 constexpr int kXMaxWaves = 16;
 
-__host__ __device__ constexpr uint32_t wave_lds_bytes_x(int mt) {
-    return kRStages * kRStageBytes + kRQueue * 16 + kRSlots * mt * 4 + kRTasks * 2;
+// a wave's region: ring, record queue, row sums (one per row of the workgroup and activation row), task list
+__host__ __device__ constexpr uint32_t wave_lds_bytes_x(int mt, uint32_t rows_cap) {
+    return kRStages * kRStageBytes + kRQueue * 16 + ((rows_cap * (uint32_t)mt * 4 + 15u) & ~15u) + kRTasks * 2;
 }
 
 struct RowsXLds {
@@ -728,12 +729,14 @@ __host__ __device__ inline RowsXLds rowsx_layout(uint32_t rows_cap, uint32_t n_c
     L.side = L.tq2 + tbl;
     L.xs = L.side + kRSideBytes;
     L.waves = L.xs + (uint32_t)mt * n_chunks * kFastChunk * 2;
-    L.total = L.waves + n_waves * wave_lds_bytes_x(mt);
+    L.total = L.waves + n_waves * wave_lds_bytes_x(mt, rows_cap);
     return L;
 }
 
+// Five to eight activation rows (MT = 8) run with eight waves of up to 256 registers: the activations of a
+// unit-quad are 128 registers per lane.
 template <int MT, bool ANY>
-__global__ void __launch_bounds__(kXMaxWaves * kWave)
+__global__ void __launch_bounds__((MT > 4 ? kXMaxWaves / 2 : kXMaxWaves) * kWave)
 k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t quads_per_wg, uint32_t flags,
                 const uint16_t *__restrict__ x, int m, int64_t ldx, uint16_t *__restrict__ y, int64_t ldy) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -748,7 +751,8 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     const uint32_t n_steps = min(quads_per_wg, n_quads - quad0);
     const uint32_t row0 = quad0 * 4;
     const uint32_t rows_here = min(n_steps * 4, P.out_f - row0);
-    const RowsXLds L = rowsx_layout(min(quads_per_wg * 4, P.out_f), n_chunks, n_waves, MT);
+    const uint32_t rows_cap = min(quads_per_wg * 4, P.out_f);
+    const RowsXLds L = rowsx_layout(rows_cap, n_chunks, n_waves, MT);
 
     // the pair table is addressed with (index bits | lane bits): it must sit at LDS address 0
     if ((uint32_t)(uintptr_t)(lds_ptr_t)smem != 0) {
@@ -760,11 +764,11 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     uint4 *const splice = reinterpret_cast<uint4 *>(smem + kRLutBytes);  // [33][2]
     uint32_t *const tq1 = reinterpret_cast<uint32_t *>(smem + L.tq1);
     uint32_t *const tq2 = reinterpret_cast<uint32_t *>(smem + L.tq2);
-    uint8_t *const wave_base = smem + L.waves + wave * wave_lds_bytes_x(MT);
+    uint8_t *const wave_base = smem + L.waves + wave * wave_lds_bytes_x(MT, rows_cap);
     uint8_t *const ring = wave_base;
     uint4 *const queue = reinterpret_cast<uint4 *>(wave_base + kRStages * kRStageBytes);
     float *const rowacc = reinterpret_cast<float *>(wave_base + kRStages * kRStageBytes + kRQueue * 16);
-    uint16_t *const tasks = reinterpret_cast<uint16_t *>(rowacc + kRSlots * MT);
+    uint16_t *const tasks = reinterpret_cast<uint16_t *>(wave_base + wave_lds_bytes_x(MT, rows_cap) - kRTasks * 2);
 
     // ---- the activation row: needs nothing but the arguments, so it is requested first.  Lane (t, l) of the copy
     // fetches piece l * 4 + t of the block and the hardware puts it at piece t * 16 + l.
@@ -805,7 +809,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         splice[2 * tid] = make_uint4(lm[0], lm[1], lm[2], 0u);
         splice[2 * tid + 1] = make_uint4(f[0], f[1], f[2], 0u);
     }
-    for (uint32_t j = lane; j < kRSlots * MT; j += kWave) rowacc[j] = 0.0f;
+    for (uint32_t j = lane; j < rows_cap * MT; j += kWave) rowacc[j] = 0.0f;
     wait_vmem<0>();  // this wave's pieces of x are in LDS
     __syncthreads();
 
@@ -1054,7 +1058,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         if ((int)j >= m) continue;
         float sum = 0.0f;
         for (uint32_t w = 0; w < n_waves; ++w)
-            sum += *reinterpret_cast<const float *>(smem + first_acc + w * wave_lds_bytes_x(MT) + t * 4);
+            sum += *reinterpret_cast<const float *>(smem + first_acc + w * wave_lds_bytes_x(MT, rows_cap) + t * 4);
         y[(int64_t)j * ldy + row0 + slot] = (uint16_t)f32_to_bf16_bits(sum);
     }
 }
@@ -1152,6 +1156,7 @@ static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
     if (k_chunks != n_chunks || k_out != P.out_f) {
         uint32_t waves = 0, quads = 0;
         for (uint32_t w : {16u, 12u, 8u}) {
+            if (MT > 4 && w > (uint32_t)kXMaxWaves / 2) continue;
             const size_t probe = rowsx_layout(min(16u, P.out_f), n_chunks, w, MT).total;
             int per_cu = 0;
             if (probe > kLdsLimit ||
@@ -1191,18 +1196,20 @@ int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x,
     const bool any = !(P.n_levels == 3 && P.bits[1] == 5);  // not (3,5,8): the resolver that walks the nested bitmaps
     if (((uintptr_t)x & 15u) != 0 || (m > 1 && (ldx & 7) != 0)) return IXH_EUNSUPPORTED;
     const uint32_t n_chunks = P.in_f / kFastChunk;
-    static const int shared_x = getenv("IXH_GEMV_SHARED_X") ? atoi(getenv("IXH_GEMV_SHARED_X")) : 4;
+    static const int shared_x = getenv("IXH_GEMV_SHARED_X") ? atoi(getenv("IXH_GEMV_SHARED_X")) : 8;
     // IXH_GEMV_SHARED_X (development): 0 = never the shared-x kernel, 1 = for one activation row only, 2 = up to
-    // two rows, 4 = up to four (default)
-    if (shared_x && P.in_f <= 65536u && P.out_f % 4u == 0 && (m == 1 || (m == 2 && shared_x >= 2) || (m <= 4 && shared_x >= 4))) {
+    // two rows, 4 = up to four, 8 = up to eight (default)
+    if (shared_x && P.in_f <= 65536u && P.out_f % 4u == 0 && (m == 1 || (m == 2 && shared_x >= 2) || (m <= 4 && shared_x >= 4) || (m <= 8 && shared_x >= 8))) {
         int rc;
         if (m == 1) rc = any ? launch_rowsx<1, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s) : launch_rowsx<1, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
         else if (m == 2) rc = any ? launch_rowsx<2, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s) : launch_rowsx<2, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
-        else rc = any ? launch_rowsx<4, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s) : launch_rowsx<4, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
+        else if (m <= 4) rc = any ? launch_rowsx<4, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s) : launch_rowsx<4, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
+        else rc = any ? launch_rowsx<8, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s) : launch_rowsx<8, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
         if (rc != IXH_EUNSUPPORTED) return rc;
     }
     const uint32_t c = (n_chunks + kRMaxWaves - 1) / kRMaxWaves;  // blocks per wave: a workgroup has at most kRMaxWaves waves
-    const int mt = m == 1 ? 1 : (m == 2 ? 2 : (m <= 4 ? 4 : 0));
+    if (m > 4) return IXH_EUNSUPPORTED;  // five to eight rows: the shared-x kernel above or nothing
+    const int mt = m == 1 ? 1 : (m == 2 ? 2 : 4);
 #define IXH_ROWS(MTV, CV) \
     if (mt == MTV && c == CV)                                                                  \
         return any ? launch_rows<MTV, CV, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s)     \

@@ -297,7 +297,7 @@ def test_gemv_staged(oracle, dev, kind, shape, level_bits):
 def test_gemv_row_block_kernel_other_schemes(oracle, dev, kind, shape, level_bits):
     """The row-block kernel takes every scheme whose first level has 3 bits (its elements above level 1 are followed
     down the nested bitmaps): chosen by itself for tensors that are almost all level 1, forced here for every mix;
-    1..4 rows in one launch, 9..16 rows four at a time."""
+    1..4 rows in one launch, 9..16 rows eight (or four) at a time."""
     from ixrun_amd import _lib
 
     out_f, in_f = shape
