@@ -271,6 +271,25 @@ def test_gemv_wide_rows(oracle, dev, kind, shape):
             check_outputs(run_gemv(dp, 512, x, m, dev, flags=flags), y64, f"{kind} {shape} m={m} flags={flags}")
 
 
+@pytest.mark.parametrize("kind", ["student_t", "rare_other", "only_l1"])
+@pytest.mark.parametrize("shape", [(8, 25600), (12, 33792), (4, 57344), (40, 5120), (4, 512)])
+def test_gemv_shared_x_kernel_lds_limits(oracle, dev, kind, shape):
+    """The row-block kernel that keeps the activation rows in LDS, at the edges of what LDS holds: whole row quads
+    with 50, 66 and 112 column blocks (12 waves, 8 waves, and no fit at all: the next kernel takes over), eight
+    activation rows beside 10 and 50 column blocks (fit / no fit), waves without a unit-quad of their own."""
+    from ixrun_amd import _lib
+
+    out_f, in_f = shape
+    p = make_packed(kind, out_f, in_f)
+    dp = device_packed(p, dev)
+    w_bits = oracle.decode_packed_bf16(p)
+    for m in (1, 2, 3, 4, 6, 8, 16):
+        x = activations(m, in_f, seed=10 + m)
+        y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
+        for flags in (0, _lib.IXH_GEMV_FORCE_358):
+            check_outputs(run_gemv(dp, 512, x, m, dev, flags=flags), y64, f"{kind} {shape} m={m} flags={flags}")
+
+
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("shape", [(64, 512), (37, 1024), (130, 2048), (24, 8704), (5, 25600)])
 @pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8), (5, 8)])
