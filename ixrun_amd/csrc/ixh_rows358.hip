@@ -37,6 +37,8 @@
 // multiple of four.
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "ixh_fast358.h"
 
 namespace ixh {
@@ -1151,32 +1153,46 @@ static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
                                                    hipFuncAttributeMaxDynamicSharedMemorySize,
                                                    (int)kLdsLimit) == hipSuccess;  // per instantiation
     if (!raised) return IXH_EUNSUPPORTED;
-    // the last answer is kept: a model asks for the same few shapes over and over
-    static uint32_t k_chunks = 0, k_out = 0, k_waves = 0, k_quads = 0;
-    if (k_chunks != n_chunks || k_out != P.out_f) {
-        uint32_t waves = 0, quads = 0;
-        for (uint32_t w : {16u, 12u, 8u}) {
-            if (MT > 4 && w > (uint32_t)kXMaxWaves / 2) continue;
-            const size_t probe = rowsx_layout(min(16u, P.out_f), n_chunks, w, MT).total;
-            int per_cu = 0;
-            if (probe > kLdsLimit ||
-                hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rowsx<MT, ANY>, (int)(w * kWave), probe) !=
-                    hipSuccess || per_cu < 1)
-                continue;
-            // whole rounds of resident workgroups, each with a contiguous run of at most 16 row quads
-            const uint32_t resident = (uint32_t)n_cu * (uint32_t)per_cu;
-            const uint32_t rounds = (n_quads + resident * (kRSlots / 4) - 1) / (resident * (kRSlots / 4));
-            uint32_t q = (n_quads + rounds * resident - 1) / (rounds * resident);
-            q = max(1u, min(q, kRSlots / 4));
-            if (rowsx_layout(min(q * 4, P.out_f), n_chunks, w, MT).total > kLdsLimit) continue;
-            waves = w;
-            quads = q;
-            break;
+    // the answers for the last few shapes are kept (a model asks for the same handful over and over), under a
+    // lock: a torn entry would launch one shape with another one's LDS layout
+    struct Plan {
+        uint32_t chunks, out_f, waves, quads;
+    };
+    static Plan plans[8] = {};
+    static uint32_t next_plan = 0;
+    static std::mutex plans_lock;
+    uint32_t k_waves = 0, k_quads = 0;
+    {
+        std::lock_guard<std::mutex> guard(plans_lock);
+        const Plan *hit = nullptr;
+        for (const Plan &pl : plans)
+            if (pl.chunks == n_chunks && pl.out_f == P.out_f) hit = &pl;
+        if (!hit) {
+            uint32_t waves = 0, quads = 0;
+            for (uint32_t w : {16u, 12u, 8u}) {
+                if (MT > 4 && w > (uint32_t)kXMaxWaves / 2) continue;
+                const size_t probe = rowsx_layout(min(16u, P.out_f), n_chunks, w, MT).total;
+                int per_cu = 0;
+                if (probe > kLdsLimit ||
+                    hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rowsx<MT, ANY>, (int)(w * kWave),
+                                                                 probe) != hipSuccess || per_cu < 1)
+                    continue;
+                // whole rounds of resident workgroups, each with a contiguous run of at most 16 row quads
+                const uint32_t resident = (uint32_t)n_cu * (uint32_t)per_cu;
+                const uint32_t rounds = (n_quads + resident * (kRSlots / 4) - 1) / (resident * (kRSlots / 4));
+                uint32_t q = (n_quads + rounds * resident - 1) / (rounds * resident);
+                q = max(1u, min(q, kRSlots / 4));
+                if (rowsx_layout(min(q * 4, P.out_f), n_chunks, w, MT).total > kLdsLimit) continue;
+                waves = w;
+                quads = q;
+                break;
+            }
+            Plan &slot = plans[next_plan++ % 8u];
+            slot = Plan{n_chunks, P.out_f, waves, quads};
+            hit = &slot;
         }
-        k_chunks = n_chunks;
-        k_out = P.out_f;
-        k_waves = waves;
-        k_quads = quads;
+        k_waves = hit->waves;
+        k_quads = hit->quads;
     }
     if (k_waves == 0) return IXH_EUNSUPPORTED;
     const uint32_t waves = k_waves, quads = k_quads;
