@@ -713,10 +713,14 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
 // with k_gemv358_rows), which leaves the lanes one addition per table or bitmap address: a lane constant plus the
 // scalar index of the unit-quad.
 constexpr int kXMaxWaves = 16;
+// Unit-quads in flight per wave, the one being read included.  Two: measured against three and four (with 16 waves
+// per CU), every stage more costs 2-3 %; fewer copies in flight leave more of a CU's cache lines to be found again
+// by the wave that works on the neighbouring column block.
+constexpr int kXStages = 2;
 
 // a wave's region: ring, record queue, row sums (one per row of the workgroup and activation row), task list
 __host__ __device__ constexpr uint32_t wave_lds_bytes_x(int mt, uint32_t rows_cap) {
-    return kRStages * kRStageBytes + kRQueue * 16 + ((rows_cap * (uint32_t)mt * 4 + 15u) & ~15u) + kRTasks * 2;
+    return kXStages * kRStageBytes + kRQueue * 16 + ((rows_cap * (uint32_t)mt * 4 + 15u) & ~15u) + kRTasks * 2;
 }
 
 struct RowsXLds {
@@ -768,8 +772,8 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     uint32_t *const tq2 = reinterpret_cast<uint32_t *>(smem + L.tq2);
     uint8_t *const wave_base = smem + L.waves + wave * wave_lds_bytes_x(MT, rows_cap);
     uint8_t *const ring = wave_base;
-    uint4 *const queue = reinterpret_cast<uint4 *>(wave_base + kRStages * kRStageBytes);
-    float *const rowacc = reinterpret_cast<float *>(wave_base + kRStages * kRStageBytes + kRQueue * 16);
+    uint4 *const queue = reinterpret_cast<uint4 *>(wave_base + kXStages * kRStageBytes);
+    float *const rowacc = reinterpret_cast<float *>(wave_base + kXStages * kRStageBytes + kRQueue * 16);
     uint16_t *const tasks = reinterpret_cast<uint16_t *>(wave_base + wave_lds_bytes_x(MT, rows_cap) - kRTasks * 2);
 
     // ---- the activation row: needs nothing but the arguments, so it is requested first.  Lane (t, l) of the copy
@@ -898,7 +902,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
                                                      (int)(((q1u * 3u) >> 5) * 4u + l1_lane), 0, 0, 0);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(b1_rsrc, (lds_ptr_t)(stage + 1024), 4, (int)b1_lane,
                                                  (int)((unit0 + c_issue.su) * 64u), 0, 0);
-        st_issue = st_issue + 1 == (uint32_t)kRStages ? 0u : st_issue + 1;
+        st_issue = st_issue + 1 == (uint32_t)kXStages ? 0u : st_issue + 1;
         advance(c_issue);
     };
 
@@ -960,9 +964,9 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     };
 
     if (n_mine > 0) {
-        const uint32_t n_pre = min((uint32_t)kRStages, n_mine);
+        const uint32_t n_pre = min((uint32_t)kXStages, n_mine);
         for (uint32_t i = 0; i < n_pre; ++i) issue();
-        if (n_mine >= (uint32_t)kRStages) wait_vmem<2 * (kRStages - 1)>();
+        if (n_mine >= (uint32_t)kXStages) wait_vmem<2 * (kXStages - 1)>();
         else wait_vmem<0>();
 
         uint32_t cw0, cw1, cw2, czrem;
@@ -986,9 +990,9 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
             if (qcount > kRQueue - kWave) resolve();  // keep room for a full wave of records
             // refill the stage whose window was read last time (it is st_issue); make unit i+1 readable
-            if (i + kRStages < n_mine) {
+            if (i + kXStages < n_mine) {
                 issue();
-                wait_vmem<2 * (kRStages - 1)>();
+                wait_vmem<2 * (kXStages - 1)>();
             } else {
                 wait_vmem<0>();
             }
@@ -1022,7 +1026,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
             }
 
             // window of this wave's next unit-quad
-            const uint32_t st_next = st_now + 1 == (uint32_t)kRStages ? 0u : st_now + 1;
+            const uint32_t st_next = st_now + 1 == (uint32_t)kXStages ? 0u : st_now + 1;
             const bool more = i + 1 < n_mine;
             if (more) {
                 uint32_t nzrem;
@@ -1054,7 +1058,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     __syncthreads();
 
     // ---- add the waves' row sums in wave order, write bf16 ----
-    const uint32_t first_acc = L.waves + kRStages * kRStageBytes + kRQueue * 16;
+    const uint32_t first_acc = L.waves + kXStages * kRStageBytes + kRQueue * 16;
     for (uint32_t t = tid; t < rows_here * MT; t += blockDim.x) {
         const uint32_t slot = t / MT, j = t - slot * MT;
         if ((int)j >= m) continue;
