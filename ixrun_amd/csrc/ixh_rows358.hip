@@ -35,6 +35,7 @@
 // registers) and k_gemv358_rowsx further down (x in LDS once per workgroup, the
 // unit-quads dealt to 16 waves), which serves the shapes whose row count is a
 // multiple of four.
+#include <math.h>
 #include <stdlib.h>
 
 #include <mutex>
@@ -718,16 +719,18 @@ constexpr int kXMaxWaves = 16;
 // by the wave that works on the neighbouring column block.
 constexpr int kXStages = 2;
 
-// a wave's region: ring, record queue, row sums (one per row of the workgroup and activation row), task list
-__host__ __device__ constexpr uint32_t wave_lds_bytes_x(int mt, uint32_t rows_cap) {
-    return kXStages * kRStageBytes + kRQueue * 16 + ((rows_cap * (uint32_t)mt * 4 + 15u) & ~15u) + kRTasks * 2;
+// a wave's region: ring, record queue (qcap records: 128, or 256 where a wave expects to fill the short one and LDS
+// holds the long one, which is resolved less often and in fuller batches), row sums (one per row of the workgroup and activation row), task list
+__host__ __device__ constexpr uint32_t wave_lds_bytes_x(int mt, uint32_t rows_cap, uint32_t qcap) {
+    return kXStages * kRStageBytes + qcap * 16 + ((rows_cap * (uint32_t)mt * 4 + 15u) & ~15u) + kRTasks * 2;
 }
 
 struct RowsXLds {
     uint32_t tq1, tq2, side, xs, waves, total;
 };
 
-__host__ __device__ inline RowsXLds rowsx_layout(uint32_t rows_cap, uint32_t n_chunks, uint32_t n_waves, int mt) {
+__host__ __device__ inline RowsXLds rowsx_layout(uint32_t rows_cap, uint32_t n_chunks, uint32_t n_waves, int mt,
+                                                 uint32_t qcap) {
     RowsXLds L;
     const uint32_t tbl = ((rows_cap * n_chunks + 1u + 3u) & ~3u) * 4u;
     L.tq1 = kRLutBytes + kRSpliceBytes;
@@ -735,13 +738,13 @@ __host__ __device__ inline RowsXLds rowsx_layout(uint32_t rows_cap, uint32_t n_c
     L.side = L.tq2 + tbl;
     L.xs = L.side + kRSideBytes;
     L.waves = L.xs + (uint32_t)mt * n_chunks * kFastChunk * 2;
-    L.total = L.waves + n_waves * wave_lds_bytes_x(mt, rows_cap);
+    L.total = L.waves + n_waves * wave_lds_bytes_x(mt, rows_cap, qcap);
     return L;
 }
 
 // Five to eight activation rows (MT = 8) run with eight waves of up to 256 registers: the activations of a
 // unit-quad are 128 registers per lane.
-template <int MT, bool ANY>
+template <int MT, bool ANY, int QCAP>
 __global__ void __launch_bounds__((MT > 4 ? kXMaxWaves / 2 : kXMaxWaves) * kWave)
 k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t quads_per_wg, uint32_t flags,
                 const uint16_t *__restrict__ x, int m, int64_t ldx, uint16_t *__restrict__ y, int64_t ldy) {
@@ -757,8 +760,9 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     const uint32_t n_steps = min(quads_per_wg, n_quads - quad0);
     const uint32_t row0 = quad0 * 4;
     const uint32_t rows_here = min(n_steps * 4, P.out_f - row0);
+    constexpr uint32_t qcap = QCAP;  // records the wave's queue holds
     const uint32_t rows_cap = min(quads_per_wg * 4, P.out_f);
-    const RowsXLds L = rowsx_layout(rows_cap, n_chunks, n_waves, MT);
+    const RowsXLds L = rowsx_layout(rows_cap, n_chunks, n_waves, MT, qcap);
 
     // the pair table is addressed with (index bits | lane bits): it must sit at LDS address 0
     if ((uint32_t)(uintptr_t)(lds_ptr_t)smem != 0) {
@@ -770,11 +774,11 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     uint4 *const splice = reinterpret_cast<uint4 *>(smem + kRLutBytes);  // [33][2]
     uint32_t *const tq1 = reinterpret_cast<uint32_t *>(smem + L.tq1);
     uint32_t *const tq2 = reinterpret_cast<uint32_t *>(smem + L.tq2);
-    uint8_t *const wave_base = smem + L.waves + wave * wave_lds_bytes_x(MT, rows_cap);
+    uint8_t *const wave_base = smem + L.waves + wave * wave_lds_bytes_x(MT, rows_cap, qcap);
     uint8_t *const ring = wave_base;
     uint4 *const queue = reinterpret_cast<uint4 *>(wave_base + kXStages * kRStageBytes);
-    float *const rowacc = reinterpret_cast<float *>(wave_base + kXStages * kRStageBytes + kRQueue * 16);
-    uint16_t *const tasks = reinterpret_cast<uint16_t *>(wave_base + wave_lds_bytes_x(MT, rows_cap) - kRTasks * 2);
+    float *const rowacc = reinterpret_cast<float *>(wave_base + kXStages * kRStageBytes + qcap * 16);
+    uint16_t *const tasks = reinterpret_cast<uint16_t *>(wave_base + wave_lds_bytes_x(MT, rows_cap, qcap) - kRTasks * 2);
 
     // ---- the activation row: needs nothing but the arguments, so it is requested first.  Lane (t, l) of the copy
     // fetches piece l * 4 + t of the block and the hardware puts it at piece t * 16 + l.
@@ -988,7 +992,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
             else if (turn == 2) __builtin_amdgcn_s_setprio(2);
             else if (turn == 3) __builtin_amdgcn_s_setprio(3);
 
-            if (qcount > kRQueue - kWave) resolve();  // keep room for a full wave of records
+            if (qcount > qcap - kWave) resolve();  // keep room for a full wave of records
             // refill the stage whose window was read last time (it is st_issue); make unit i+1 readable
             if (i + kXStages < n_mine) {
                 issue();
@@ -1058,13 +1062,13 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     __syncthreads();
 
     // ---- add the waves' row sums in wave order, write bf16 ----
-    const uint32_t first_acc = L.waves + kXStages * kRStageBytes + kRQueue * 16;
+    const uint32_t first_acc = L.waves + kXStages * kRStageBytes + qcap * 16;
     for (uint32_t t = tid; t < rows_here * MT; t += blockDim.x) {
         const uint32_t slot = t / MT, j = t - slot * MT;
         if ((int)j >= m) continue;
         float sum = 0.0f;
         for (uint32_t w = 0; w < n_waves; ++w)
-            sum += *reinterpret_cast<const float *>(smem + first_acc + w * wave_lds_bytes_x(MT, rows_cap) + t * 4);
+            sum += *reinterpret_cast<const float *>(smem + first_acc + w * wave_lds_bytes_x(MT, rows_cap, qcap) + t * 4);
         y[(int64_t)j * ldy + row0 + slot] = (uint16_t)f32_to_bf16_bits(sum);
     }
 }
@@ -1153,32 +1157,34 @@ static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
         if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
         return v;
     }();
-    static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_rowsx<MT, ANY>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                   (int)kLdsLimit) == hipSuccess;  // per instantiation
+    static const bool raised =  // per instantiation
+        hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_rowsx<MT, ANY, 128>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit) == hipSuccess &&
+        hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_rowsx<MT, ANY, 256>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit) == hipSuccess;
     if (!raised) return IXH_EUNSUPPORTED;
     // the answers for the last few shapes are kept (a model asks for the same handful over and over), under a
     // lock: a torn entry would launch one shape with another one's LDS layout
     struct Plan {
-        uint32_t chunks, out_f, waves, quads;
+        uint32_t chunks, out_f, waves, quads, qcap;
     };
     static Plan plans[8] = {};
     static uint32_t next_plan = 0;
     static std::mutex plans_lock;
-    uint32_t k_waves = 0, k_quads = 0;
+    uint32_t k_waves = 0, k_quads = 0, k_qcap = 0;
     {
         std::lock_guard<std::mutex> guard(plans_lock);
         const Plan *hit = nullptr;
         for (const Plan &pl : plans)
             if (pl.chunks == n_chunks && pl.out_f == P.out_f) hit = &pl;
         if (!hit) {
-            uint32_t waves = 0, quads = 0;
+            uint32_t waves = 0, quads = 0, qcap = 0;
             for (uint32_t w : {16u, 12u, 8u}) {
                 if (MT > 4 && w > (uint32_t)kXMaxWaves / 2) continue;
-                const size_t probe = rowsx_layout(min(16u, P.out_f), n_chunks, w, MT).total;
+                const size_t probe = rowsx_layout(min(16u, P.out_f), n_chunks, w, MT, kRQueue).total;
                 int per_cu = 0;
                 if (probe > kLdsLimit ||
-                    hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rowsx<MT, ANY>, (int)(w * kWave),
+                    hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rowsx<MT, ANY, 128>, (int)(w * kWave),
                                                                  probe) != hipSuccess || per_cu < 1)
                     continue;
                 // whole rounds of resident workgroups, each with a contiguous run of at most 16 row quads
@@ -1186,26 +1192,39 @@ static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
                 const uint32_t rounds = (n_quads + resident * (kRSlots / 4) - 1) / (resident * (kRSlots / 4));
                 uint32_t q = (n_quads + rounds * resident - 1) / (rounds * resident);
                 q = max(1u, min(q, kRSlots / 4));
-                if (rowsx_layout(min(q * 4, P.out_f), n_chunks, w, MT).total > kLdsLimit) continue;
+                if (rowsx_layout(min(q * 4, P.out_f), n_chunks, w, MT, kRQueue).total > kLdsLimit) continue;
                 waves = w;
                 quads = q;
+                // A longer queue pays where a wave fills the short one before it is through (5120 x 5120 with 1.8 %
+                // of the elements above level 1: -3 %); where it never does, the larger LDS footprint costs 1 %.
+                // Records a wave expects: its unit-quads x 64 lanes x the chance of a bitmap word with a zero bit.
+                qcap = kRQueue;
+                const double l1_share = min(1.0, (double)P.st_words[0] * (32.0 / 3.0) / (double)P.n);
+                const double expected = (double)((q * n_chunks + w - 1) / w) * 64.0 * (1.0 - pow(l1_share, 32.0));
+                if (expected > 0.75 * kRQueue && rowsx_layout(min(q * 4, P.out_f), n_chunks, w, MT, 256).total <= kLdsLimit)
+                    qcap = 256;
                 break;
             }
             Plan &slot = plans[next_plan++ % 8u];
-            slot = Plan{n_chunks, P.out_f, waves, quads};
+            slot = Plan{n_chunks, P.out_f, waves, quads, qcap};
             hit = &slot;
         }
         k_waves = hit->waves;
         k_quads = hit->quads;
+        k_qcap = hit->qcap;
     }
     if (k_waves == 0) return IXH_EUNSUPPORTED;
     const uint32_t waves = k_waves, quads = k_quads;
     const uint32_t groups = (n_quads + quads - 1) / quads;
     uint32_t flags = 0;
     if (((uintptr_t)P.last & 3u) == 0) flags |= kFlagStageSide;
-    const size_t lds = rowsx_layout(min(quads * 4, P.out_f), n_chunks, waves, MT).total;
-    hipLaunchKernelGGL((k_gemv358_rowsx<MT, ANY>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks, quads,
-                       flags, x, m, ldx, y, ldy);
+    const size_t lds = rowsx_layout(min(quads * 4, P.out_f), n_chunks, waves, MT, k_qcap).total;
+    if (k_qcap == 256)
+        hipLaunchKernelGGL((k_gemv358_rowsx<MT, ANY, 256>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix,
+                           n_chunks, quads, flags, x, m, ldx, y, ldy);
+    else
+        hipLaunchKernelGGL((k_gemv358_rowsx<MT, ANY, 128>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix,
+                           n_chunks, quads, flags, x, m, ldx, y, ldy);
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }
 
