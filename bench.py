@@ -32,7 +32,7 @@ MFMA_BF16_PEAK = 2.5e15  # FLOP/s dense bf16, MI355X published
 # WRITE_SIZE, KiB per dispatch, scaled by what the same counters read for the 256 MiB copy of --calibrate-copy:
 # x 2.0 and x 1.0); the counter summaries are kept under profiles/.  Workloads without a counter run report null.
 MEASURED_TRAFFIC_BYTES = {
-    "down_proj_5120x17408_m1_student_t": 23020.0 * 2.0 * 1024 + 16.0 * 1024,
+    "down_proj_5120x17408_m1_student_t": 23023.0 * 2.0 * 1024 + 16.0 * 1024,
     "down_proj_5120x17408_m1_calibrated": 33662.0 * 2.0 * 1024 + 40.0 * 1024,
     "prefill_5120x5120_m512_five_level": 50297.9 * 2.0 * 1024 + 30720.0 * 1024,
     "attn_proj_5120x5120_m1_student_t": 7118.0 * 2.0 * 1024 + 16.0 * 1024,
