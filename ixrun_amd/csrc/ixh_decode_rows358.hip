@@ -30,7 +30,7 @@ namespace ixh {
 typedef uint32_t dr_u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void *dr_lds_ptr_t;
 
-constexpr int kDrStages = 3;              // unit-quads in flight per wave
+constexpr int kDrStages = 2;  // unit-quads in flight per wave, the one being read included (three: 1 % slower)
 constexpr uint32_t kDrStageBytes = 1280;  // 1024 stream + 256 bitmap
 constexpr uint32_t kDrQueue = 128;        // records per wave
 constexpr uint32_t kDrTasks = 192;        // elements of 64 records that are spread over the lanes
@@ -479,12 +479,16 @@ k_decode358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_quads, ui
             qmark = 0;
         }
         // Refill the stage whose window was read last time; make unit-quad i+1 readable.  Behind its two copies the
-        // wave has issued: four stores (quad i-2), two copies, four stores (quad i-1), two copies; the first two
-        // quads have fewer stores behind them.  (The count is exact because every quad is whole: all four stores of
-        // an iteration are always issued.)
+        // wave has issued, with a ring of two: four stores (quad i-1), two copies; with a ring of three: four
+        // stores (quad i-2), two copies, four stores (quad i-1), two copies; the first quads have fewer stores
+        // behind them.  (The count is exact because every quad is whole: all four stores of an iteration are always
+        // issued.)
         if (i + kDrStages < n_mine) {
             issue(i + kDrStages);
-            if (i == 0) dr_wait_vmem<4>();
+            if (kDrStages == 2) {  // behind the copies of quad i+1: four stores (quad i-1), two copies
+                if (i == 0) dr_wait_vmem<2>();
+                else dr_wait_vmem<6>();
+            } else if (i == 0) dr_wait_vmem<4>();
             else if (i == 1) dr_wait_vmem<8>();
             else dr_wait_vmem<12>();
         } else {
