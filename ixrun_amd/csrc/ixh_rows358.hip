@@ -977,6 +977,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         open_window(0, c_now, cw0, cw1, cw2, czrem);
         while (__ballot(czrem != 0) != 0) splice_once(cw0, cw1, cw2, czrem);
         uint32_t st_now = 0;  // ring stage of the unit-quad whose window is open
+        const bool long_run = n_total > 4 * n_waves;
         constexpr int NA = MT == 1 ? 4 : (MT == 2 ? 2 : 1);  // independent accumulators per activation row
         float acc[MT][NA];
 #pragma unroll
@@ -985,9 +986,14 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
             for (int a = 0; a < NA; ++a) acc[j][a] = 0.0f;
 
         for (uint32_t i = 0; i < n_mine; ++i) {
-            // the waves that share a SIMD take turns at the issue priority (see k_gemv358_rows)
+            // The waves that share a SIMD take turns at the issue priority (see k_gemv358_rows).  Measured: with more
+            // than four unit-quads per wave (and four waves per SIMD) a turn of two unit-quads beats a turn of one by
+            // 1-2 %, and turns of three or four; with fewer unit-quads, turns of one handed round in the other
+            // direction are 1-2 % better for (3,5,8) and as much worse for the resolver that walks nested bitmaps.
             __builtin_amdgcn_s_setprio(0);
-            const uint32_t turn = ((wave >> 2) + i) & 3u;
+            const uint32_t turn = (MT > 4 ? (wave >> 2) + i
+                                   : long_run ? (wave >> 2) + (i >> 1)
+                                              : (ANY ? (wave >> 2) + i : (wave >> 2) - i)) & 3u;
             if (turn == 1) __builtin_amdgcn_s_setprio(1);
             else if (turn == 2) __builtin_amdgcn_s_setprio(2);
             else if (turn == 3) __builtin_amdgcn_s_setprio(3);
