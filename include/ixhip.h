@@ -77,6 +77,18 @@ int ixh_version(void);
 const char *ixh_last_error(void);
 
 /*
+ * Testing and measurement hook; no counterpart in the reference.  Overrides, for the whole process, a choice the
+ * library otherwise makes from the tensor (the defaults are what every other caller gets):
+ *   "decode_kernel"  0 = by the tensor (default), 1 = the row-block decoder, 2 = the level-by-level decoder,
+ *                    3 = the staged decoder, 4 = the wave-per-unit decoder; a named decoder that cannot take a
+ *                    call is skipped for that call
+ *   "gemv_shared_x"  most activation rows (0..8, default 8) that ixh_gemv gives to the row-block kernel that
+ *                    shares the activations through on-chip memory; 0 = never
+ * Returns IXH_EINVAL for an unknown name or a value out of range.  Calls already running are not affected.
+ */
+int ixh_set_option(const char *name, int64_t value);
+
+/*
  * Number of int32 entries per level of a prefix table with the given chunk:
  * ceil(n / chunk) + 1.
  */
@@ -137,7 +149,8 @@ int ixh_decode_gs(const IxhPacked *packed, const int32_t *prefix, int64_t chunk,
  * a row are combined in a fixed order through `workspace`
  * (ixh_gemv_workspace_bytes) and written to y, or, with IXH_GEMV_ATOMIC, added
  * into the caller-zeroed fp32 y32 [M, out_f] with atomics as the reference's
- * split kernel does (fused.py:294); y may then be NULL.
+ * split kernel does (fused.py:294); y may then be NULL.  Kernels that own whole
+ * rows add each output once (the same kernels as without the flag, up to 8 rows).
  */
 int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, const uint16_t *x,
              int32_t m, int64_t ldx, uint16_t *y, int64_t ldy, float *y32, void *workspace,

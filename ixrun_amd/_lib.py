@@ -57,7 +57,7 @@ _lib = None
 _ENV_GEMV_FLAGS = int(os.environ.get("IXH_GEMV_FLAGS", "0"))
 
 EXPORTS = (
-    "ixh_version", "ixh_last_error", "ixh_prefix_entries", "ixh_prefix_build", "ixh_decode",
+    "ixh_version", "ixh_last_error", "ixh_set_option", "ixh_prefix_entries", "ixh_prefix_build", "ixh_decode",
     "ixh_gemv", "ixh_gemv_workspace_bytes", "ixh_gemm", "ixh_gemm_workspace_bytes",
     "ixh_encode_workspace_bytes", "ixh_encode_scan", "ixh_encode_pack", "ixh_decode_gs",
 )
@@ -75,6 +75,8 @@ def lib() -> C.CDLL:
         L = C.CDLL(LIB_PATH)
         L.ixh_version.restype = C.c_int
         L.ixh_last_error.restype = C.c_char_p
+        L.ixh_set_option.restype = C.c_int
+        L.ixh_set_option.argtypes = [C.c_char_p, C.c_int64]
         L.ixh_prefix_entries.restype = C.c_int64
         L.ixh_prefix_entries.argtypes = [C.c_int64, C.c_int64]
         L.ixh_prefix_build.restype = C.c_int
@@ -114,6 +116,17 @@ def lib() -> C.CDLL:
 def check(code: int) -> None:
     if code != 0:
         raise IxhError(code, lib().ixh_last_error().decode())
+
+
+DECODE_KERNELS = {"auto": 0, "rows": 1, "dense": 2, "staged": 3, "generic": 4}
+
+
+def set_option(name: str, value) -> None:
+    """Process-wide testing / measurement switch of the library (``ixh_set_option``); ``decode_kernel`` also takes
+    the decoder's name."""
+    if name == "decode_kernel" and isinstance(value, str):
+        value = DECODE_KERNELS[value]
+    check(lib().ixh_set_option(name.encode(), int(value)))
 
 
 def current_stream(device) -> C.c_void_p:

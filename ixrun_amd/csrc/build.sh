@@ -1,9 +1,13 @@
 #!/bin/sh
-# Builds libixhip.so for gfx950 next to the sources (hipcc cross-compiles, no GPU needed).
+# Builds libixhip.so for gfx950 next to the sources (hipcc cross-compiles, no GPU needed).  One object per
+# source file, compiled side by side (JOBS, default 8), then linked.
 set -e
 cd "$(dirname "$0")"
 HIPCC="${HIPCC:-/opt/rocm/bin/hipcc}"
-exec "$HIPCC" --offload-arch=gfx950 -O3 -std=c++17 -fPIC -shared \
-    -Xclang -target-feature -Xclang -packed-fp32-ops \
-    -Wall -Wno-unused-function -Wno-pass-failed \
-    ixh_api.hip ixh_generic.hip ixh_fast358.hip ixh_rows358.hip ixh_prefill.hip ixh_decode_staged.hip ixh_gemv_staged.hip ixh_encode.hip ixh_dense358.hip ixh_decode_rows358.hip -o libixhip.so "$@"
+SRCS="ixh_api.hip ixh_generic.hip ixh_fast358.hip ixh_rows358.hip ixh_prefill.hip ixh_decode_staged.hip ixh_gemv_staged.hip ixh_encode.hip ixh_dense358.hip ixh_decode_rows358.hip"
+FLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Xclang -target-feature -Xclang -packed-fp32-ops -Wall -Wno-unused-function -Wno-pass-failed $*"
+mkdir -p build
+OBJS=""
+for s in $SRCS; do OBJS="$OBJS build/${s%.hip}.o"; done
+printf '%s\n' $SRCS | xargs -P "${JOBS:-8}" -I{} sh -c "rm -f build/\$(basename {} .hip).o; $HIPCC $FLAGS -c {} -o build/\$(basename {} .hip).o 2>&1 | grep -v 'packed-fp32-ops' >&2; test -f build/\$(basename {} .hip).o"
+exec "$HIPCC" --offload-arch=gfx950 -shared -fPIC $OBJS -o libixhip.so

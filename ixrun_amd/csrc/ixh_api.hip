@@ -13,6 +13,9 @@ namespace ixh {
 
 static thread_local char g_error[512] = "";
 
+std::atomic<int> g_opt_decode_kernel{kDecodeAuto};
+std::atomic<int> g_opt_gemv_shared_x{8};
+
 void set_error(const char *fmt, ...) {
     va_list ap;
     va_start(ap, fmt);
@@ -84,6 +87,22 @@ int ixh_version(void) { return 100; }
 
 const char *ixh_last_error(void) { return g_error; }
 
+int ixh_set_option(const char *name, int64_t value) {
+    if (!name) { set_error("option name is NULL"); return IXH_EINVAL; }
+    if (strcmp(name, "decode_kernel") == 0) {
+        if (value < kDecodeAuto || value > kDecodeGeneric) { set_error("decode_kernel %lld not in 0..4", (long long)value); return IXH_EINVAL; }
+        g_opt_decode_kernel.store((int)value, std::memory_order_relaxed);
+        return IXH_OK;
+    }
+    if (strcmp(name, "gemv_shared_x") == 0) {
+        if (value < 0 || value > 8) { set_error("gemv_shared_x %lld not in 0..8", (long long)value); return IXH_EINVAL; }
+        g_opt_gemv_shared_x.store((int)value, std::memory_order_relaxed);
+        return IXH_OK;
+    }
+    set_error("unknown option '%s'", name);
+    return IXH_EINVAL;
+}
+
 int64_t ixh_prefix_entries(int64_t n, int64_t chunk) {
     if (n < 0 || chunk <= 0) return -1;
     return (n + chunk - 1) / chunk + 1;
@@ -109,20 +128,20 @@ static int decode_any(const IxhPacked *packed, const int32_t *prefix, int64_t ch
     if (d.n == 0) return IXH_OK;
     if (!prefix) { set_error("prefix is NULL"); return IXH_EINVAL; }
     if (!out_i8 && !out_bf16) { set_error("both outputs are NULL"); return IXH_EINVAL; }
-    // Which decoder: by the tensor, unless IXH_DECODE_KERNEL names one (rows | dense | staged | generic; read per call,
-    // so that tests and measurements can take each of them; a named kernel that does not support the call is skipped).
-    const char *want = getenv("IXH_DECODE_KERNEL");
-    auto allowed = [&](const char *name) { return !want || !*want || strcmp(want, name) == 0; };
-    const bool forced = want && *want;
+    // Which decoder: by the tensor, unless the option "decode_kernel" names one (so that tests and measurements can
+    // take each of them; a named kernel that does not support the call is skipped).
+    const int want = g_opt_decode_kernel.load(std::memory_order_relaxed);
+    auto allowed = [&](int which) { return want == kDecodeAuto || want == which; };
+    const bool forced = want != kDecodeAuto;
     // level 1 holds at least 97 % of the elements (from the size of its stream)
     const bool mostly_l1 = (uint64_t)d.st_words[0] * 32u / 3u >= (uint64_t)d.n / 100u * 97u;
-    if (allowed("rows") && (forced || mostly_l1) && !gs.fp16 && decode_rows358_supports(d, (uint32_t)chunk, out_i8, out_bf16))
+    if (allowed(kDecodeRows) && (forced || mostly_l1) && !gs.fp16 && decode_rows358_supports(d, (uint32_t)chunk, out_i8, out_bf16))
         // first level of 3 bits, almost all level 1, whole unit-quads: the row-block decoder (ixh_decode_rows358.hip)
         rc = launch_decode_rows358(d, prefix, out_bf16, (hipStream_t)stream);
-    else if (allowed("dense") && (forced || !mostly_l1) && decode_dense358_supports(d, (uint32_t)chunk, out_i8, out_bf16, gs))
+    else if (allowed(kDecodeDense) && (forced || !mostly_l1) && decode_dense358_supports(d, (uint32_t)chunk, out_i8, out_bf16, gs))
         // (3,5,8) with many elements above level 1: the level-by-level decoder (ixh_dense358.hip)
         rc = launch_decode_dense358(d, prefix, out_bf16, gs, (hipStream_t)stream);
-    else if ((allowed("staged") || allowed("rows") || allowed("dense")) &&
+    else if ((allowed(kDecodeStaged) || allowed(kDecodeRows) || allowed(kDecodeDense)) &&
              decode_staged_supports(d, (uint32_t)chunk, out_i8, out_bf16, gs))
         rc = launch_decode_staged(d, prefix, out_bf16, gs, (hipStream_t)stream);
     else
@@ -205,11 +224,13 @@ int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, cons
     const bool fast_any = !fast && !is_358(d) && d.n_levels >= 2 && d.bits[0] == 3 &&
                           !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED | IXH_GEMV_DENSE | IXH_GEMV_COLUMN_KERNEL)) &&
                           fast358_supports(d, (uint32_t)chunk, m) && (mostly_l1 || (flags & IXH_GEMV_FORCE_358));
-    if ((fast || fast_any) && !atomic && !(flags & IXH_GEMV_COLUMN_KERNEL)) {
+    if ((fast || fast_any) && !(flags & IXH_GEMV_COLUMN_KERNEL) && (!atomic || m <= 8)) {
         if (m <= 8) {
             // up to four rows: one of the row-block kernels; five to eight: the shared-x row-block kernel where the
-            // activation rows fit in LDS, else (IXH_EUNSUPPORTED) the column-block kernel below
-            rc = launch_gemv_358_rows(d, prefix, x, m, ldx, y, ldy, (hipStream_t)stream);
+            // activation rows fit in LDS, else (IXH_EUNSUPPORTED) the column-block kernel below.  A workgroup owns
+            // whole rows, so the split-K contract (add into the caller's fp32 vector) costs it one addition per output.
+            rc = launch_gemv_358_rows(d, prefix, x, m, ldx, atomic ? nullptr : y, ldy, atomic ? y32 : nullptr,
+                                      (hipStream_t)stream);
         } else {
             // 9..16 rows: the row-block kernels eight or four rows at a time beat the column-block kernel's 16-row
             // version (175 us on 17408 x 5120)
@@ -217,7 +238,7 @@ int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, cons
                 rc = IXH_OK;
                 for (int j = 0; j < m && rc == IXH_OK; j += group)
                     rc = launch_gemv_358_rows(d, prefix, x + (int64_t)j * ldx, m - j < group ? m - j : group, ldx,
-                                              y + (int64_t)j * ldy, ldy, (hipStream_t)stream);
+                                              y + (int64_t)j * ldy, ldy, nullptr, (hipStream_t)stream);
             }
         }
     }

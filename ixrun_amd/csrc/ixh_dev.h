@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/ixhip.h"
 
 namespace ixh {
@@ -135,5 +137,10 @@ int launch_encode_scan(const uint16_t *w, uint32_t n, int n_levels, const int *b
 int launch_encode_pack(const uint16_t *w, const Dev &P, const int32_t *table, hipStream_t s);
 int launch_fill_u16(uint16_t *dst, uint32_t n, uint16_t value, hipStream_t s);
 void set_error(const char *fmt, ...);
+
+// Process-wide switches of ixh_set_option (testing and measurement; the defaults are what a caller gets).
+enum DecodeKernel : int { kDecodeAuto = 0, kDecodeRows = 1, kDecodeDense = 2, kDecodeStaged = 3, kDecodeGeneric = 4 };
+extern std::atomic<int> g_opt_decode_kernel;   // a DecodeKernel
+extern std::atomic<int> g_opt_gemv_shared_x;   // most activation rows the shared-x row-block kernel serves (0..8)
 
 }  // namespace ixh

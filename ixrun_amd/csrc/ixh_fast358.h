@@ -11,9 +11,11 @@ bool fast358_supports(const Dev &P, uint32_t chunk, int m);
 // x / ld alignment is checked at launch; returns IXH_EUNSUPPORTED if it does not fit
 int launch_gemv_358(const Dev &P, const int32_t *prefix, uint32_t chunk, const uint16_t *x, int m, int64_t ldx,
                     uint16_t *y, int64_t ldy, float *y32, float *ws, bool atomic, hipStream_t s);
-// single-launch row-block kernel (ixh_rows358.hip); IXH_EUNSUPPORTED if the shape does not fit it
+// single-launch row-block kernel (ixh_rows358.hip); IXH_EUNSUPPORTED if the shape does not fit it.  y32 == nullptr:
+// bf16 results to y; otherwise the fp32 row sums are added into y32 [m, out_f] (one addition per output) and y is
+// not touched
 int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
-                         int64_t ldy, hipStream_t s);
+                         int64_t ldy, float *y32, hipStream_t s);
 // level-by-level kernel for one activation row and mixes with many elements above level 1 (ixh_dense358.hip)
 bool gemv_dense358_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x);
 int launch_gemv_dense358(const Dev &P, const int32_t *prefix, const uint16_t *x, uint16_t *y, float *y32, float *ws,

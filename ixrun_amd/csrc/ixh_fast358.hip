@@ -334,11 +334,6 @@ bool fast358_supports(const Dev &P, uint32_t chunk, int m) {
 }
 
 static uint32_t pick_rows_per_wave(const Dev &P, uint32_t n_chunks) {
-    static const int forced = [] {
-        const char *e = getenv("IXH_ROWS_PER_WAVE");
-        return e ? atoi(e) : 0;
-    }();
-    if (forced >= 4 && forced <= kFRowSlots) return (uint32_t)(forced & ~3);
     // aim for at least ~4 waves per SIMD of a 256-CU part
     uint32_t rows = kFRowSlots;
     while (rows > 8 && (uint64_t)n_chunks * ((P.out_f + rows - 1) / rows) < 4096) rows >>= 1;

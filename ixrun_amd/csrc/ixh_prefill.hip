@@ -93,17 +93,7 @@ __device__ __forceinline__ void mfma_column(__amdgpu_buffer_rsrc_t x_rs, uint32_
 template <int L>
 __global__ void __launch_bounds__(kWave *kPWaves, L <= 5 ? 4 : 2)  // four waves per SIMD (two workgroups per CU) where the registers allow
 k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const uint16_t *__restrict__ x, uint32_t m_rows,
-          int64_t ldx, float *__restrict__ ws, uint32_t n_slices
-#ifdef IXH_VARIANTS
-          , unsigned long long *trace
-#endif
-          ) {
-#ifdef IXH_VARIANTS  // timing experiments only
-#define PF_STAMP(k) do { if (trace && (threadIdx.x & 63) == 0) trace[(blockIdx.x * 8 + (threadIdx.x >> 6)) * 16 + (k)] = wall_clock64(); } while (0)
-#else
-#define PF_STAMP(k) do { } while (0)
-#endif
-    PF_STAMP(0);
+          int64_t ldx, float *__restrict__ ws, uint32_t n_slices) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *const wt = reinterpret_cast<uint16_t *>(smem);  // [64][520]
     constexpr int kDma = staged_dma_count(L);
@@ -153,7 +143,6 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
         put_unit<L>(slot + staged_slot_words(L) * 4, lane, S);
     };
     for (uint32_t t = 0; t < kPRing - 1 && t < total; ++t) stage_row(t, c_begin);
-    PF_STAMP(1);
 
     // output tile of this wave: m in [64 w, +64), the 32 n of the workgroup
     const uint32_t m_tiles = kPWaveM * wave < m_rows ? min(kPMTiles, (m_rows - kPWaveM * wave + 31) / 32) : 0u;
@@ -171,7 +160,6 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
     for (uint32_t c = c_begin; c < c_end; ++c) {
         const uint32_t q3 = table_at(c + 3);
         barrier_lds();  // the previous column's MFMAs are done with the weight tile
-        if (c == c_begin) PF_STAMP(2);
         // ---- decode the 64 x 512 weight tile of unit column c: wave w takes rows 8w .. 8w+7 ----
 #pragma unroll 1
         for (uint32_t j = 0; j < kPRowsPerWave; ++j) {
@@ -184,11 +172,7 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
             else if (after == 1) wait_vmcnt<kDma>();
             else wait_vmcnt<0>();
             uint16_t *wrow = wt + (wave * kPRowsPerWave + j) * kPWStride;
-#ifdef IXH_PF_NO_DECODE
-            if (false) {
-#else
             if (row_first + j < P.out_f) {
-#endif
                 const uint32_t slot = my_slots + (t % kPRing) * prefill_slot_bytes(L);
                 StagedUnit<L> S;
                 get_unit<L>(slot + staged_slot_words(L) * 4, S);
@@ -199,27 +183,19 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
 #pragma unroll 1
                 for (uint32_t g = 0; g < kStagedChunk / kWave; ++g) wrow[g * kWave + lane] = 0;
             }
-            if (c == c_begin) PF_STAMP(3 + j);
         }
         q0 = q1, q1 = q2, q2 = q3;
         barrier_lds();  // weight tile complete
-        if (c == c_begin) PF_STAMP(11);
 
         // ---- eight blocks of 64 k over the decoded tile ----
         const uint16_t *b_lane = wt + (lane & 31) * kPWStride + 32 * (lane >> 5);
         const uint32_t x_col = x_lane + c * (kStagedChunk * 2);
-#ifdef IXH_PF_NO_MFMA
-        switch (0u) {
-#else
         switch (m_tiles) {
-#endif
             case 2: mfma_column<2>(x_rs, x_col, x_tile, b_lane, acc); break;
             case 1: mfma_column<1>(x_rs, x_col, x_tile, b_lane, acc); break;
             default: break;
         }
-        if (c == c_begin) PF_STAMP(12);
     }
-    PF_STAMP(13);
 
     // ---- partial sums of this K slice: ws[slice][m][n] ----
     const uint32_t n = n0 + (lane & 31);
@@ -232,7 +208,6 @@ k_prefill(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const ui
                 if (m < m_rows) ws[((size_t)slice * m_rows + m) * P.out_f + n] = acc[t][r];
             }
     }
-    PF_STAMP(14);
 }
 
 // y[m][n] = bf16(sum over the K slices, in slice order)
@@ -284,13 +259,6 @@ bool prefill_supports(const Dev &P, const uint16_t *x, int64_t ldx) {
            (ldx & 7) == 0 && ldx < (1 << 20) && ((uintptr_t)P.last & 3u) == 0 && P.n_levels >= 2 && P.n_levels <= IXH_MAX_LEVELS;
 }
 
-#ifdef IXH_VARIANTS
-static unsigned long long *g_pf_trace = nullptr;
-extern "C" int ixh_debug_prefill_trace(unsigned long long *host_out, int n) {
-    if (!g_pf_trace) return -1;
-    return hipMemcpy(host_out, g_pf_trace, (size_t)n * 8, hipMemcpyDeviceToHost) == hipSuccess ? 0 : -2;
-}
-#endif
 
 template <int L>
 static int prefill_launch(const Dev &P, const int32_t *prefix, const uint16_t *x, uint32_t m_rows, int64_t ldx,
@@ -308,14 +276,8 @@ static int prefill_launch(const Dev &P, const int32_t *prefix, const uint16_t *x
     const uint32_t n_slices = pick_slices(tiles, n_chunks);
     for (uint32_t m0 = 0; m0 < m_rows; m0 += kPMaxM) {
         const uint32_t mb = min(kPMaxM, m_rows - m0);
-#ifdef IXH_VARIANTS
-        if (!g_pf_trace) (void)hipMalloc(&g_pf_trace, 2048 * 8 * 16 * 8);
-        hipLaunchKernelGGL(k_prefill<L>, dim3(tiles * n_slices), dim3(kWave * kPWaves), lds, s, P, prefix, n_chunks,
-                           x + (int64_t)m0 * ldx, mb, ldx, ws, n_slices, tiles * n_slices <= 2048 ? g_pf_trace : nullptr);
-#else
         hipLaunchKernelGGL(k_prefill<L>, dim3(tiles * n_slices), dim3(kWave * kPWaves), lds, s, P, prefix, n_chunks,
                            x + (int64_t)m0 * ldx, mb, ldx, ws, n_slices);
-#endif
         const size_t total = (size_t)mb * P.out_f;
         hipLaunchKernelGGL(k_prefill_reduce, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, ws, mb, P.out_f,
                            n_slices, y + (int64_t)m0 * ldy, ldy);

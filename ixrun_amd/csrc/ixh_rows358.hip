@@ -322,21 +322,9 @@ __device__ __forceinline__ void set_wave_priority(uint32_t p) {
 
 template <int MT, int C, bool ANY = false>
 __global__ void __launch_bounds__(kRMaxWaves * kWave)
-k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t quads_per_wg_arg, uint32_t flags,
-               const uint16_t *__restrict__ x, int m, int64_t ldx, uint16_t *__restrict__ y, int64_t ldy
-#ifdef IXH_VARIANTS
-               , unsigned long long *trace
-#endif
-               ) {
-#ifdef IXH_VARIANTS  // timing experiments only: stamps, and bits 16.. of the argument switch parts off
-#define IXH_STAMP(k) do { if (trace && threadIdx.x == 0) trace[blockIdx.x * 8 + (k)] = wall_clock64(); } while (0)
-    const uint32_t dbg = quads_per_wg_arg >> 16, quads_per_wg = quads_per_wg_arg & 0xFFFFu;
-#else
-#define IXH_STAMP(k) do { } while (0)
-    constexpr uint32_t dbg = 0;
-    const uint32_t quads_per_wg = quads_per_wg_arg;
-#endif
-    IXH_STAMP(0);
+k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t quads_per_wg, uint32_t flags,
+               const uint16_t *__restrict__ x, int m, int64_t ldx, uint16_t *__restrict__ y, int64_t ldy,
+               float *__restrict__ y32) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
@@ -356,7 +344,10 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     // ever not hold, say so in the output instead of computing garbage.
     if ((uint32_t)(uintptr_t)(lds_ptr_t)smem != 0) {
         for (uint32_t t = tid; t < rows_here * MT; t += blockDim.x)
-            if ((int)(t % MT) < m) y[(int64_t)(t % MT) * ldy + row0 + t / MT] = 0x7FC0;  // NaN
+            if ((int)(t % MT) < m) {
+                if (y32) y32[(size_t)(t % MT) * P.out_f + row0 + t / MT] = __uint_as_float(0x7FC00000u);  // NaN
+                else y[(int64_t)(t % MT) * ldy + row0 + t / MT] = 0x7FC0;
+            }
         return;
     }
     uint32_t *const lut = reinterpret_cast<uint32_t *>(smem);            // [64][32]
@@ -373,14 +364,12 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     // ---- workgroup set-up: table slices and x first (they wait on memory), then the tables built here ----
     const uint32_t unit0 = row0 * n_chunks;
     const uint32_t entries = P.out_f * n_chunks + 1;
-    if (!(dbg & 16))
-        for (uint32_t i = tid; i <= rows_here * n_chunks; i += blockDim.x) {
+    for (uint32_t i = tid; i <= rows_here * n_chunks; i += blockDim.x) {
             tq1[i] = (uint32_t)prefix[unit0 + i];
             if (!ANY) tq2[i] = (uint32_t)prefix[entries + unit0 + i];
         }
     const float scale = bf16_bits_to_f32(*P.scale);
-    if (!(dbg & 8))
-        for (uint32_t i = tid; i < 64 * 32; i += blockDim.x) {
+    for (uint32_t i = tid; i < 64 * 32; i += blockDim.x) {
             const int c0 = (i >> 5) & 7, c1 = i >> 8;
             const uint32_t w0 = c0 < 7 ? f32_to_bf16_bits((float)(c0 - 3) * scale) : 0u;
             const uint32_t w1 = c1 < 7 ? f32_to_bf16_bits((float)(c1 - 3) * scale) : 0u;
@@ -402,7 +391,6 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     }
     for (uint32_t j = lane; j < kRSlots * MT; j += kWave) rowacc[j] = 0.0f;
     __syncthreads();
-    IXH_STAMP(1);
 
     const uint32_t col0 = wave * C;
 
@@ -417,7 +405,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
             const uint32_t col = min(col0 + cc, n_chunks - 1);
 #pragma unroll
             for (int j = 0; j < MT; ++j)
-                if (j < m && !(dbg & 32))
+                if (j < m)
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(
                         x_rsrc, (lds_ptr_t)(xs + (j * C + cc) * (kFastChunk / 2)), 16,
                         (int)(((int64_t)j * ldx + col * kFastChunk) * 2 + lane * 16), 0, 0, 0);
@@ -552,8 +540,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     const uint32_t xs_addr = (uint32_t)(uintptr_t)(lds_ptr_t)xs;
     const uint32_t rowacc_addr = (uint32_t)(uintptr_t)(lds_ptr_t)rowacc;
     auto resolve = [&]() {
-        if (dbg & 128) {
-        } else if (ANY)
+        if (ANY)
             resolve_rows<MT, false, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks, xs_addr,
                                           C * kFastChunk, col0 * kFastChunk, m, scale, lane, prefix, entries);
         else if (sv.staged)
@@ -570,7 +557,6 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     for (uint32_t i = 0; i < n_pre; ++i) issue(i);
     if (n_units >= (uint32_t)kRStages) wait_vmem<2 * (kRStages - 1)>();
     else wait_vmem<0>();
-    IXH_STAMP(2);
 
     // this lane's activations: C blocks x MT rows x 16 packed bf16 pairs
     uint32_t xr[C][MT][16];
@@ -578,7 +564,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     for (int cc = 0; cc < C; ++cc)
 #pragma unroll
         for (int j = 0; j < MT; ++j) {
-            if (j < m && !(dbg & 32)) {
+            if (j < m) {
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     const u32x4 v = lds_u128((uint32_t)(uintptr_t)(lds_ptr_t)xs +
@@ -604,7 +590,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
         // The waves that share a SIMD take turns at the issue priority, one row quad each: without this the
         // oldest wave is served first throughout, finishes early and leaves the others to end the kernel with
         // nothing to hide their waits behind.
-        if (!(dbg & 512)) set_wave_priority(((wave >> 2) + step) % 3u);
+        set_wave_priority(((wave >> 2) + step) % 3u);
         float acc[MT][NA];
 #pragma unroll
         for (int j = 0; j < MT; ++j)
@@ -618,19 +604,16 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
             const uint32_t i = step * C + cc;
             if (qcount > kRQueue - kWave) resolve();  // keep room for a full wave of records
             // refill the stage whose window was read last time; make unit i+1 readable
-            if (!(dbg & 4)) {
-                if (i + kRStages < n_units) {
-                    issue(i + kRStages);
-                    wait_vmem<2 * (kRStages - 1)>();
-                } else {
-                    wait_vmem<0>();
-                }
+            if (i + kRStages < n_units) {
+                issue(i + kRStages);
+                wait_vmem<2 * (kRStages - 1)>();
+            } else {
+                wait_vmem<0>();
             }
 
             // The 16 code pairs of unit i go through the pair table and meet the x pairs.  Written first: the pair
             // table reads and the first reads of the next window then sit in one basic block (the record store
             // below ends it), so they are issued together and the dot products fill the wait for the window.
-            if (!(dbg & 1))
 #pragma unroll
             for (int t = 0; t < 16; ++t) {
                 const int bit = 6 * t, ob = bit & 31, d = bit >> 5;
@@ -648,8 +631,8 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
             }
 
             // window of unit i+1 (or, past the end, a void one)
-            uint32_t nw0 = cw0 + 1, nw1 = cw1 + 1, nw2 = cw2, nzrem = 0;
-            if (!(dbg & 2)) {
+            uint32_t nw0, nw1, nw2, nzrem;
+            {
                 const bool last_cc = cc == C - 1;
                 const uint32_t n_i = min(i + 1, n_units - 1);
                 open_window(n_i, 4 * (last_cc ? step + 1 : step) + quarter, last_cc ? lrn_next : lrn_step,
@@ -658,7 +641,6 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
             }
 
             // lanes with more than one element above level 1 (rare): splice on
-            if (!(dbg & 256))
             while (__ballot(nzrem != 0) != 0) splice_once(nw0, nw1, nw2, nzrem);
             cw0 = nw0; cw1 = nw1; cw2 = nw2;
         }
@@ -674,20 +656,10 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
         valid_step = valid_next;
     }
 
-    IXH_STAMP(3);
-#ifdef IXH_VARIANTS
-    if (trace && lane == 0) trace[4096 + blockIdx.x * 32 + wave * 2] = wall_clock64();
-#endif
     resolve();
-#ifdef IXH_VARIANTS
-    if (trace && lane == 0) trace[4096 + blockIdx.x * 32 + wave * 2 + 1] = wall_clock64();
-#endif
-    IXH_STAMP(4);
     __syncthreads();
-    IXH_STAMP(5);
 
     // ---- add the waves' row sums in wave order, write bf16 ----
-    if (dbg & 64) return;
     const uint32_t first_acc = L.waves + kRStages * kRStageBytes + kRQueue * 16;
     for (uint32_t t = tid; t < rows_here * MT; t += blockDim.x) {
         const uint32_t slot = t / MT, j = t - slot * MT;
@@ -695,9 +667,10 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
         float sum = 0.0f;
         for (uint32_t w = 0; w < n_waves; ++w)
             sum += *reinterpret_cast<const float *>(smem + first_acc + w * wave_lds_bytes(MT, C) + t * 4);
-        y[(int64_t)j * ldy + row0 + slot] = (uint16_t)f32_to_bf16_bits(sum);
+        // a workgroup owns whole rows: the one addition per output a split-K caller's fp32 vector takes, or bf16
+        if (y32) atomicAdd(&y32[(size_t)j * P.out_f + row0 + slot], sum);
+        else y[(int64_t)j * ldy + row0 + slot] = (uint16_t)f32_to_bf16_bits(sum);
     }
-    IXH_STAMP(6);
 }
 
 // ---------------------------------------------------------------------------
@@ -747,7 +720,8 @@ __host__ __device__ inline RowsXLds rowsx_layout(uint32_t rows_cap, uint32_t n_c
 template <int MT, bool ANY, int QCAP>
 __global__ void __launch_bounds__((MT > 4 ? kXMaxWaves / 2 : kXMaxWaves) * kWave)
 k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t quads_per_wg, uint32_t flags,
-                const uint16_t *__restrict__ x, int m, int64_t ldx, uint16_t *__restrict__ y, int64_t ldy) {
+                const uint16_t *__restrict__ x, int m, int64_t ldx, uint16_t *__restrict__ y, int64_t ldy,
+               float *__restrict__ y32) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
@@ -767,7 +741,10 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     // the pair table is addressed with (index bits | lane bits): it must sit at LDS address 0
     if ((uint32_t)(uintptr_t)(lds_ptr_t)smem != 0) {
         for (uint32_t t = tid; t < rows_here * MT; t += blockDim.x)
-            if ((int)(t % MT) < m) y[(int64_t)(t % MT) * ldy + row0 + t / MT] = 0x7FC0;  // NaN
+            if ((int)(t % MT) < m) {
+                if (y32) y32[(size_t)(t % MT) * P.out_f + row0 + t / MT] = __uint_as_float(0x7FC00000u);  // NaN
+                else y[(int64_t)(t % MT) * ldy + row0 + t / MT] = 0x7FC0;
+            }
         return;
     }
     uint32_t *const lut = reinterpret_cast<uint32_t *>(smem);            // [64][32]
@@ -1075,32 +1052,21 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         float sum = 0.0f;
         for (uint32_t w = 0; w < n_waves; ++w)
             sum += *reinterpret_cast<const float *>(smem + first_acc + w * wave_lds_bytes_x(MT, rows_cap, qcap) + t * 4);
-        y[(int64_t)j * ldy + row0 + slot] = (uint16_t)f32_to_bf16_bits(sum);
+        // a workgroup owns whole rows: the one addition per output a split-K caller's fp32 vector takes, or bf16
+        if (y32) atomicAdd(&y32[(size_t)j * P.out_f + row0 + slot], sum);
+        else y[(int64_t)j * ldy + row0 + slot] = (uint16_t)f32_to_bf16_bits(sum);
     }
 }
 
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
-#ifdef IXH_VARIANTS
-static unsigned long long *g_trace = nullptr;
-extern "C" int ixh_debug_trace(unsigned long long *host_out, int n) {
-    if (!g_trace) return -1;
-    return hipMemcpy(host_out, g_trace, (size_t)n * 8, hipMemcpyDeviceToHost) == hipSuccess ? 0 : -2;
-}
-#endif
-
-static int env_int(const char *name) {
-    const char *e = getenv(name);
-    return e ? atoi(e) : 0;
-}
 
 constexpr size_t kLdsLimit = 160 * 1024;
 
 template <int MT, int C, bool ANY>
 static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, const uint16_t *x, int m,
-                       int64_t ldx, uint16_t *y, int64_t ldy, hipStream_t s) {
-    static const int forced_quads = env_int("IXH_QUADS_PER_WG");
+                       int64_t ldx, uint16_t *y, int64_t ldy, float *y32, hipStream_t s) {
     const uint32_t waves = (n_chunks + C - 1) / C;
     const uint32_t n_quads = (P.out_f + 3) / 4;
     // how many workgroups a CU holds, by registers and LDS (asked once per workgroup size)
@@ -1123,7 +1089,7 @@ static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, c
     // a last round with a few workgroups in it would cost as much as a full one
     const uint32_t resident = (uint32_t)n_cu * (uint32_t)per_cu;
     const uint32_t rounds = (n_quads + resident * (kRSlots / 4) - 1) / (resident * (kRSlots / 4));
-    uint32_t quads = forced_quads > 0 ? (uint32_t)forced_quads : (n_quads + rounds * resident - 1) / (rounds * resident);
+    uint32_t quads = (n_quads + rounds * resident - 1) / (rounds * resident);
     quads = max(1u, min(quads, kRSlots / 4));
     const uint32_t groups = (n_quads + quads - 1) / quads;
     const uint32_t rows_cap = min(quads * 4, P.out_f);
@@ -1140,15 +1106,8 @@ static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, c
             raised = true;
         }
     }
-#ifdef IXH_VARIANTS
-    static const int dbg = env_int("IXH_DBG");
-    if (!g_trace) (void)hipMalloc(&g_trace, 4096 * 8 * 8);
-    hipLaunchKernelGGL((k_gemv358_rows<MT, C, ANY>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks,
-                       quads | ((uint32_t)dbg << 16), flags, x, m, ldx, y, ldy, g_trace);
-#else
     hipLaunchKernelGGL((k_gemv358_rows<MT, C, ANY>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks, quads,
-                       flags, x, m, ldx, y, ldy);
-#endif
+                       flags, x, m, ldx, y, ldy, y32);
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }
 
@@ -1156,7 +1115,7 @@ static int launch_rows(const Dev &P, const int32_t *prefix, uint32_t n_chunks, c
 // fit beside them.
 template <int MT, bool ANY>
 static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, const uint16_t *x, int m, int64_t ldx,
-                        uint16_t *y, int64_t ldy, hipStream_t s) {
+                        uint16_t *y, int64_t ldy, float *y32, hipStream_t s) {
     const uint32_t n_quads = (P.out_f + 3) / 4;
     static const int n_cu = [] {
         int dev = 0, v = 256;
@@ -1227,29 +1186,29 @@ static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
     const size_t lds = rowsx_layout(min(quads * 4, P.out_f), n_chunks, waves, MT, k_qcap).total;
     if (k_qcap == 256)
         hipLaunchKernelGGL((k_gemv358_rowsx<MT, ANY, 256>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix,
-                           n_chunks, quads, flags, x, m, ldx, y, ldy);
+                           n_chunks, quads, flags, x, m, ldx, y, ldy, y32);
     else
         hipLaunchKernelGGL((k_gemv358_rowsx<MT, ANY, 128>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix,
-                           n_chunks, quads, flags, x, m, ldx, y, ldy);
+                           n_chunks, quads, flags, x, m, ldx, y, ldy, y32);
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }
 
 // Row-block kernel for the shapes whose x slices fit the register budget of a
 // full workgroup; IXH_EUNSUPPORTED sends the caller to the column kernel.
 int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
-                         int64_t ldy, hipStream_t s) {
+                         int64_t ldy, float *y32, hipStream_t s) {
     const bool any = !(P.n_levels == 3 && P.bits[1] == 5);  // not (3,5,8): the resolver that walks the nested bitmaps
     if (((uintptr_t)x & 15u) != 0 || (m > 1 && (ldx & 7) != 0)) return IXH_EUNSUPPORTED;
     const uint32_t n_chunks = P.in_f / kFastChunk;
-    static const int shared_x = getenv("IXH_GEMV_SHARED_X") ? atoi(getenv("IXH_GEMV_SHARED_X")) : 8;
-    // IXH_GEMV_SHARED_X (development): 0 = never the shared-x kernel, 1 = for one activation row only, 2 = up to
-    // two rows, 4 = up to four, 8 = up to eight (default)
+    // option "gemv_shared_x" (ixh_set_option): 0 = never the shared-x kernel, 1 = for one activation row only, 2 = up
+    // to two rows, 4 = up to four, 8 = up to eight (default)
+    const int shared_x = g_opt_gemv_shared_x.load(std::memory_order_relaxed);
     if (shared_x && P.in_f <= 65536u && P.out_f % 4u == 0 && (m == 1 || (m == 2 && shared_x >= 2) || (m <= 4 && shared_x >= 4) || (m <= 8 && shared_x >= 8))) {
         int rc;
-        if (m == 1) rc = any ? launch_rowsx<1, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s) : launch_rowsx<1, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
-        else if (m == 2) rc = any ? launch_rowsx<2, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s) : launch_rowsx<2, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
-        else if (m <= 4) rc = any ? launch_rowsx<4, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s) : launch_rowsx<4, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
-        else rc = any ? launch_rowsx<8, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s) : launch_rowsx<8, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
+        if (m == 1) rc = any ? launch_rowsx<1, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, y32, s) : launch_rowsx<1, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, y32, s);
+        else if (m == 2) rc = any ? launch_rowsx<2, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, y32, s) : launch_rowsx<2, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, y32, s);
+        else if (m <= 4) rc = any ? launch_rowsx<4, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, y32, s) : launch_rowsx<4, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, y32, s);
+        else rc = any ? launch_rowsx<8, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, y32, s) : launch_rowsx<8, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, y32, s);
         if (rc != IXH_EUNSUPPORTED) return rc;
     }
     const uint32_t c = (n_chunks + kRMaxWaves - 1) / kRMaxWaves;  // blocks per wave: a workgroup has at most kRMaxWaves waves
@@ -1257,8 +1216,8 @@ int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x,
     const int mt = m == 1 ? 1 : (m == 2 ? 2 : 4);
 #define IXH_ROWS(MTV, CV) \
     if (mt == MTV && c == CV)                                                                  \
-        return any ? launch_rows<MTV, CV, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, s)     \
-                   : launch_rows<MTV, CV, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, s);
+        return any ? launch_rows<MTV, CV, true>(P, prefix, n_chunks, x, m, ldx, y, ldy, y32, s)     \
+                   : launch_rows<MTV, CV, false>(P, prefix, n_chunks, x, m, ldx, y, ldy, y32, s);
     IXH_ROWS(1, 1) IXH_ROWS(1, 2) IXH_ROWS(1, 3) IXH_ROWS(1, 4)
     IXH_ROWS(2, 1) IXH_ROWS(2, 2)
     IXH_ROWS(4, 1)

@@ -91,11 +91,9 @@ __device__ __forceinline__ void stage_unit(const Dev &P, uint32_t u, uint32_t ch
     uint32_t off = 0;  // bytes used so far, a multiple of 16
     auto copy = [&](__amdgpu_buffer_rsrc_t rs, uint32_t first_word, uint32_t n_words) {
         const uint32_t n4 = max((n_words + 3u) >> 2, 1u);  // 16-byte pieces, one per lane (at most 33)
-#ifndef IXH_PF_NO_STAGE
         if (lane < n4)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)(uintptr_t)(slot + off), 16,
                                                      (int)(first_word * 4u + lane * 16u), 0, 0, 0);
-#endif
         off += n4 * 16u;
     };
 #pragma unroll

@@ -18,3 +18,16 @@ def oracle():
 
     ix_oracle.build()
     return ix_oracle
+
+
+@pytest.fixture
+def force_decoder():
+    """Force one of the library's decoders for the duration of a test (``ixh_set_option``), then give the choice
+    back to the library."""
+    from ixrun_amd import _lib
+
+    def force(name: str) -> None:
+        _lib.set_option("decode_kernel", name)
+
+    yield force
+    _lib.set_option("decode_kernel", "auto")

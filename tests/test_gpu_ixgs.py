@@ -33,11 +33,11 @@ def packed_from_ints(oracle, q, scales, out_f, in_f, group):
 
 
 @pytest.fixture(params=["by_mix", "staged", "dense"])
-def decoder(request, monkeypatch):
+def decoder(request, force_decoder):
     """Which of the two unit-512 decoders runs: chosen by the mix of tiers, or forced (level by level where the
     group size allows it, or the one that stages the streams)."""
     if request.param != "by_mix":
-        monkeypatch.setenv("IXH_DECODE_KERNEL", request.param)
+        force_decoder(request.param)
     return request.param
 
 

@@ -149,12 +149,12 @@ def test_decode_bf16_only(oracle, dev, kind, shape, level_bits):
 @pytest.mark.parametrize("shape", [(1, 1), (1, 31), (1, 512), (3, 171), (5, 413), (33, 1000), (64, 1536), (300, 1031),
                                    (256, 4608), (17, 2048), (1, 2049), (4, 512), (8, 512), (52, 512), (200, 1024),
                                    (1000, 2048), (2600, 1024)])
-def test_decode_358_each_decoder(oracle, dev, monkeypatch, kind, shape, decoder):
+def test_decode_358_each_decoder(oracle, dev, force_decoder, kind, shape, decoder):
     """(3,5,8) to bf16 at unit 512 through each of the three decoders, whatever the mix of levels would choose:
     the level-by-level one (partial last lane, partial last span, tensors smaller than a lane), the one that
     stages the streams, and the row-block one (whole unit-quads only: other sizes fall through to the staged one;
     with dense mixes its record queue is resolved every few units)."""
-    monkeypatch.setenv("IXH_DECODE_KERNEL", decoder)
+    force_decoder(decoder)
     if kind == "all_l3":
         g = torch.Generator("cpu").manual_seed(shape[1])
         w = ((torch.randint(0, 2, shape, generator=g) * 2 - 1) * (0.25 + 0.5 * torch.rand(shape, generator=g))).bfloat16()
@@ -174,11 +174,11 @@ def test_decode_358_each_decoder(oracle, dev, monkeypatch, kind, shape, decoder)
 @pytest.mark.parametrize("level_bits", [(3, 4, 5, 6, 8), (3, 8), (3, 3, 8), (3, 4, 8), (3, 5, 6, 7, 8), (3, 4, 5, 6, 7, 8)])
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("shape", [(8, 512), (64, 1536), (1000, 2048)])
-def test_decode_row_block_decoder_other_schemes(oracle, dev, monkeypatch, kind, shape, level_bits):
+def test_decode_row_block_decoder_other_schemes(oracle, dev, force_decoder, kind, shape, level_bits):
     """The row-block decoder takes every scheme whose first level has 3 bits; its elements above level 1 are followed
     down the nested bitmaps one by one.  Forced here for every mix (it is chosen only for tensors that are almost all
     level 1)."""
-    monkeypatch.setenv("IXH_DECODE_KERNEL", "rows")
+    force_decoder("rows")
     p = make_packed(kind, *shape, level_bits)
     dp = device_packed(p, dev)
     table = dp.prefix_build(512)
