@@ -100,6 +100,8 @@ class StreamingLinear(nn.Module):
         else:
             self._bias = None
         self._w_buf = None  # set by the engine
+        # the shared scratch takes its final size now, not inside some later forward (or graph capture)
+        shared_workspace(self._scale.device, self._dp.gemv_workspace_bytes(self._unit, MAX_FUSED_ROWS))
 
     def _bind(self):
         n_levels = len(self.level_bits)

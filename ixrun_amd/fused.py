@@ -108,36 +108,46 @@ def pick_unit(in_f: int) -> int:
     return max(in_f, 1)
 
 
-_loose_cache: dict = {}
+_loose_cache: dict = {}  # id(b1) -> (weakref to b1, signature, rank table, unit); the entry dies with b1
 
 
 def _tables_for(b1, b2, l1, l2, l3, scale, out_f, in_f):
-    """DevicePacked + rank table for loose (3,5,8) tensors, remembered per bitmap tensor."""
+    """DevicePacked + rank table for loose (3,5,8) tensors.  The table is remembered for as long as ``b1`` lives
+    (a weak reference: the cache keeps no packed tensor alive); the argument struct is rebuilt from the live
+    tensors on every call."""
+    dp = _lib.DevicePacked((3, 5, 8), out_f, in_f, [b1, b2], [l1, l2, l3], scale.reshape(1))
     key = id(b1)
-    hit = _loose_cache.get(key)
     sig = (b1.data_ptr(), b2.data_ptr(), l1.data_ptr(), l2.data_ptr(), l3.data_ptr(), scale.data_ptr(),
            b1._version, b2._version, out_f, in_f)
+    hit = _loose_cache.get(key)
     if hit is not None and hit[0]() is b1 and hit[1] == sig:
-        return hit[2], hit[3], hit[4]
-    for k in [k for k, v in _loose_cache.items() if v[0]() is None]:
-        del _loose_cache[k]
-    dp = _lib.DevicePacked((3, 5, 8), out_f, in_f, [b1, b2], [l1, l2, l3], scale.reshape(1))
+        return dp, hit[2], hit[3]
     unit = pick_unit(in_f)
     table = dp.prefix_build(unit)
-    _loose_cache[key] = (weakref.ref(b1), sig, dp, table, unit)
+    _loose_cache[key] = (weakref.ref(b1, lambda _ref, _key=key: _loose_cache.pop(_key, None)), sig, table, unit)
     return dp, table, unit
 
 
-_workspaces: dict = {}
+_workspaces: dict = {}  # device -> the scratch in use
+_retired: list = []     # replaced scratches: graphs captured earlier still write their partial sums there
 
 
 def shared_workspace(device, nbytes: int) -> torch.Tensor | None:
-    """One grow-only fp32 scratch per device for the per-chunk partial sums.
-    Layers run one after another on a stream, so they can share it."""
+    """One fp32 scratch per device for the partial sums of the kernels that combine pieces of a row.
+
+    Layers run one after another on the device's stream and every kernel pair writes its partial sums before it
+    reads them, so the layers share it (callers that run layers on several streams of one device at once must give
+    ``gemv`` / ``gemm`` workspaces of their own).  It only grows, to at least twice its size, and a replaced buffer
+    is never freed: a hipGraph captured earlier holds its address and goes on using it.  ``StreamingLinear`` asks
+    for the size of its widest fused call when it is built, so a deployed model does not grow it afterwards."""
     if nbytes == 0:
         return None
+    device = torch.device(device)
     ws = _workspaces.get(device)
     if ws is None or ws.numel() * 4 < nbytes:
+        if ws is not None:
+            _retired.append(ws)
+            nbytes = max(nbytes, ws.numel() * 8)
         ws = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=device)
         _workspaces[device] = ws
     return ws

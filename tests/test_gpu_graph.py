@@ -104,3 +104,107 @@ def test_graph_replay_many_rows(shared_buffer):
         torch.cuda.synchronize()
         assert torch.equal(static_y, eager), f"replay {rep} differs from the eager result"
         del junk
+
+
+def _capture(fn, static_x):
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn(static_x)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y = fn(static_x)
+    return graph, static_y
+
+
+def test_graph_64_layers_of_5120x5120():
+    """BASELINE config 5b as stated: a sequence of 64 packed 5120 x 5120 layers (64 distinct device copies, 0.85 GB
+    of packed bytes), every per-layer launch captured in one hipGraph.  Replays equal the eager pass bit for bit; the
+    first and the last layer's outputs are checked against the fp64 oracle on the inputs they really saw."""
+    from ixrun_amd.engine import StreamingLinear
+    from ixrun_amd.quantize import int8x_quantize
+    from oracle import ix_oracle
+    from test_gpu_parity import check_outputs
+
+    dev = torch.device("cuda:0")
+    width, n_layers, n_distinct = 5120, 64, 4
+    packed = [int8x_quantize(student_t_weight(width, width, seed=k)) for k in range(n_distinct)]
+    layers = [StreamingLinear(packed[k % n_distinct]) for k in range(n_layers)]
+
+    def chain(x, keep=None):
+        h = x
+        for k, sl in enumerate(layers):
+            if keep is not None and k == n_layers - 1:
+                keep["last_in"] = h.clone()
+            h = sl(h) * 0.7  # output std is 1.43 x input std at this width: keep the chain in range
+            if keep is not None and k == 0:
+                keep["first_out"] = h.clone()
+        return h
+
+    x = activations(1, width, seed=3).to(dev)
+    seen = {}
+    eager = chain(x, seen).clone()
+    torch.cuda.synchronize()
+    assert torch.isfinite(eager.float()).all() and eager.float().abs().max() > 0
+
+    # layer outputs against the oracle (the 0.7 is a bf16 multiply: applied to the oracle's bf16-rounded result)
+    for w, xin, got in ((packed[0], x, seen["first_out"]), (packed[(n_layers - 1) % n_distinct], seen["last_in"], eager)):
+        y64 = ix_oracle.gemm_f64(ix_oracle.decode_packed_bf16(w), bf16_bits(xin))
+        y_layer = torch.from_numpy(ix_oracle.bf16_bits_to_f32(ix_oracle.f32_to_bf16_bits(y64.astype(np.float32))))
+        want = (y_layer.bfloat16() * 0.7).double().numpy()
+        err = np.linalg.norm(got.double().cpu().numpy() - want) / np.linalg.norm(want)
+        assert err <= 1e-3, err
+
+    static_x = x.clone()
+    graph, static_y = _capture(chain, static_x)
+    for rep in range(3):
+        junk = torch.randn(1 << 16, device=dev).sum()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y, eager), f"replay {rep} differs from the eager pass"
+        del junk
+    x2 = activations(1, width, seed=4).to(dev)
+    static_x.copy_(x2)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(static_y, chain(x2))
+
+
+def test_graph_survives_a_larger_workspace_request():
+    """A graph captured while the shared scratch was small keeps working after a bigger layer made the scratch grow:
+    the replaced buffer stays alive, so the replay neither reads freed memory nor writes into tensors allocated
+    afterwards."""
+    from ixrun_amd import fused
+    from ixrun_amd.engine import StreamingLinear
+    from ixrun_amd.quantize import int8x_quantize
+
+    dev = torch.device("cuda:0")
+    fused._workspaces.pop(dev, None)  # start from no scratch, whatever earlier tests left
+    # five-level layers with a dense mix: the staged kernel, whose pieces of a row meet in the workspace
+    layers = [StreamingLinear(int8x_quantize(outlier_weight(256, 2048, seed=k), (3, 4, 5, 6, 8))) for k in range(2)]
+    layers.append(StreamingLinear(int8x_quantize(outlier_weight(2048, 256, seed=9), (3, 4, 5, 6, 8))))
+
+    def chain(x):
+        return layers[1](layers[2](layers[0](x)))
+
+    x = activations(3, 2048, seed=3).to(dev)
+    eager = chain(x).clone()
+    small = fused._workspaces[dev]
+    static_x = x.clone()
+    graph, static_y = _capture(chain, static_x)
+    assert fused._workspaces[dev] is small  # the capture itself did not grow it
+
+    big = StreamingLinear(int8x_quantize(outlier_weight(4096, 8192, seed=5), (3, 4, 5, 6, 8)))
+    big(activations(16, 8192, seed=1).to(dev))
+    assert fused._workspaces[dev] is not small and any(t is small for t in fused._retired)
+    del small
+    torch.cuda.synchronize()
+    canaries = [torch.full((1 << 18,), 3.0, device=dev) for _ in range(16)]  # what a freed scratch would be given to
+    for rep in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y, eager), f"replay {rep} after the scratch grew"
+        assert all(bool((c == 3.0).all()) for c in canaries)

@@ -407,6 +407,66 @@ def test_reference_call_surface(oracle, dev, shape):
         assert rel_l2(got, want) < 6e-3  # bias add and output are bf16-rounded
 
 
+@pytest.fixture(scope="module")
+def gate_up_layer(oracle, dev):
+    """BASELINE config 4's layer, 17408 x 5120 Student-t, packed once for its four batch sizes."""
+    from ixrun_amd.engine import StreamingLinear
+
+    p = quantize(student_t_weight(17408, 5120, seed=0))
+    w_bits = oracle.decode_packed_bf16(p)
+    return StreamingLinear(p), w_bits
+
+
+@pytest.mark.parametrize("m", [2, 4, 8, 16])
+def test_full_size_config4_every_batch(oracle, dev, gate_up_layer, m):
+    """BASELINE config 4 as stated: 17408 x 5120 with M in {2, 4, 8, 16} activation rows, each through the kernel the
+    library picks for it (2 and 4 rows: 16 waves; 8 rows: the eight-wave variant; 16 rows: more than one launch)."""
+    sl, w_bits = gate_up_layer
+    x = activations(m, 5120, seed=1)
+    y = sl(x.to(dev))
+    assert y.shape == (m, 17408)
+    check_outputs(bf16_bits(y), oracle.gemm_f64(w_bits, bf16_bits(x)), f"config 4 m={m}")
+
+
+def test_full_size_split_k_contract(oracle, dev):
+    """The reference's split-K call on the headline shape (ixrun/engine.py:148-159: fused_gemv(..., chunk=8704, y32)
+    on 5120 x 17408): the caller-zeroed fp32 vector comes back holding the sums, and a second call adds to it."""
+    from ixrun_amd.fused import compute_row_prefixes, fused_gemv, _pick_split
+
+    out_f, in_f = 5120, 17408
+    p = quantize(student_t_weight(out_f, in_f, seed=0))
+    assert _pick_split(in_f) == 2
+    chunk = in_f // 2
+    x = activations(1, in_f, seed=1).reshape(in_f)
+    y64 = oracle.gemm_f64(oracle.decode_packed_bf16(p), bf16_bits(x).reshape(1, -1))
+    b1, b2 = (t.to(dev) for t in p["bitmaps"])
+    l1, l2, l3 = (t.to(dev) for t in p["streams"])
+    q1c, q2c = compute_row_prefixes(p, chunk)
+    y32 = torch.zeros(out_f, dtype=torch.float32, device=dev)
+    args = (x.to(dev), b1, b2, l1, l2, l3, q1c.to(dev), q2c.to(dev), p["scale"].to(dev), out_f, in_f)
+    ret = fused_gemv(*args, chunk=chunk, y32=y32)
+    assert ret is y32
+    once = y32.cpu().numpy().copy()
+    check_outputs(once.reshape(1, -1), y64, "split-K 5120x17408")
+    fused_gemv(*args, chunk=chunk, y32=y32)  # the contract is "add": a second call doubles every entry
+    assert np.array_equal(y32.cpu().numpy(), once + once)
+
+
+def test_headline_kernel_is_reproducible(oracle, dev):
+    """Repeat launches of the row-block kernel on a layer that is almost all level 1 (the headline workload's kernel,
+    5120 x 17408 Student-t) give the same bits, for one and for four activation rows."""
+    from ixrun_amd.engine import StreamingLinear
+
+    p = quantize(student_t_weight(5120, 17408, seed=0))
+    assert p["counts"][0] >= 0.97 * p["N"]
+    sl = StreamingLinear(p)
+    for m in (1, 4):
+        x = activations(m, 17408, seed=5).to(dev)
+        first = bf16_bits(sl(x))
+        for _ in range(5):
+            assert np.array_equal(bf16_bits(sl(x)), first), m
+
+
 @pytest.mark.parametrize("shape,m", [((5120, 5120), 1), ((5120, 17408), 1), ((17408, 5120), 4)])
 def test_full_size_layers(oracle, dev, shape, m):
     """BASELINE configs 2, 3 and 4 at full size: decoded int8 bit-exact, outputs within tolerance."""

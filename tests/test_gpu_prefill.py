@@ -115,14 +115,23 @@ def test_streaming_linear_takes_the_fused_gemm(oracle, dev):
     check_outputs(bf16_bits(y.reshape(48, out_f)), y64, "StreamingLinear m=48")
 
 
-def test_full_size_prefill(oracle, dev):
-    """BASELINE config 5: 5120 x 5120 five-level, 512 rows; a sample of output columns against the oracle."""
-    out_f, in_f, m = 5120, 5120, 512
+def _full_size_prefill(oracle, dev, out_f, in_f, m, what):
     p = quantize(student_t_weight(out_f, in_f, seed=0), (3, 4, 5, 6, 8))
     dp = device_packed(p, dev)
     x = activations(m, in_f, seed=1)
     y = run_gemm(dp, x, dev)
     w_bits = oracle.decode_packed_bf16(p)
-    rows = np.r_[0:64, 2500:2564, 5056:5120]
+    rows = np.r_[0:64, 2500:2564, out_f - 64:out_f]
     y64 = oracle.gemm_f64(np.ascontiguousarray(w_bits[rows]), bf16_bits(x))
-    check_outputs(np.ascontiguousarray(y[:, rows]), y64, "full-size prefill")
+    check_outputs(np.ascontiguousarray(y[:, rows]), y64, what)
+
+
+def test_full_size_prefill_square_layer(oracle, dev):
+    """5120 x 5120 five-level, 512 rows through ixh_gemm; 192 sampled output columns against the oracle."""
+    _full_size_prefill(oracle, dev, 5120, 5120, 512, "5120x5120 five-level m=512")
+
+
+def test_full_size_prefill_config5(oracle, dev):
+    """BASELINE config 5 as stated: W 5120 x 17408 in the five-level scheme (3,4,5,6,8), 512 activation rows, through
+    ixh_gemm (decode into LDS tiles, bf16 MFMA, fp32 accumulate); 192 sampled output columns against the fp64 oracle."""
+    _full_size_prefill(oracle, dev, 5120, 17408, 512, "config 5: 5120x17408 five-level m=512")
