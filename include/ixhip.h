@@ -159,6 +159,21 @@ int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, cons
 size_t ixh_gemv_workspace_bytes(const IxhPacked *packed, int64_t chunk, int32_t m, uint32_t flags);
 
 /*
+ * ixh_gemv for callers that cannot allocate device memory (code under stream capture, serving loops and
+ * harnesses that forbid hipMalloc); it has no counterpart in the reference.  Same arguments, kernels and results
+ * as ixh_gemv without IXH_GEMV_ATOMIC, but the partial sums of the kernels that need a workspace go to a buffer
+ * of IXH_NOALLOC_WORKSPACE_BYTES that is part of the library's code object (every GPU the library runs on holds
+ * it until the process ends).  The call allocates and frees nothing.  A request whose partial sums need more
+ * (ixh_gemv_workspace_bytes) fails with IXH_EWORKSPACE; IXH_GEMV_ATOMIC fails with IXH_EINVAL.  The device that
+ * is current at the call must be the one the tensors live on; the first call on a device looks the buffer's
+ * address up (make that call outside stream capture).  All calls on one GPU share the buffer: calls that may
+ * overlap there (two streams, two threads) race on it and must be ordered by the caller.
+ */
+#define IXH_NOALLOC_WORKSPACE_BYTES (16u << 20)
+int ixh_gemv_noalloc(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, const uint16_t *x, int32_t m,
+                     int64_t ldx, uint16_t *y, int64_t ldy, uint32_t flags, ixh_stream_t stream);
+
+/*
  * Fused decode + GEMM for many activation rows (prefill, m > 16 in the reference's
  * dispatch): y[j, r] = bf16( sum_k f32(x[j, k]) * f32(w[r, k]) ) with
  * w = bf16(f32(v) * f32(scale)) decoded into on-chip memory tile by tile and multiplied

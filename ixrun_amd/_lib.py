@@ -58,7 +58,7 @@ _ENV_GEMV_FLAGS = int(os.environ.get("IXH_GEMV_FLAGS", "0"))
 
 EXPORTS = (
     "ixh_version", "ixh_last_error", "ixh_set_option", "ixh_prefix_entries", "ixh_prefix_build", "ixh_decode",
-    "ixh_gemv", "ixh_gemv_workspace_bytes", "ixh_gemm", "ixh_gemm_workspace_bytes",
+    "ixh_gemv", "ixh_gemv_workspace_bytes", "ixh_gemv_noalloc", "ixh_gemm", "ixh_gemm_workspace_bytes",
     "ixh_encode_workspace_bytes", "ixh_encode_scan", "ixh_encode_pack", "ixh_decode_gs",
 )
 
@@ -90,6 +90,11 @@ def lib() -> C.CDLL:
         L.ixh_gemv.argtypes = [
             C.POINTER(IxhPacked), C.c_void_p, C.c_int64, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p,
             C.c_int64, C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint32, C.c_void_p,
+        ]
+        L.ixh_gemv_noalloc.restype = C.c_int
+        L.ixh_gemv_noalloc.argtypes = [
+            C.POINTER(IxhPacked), C.c_void_p, C.c_int64, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p,
+            C.c_int64, C.c_uint32, C.c_void_p,
         ]
         L.ixh_gemv_workspace_bytes.restype = C.c_size_t
         L.ixh_gemv_workspace_bytes.argtypes = [C.POINTER(IxhPacked), C.c_int64, C.c_int32, C.c_uint32]
@@ -248,6 +253,24 @@ class DevicePacked:
             workspace.data_ptr() if workspace is not None else None,
             workspace.numel() * workspace.element_size() if workspace is not None else 0,
             int(flags), current_stream(self.device)))
+
+    def gemv_noalloc(self, table, chunk, x, y, flags=0) -> None:
+        """``gemv`` through the entry point that allocates nothing: partial sums go to the library's own buffer
+        (``IXH_NOALLOC_WORKSPACE_BYTES``); larger requests raise ``IxhError(IXH_EWORKSPACE)``."""
+        if not x.is_cuda:
+            raise RuntimeError(f"x must live on the GPU (got {x.device}); the HIP path has no CPU fallback")
+        if x.dtype != torch.bfloat16:
+            raise ValueError("x must be bf16")
+        x2 = x.reshape(-1, self.in_f)
+        if x2.stride(1) != 1:
+            raise ValueError("x rows must be contiguous")
+        m = x2.shape[0]
+        ldx = x2.stride(0) if m > 1 else self.in_f
+        ldy = y.stride(0) if (y.dim() == 2 and m > 1) else self.out_f
+        with torch.cuda.device(self.device):
+            check(lib().ixh_gemv_noalloc(
+                C.byref(self.struct), table.data_ptr(), int(chunk), x2.data_ptr(), m, ldx, y.data_ptr(), ldy,
+                int(flags), current_stream(self.device)))
 
     def gemm_workspace_bytes(self, m: int) -> int:
         return int(lib().ixh_gemm_workspace_bytes(C.byref(self.struct), int(m)))

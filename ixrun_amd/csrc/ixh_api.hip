@@ -5,6 +5,7 @@
 #include <string.h>
 
 #include <cstdlib>
+#include <mutex>
 
 #include "ixh_dev.h"
 #include "ixh_fast358.h"
@@ -182,9 +183,9 @@ size_t ixh_gemv_workspace_bytes(const IxhPacked *packed, int64_t chunk, int32_t 
     return n_chunks * (size_t)m * d.out_f * sizeof(float);
 }
 
-int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, const uint16_t *x, int32_t m,
-             int64_t ldx, uint16_t *y, int64_t ldy, float *y32, void *workspace, size_t workspace_bytes,
-             uint32_t flags, ixh_stream_t stream) {
+static int gemv_any(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, const uint16_t *x, int32_t m,
+                    int64_t ldx, uint16_t *y, int64_t ldy, float *y32, void *workspace, size_t workspace_bytes,
+                    uint32_t flags, ixh_stream_t stream) {
     Dev d;
     int rc = to_dev(packed, &d);
     if (rc) return rc;
@@ -262,6 +263,63 @@ int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, cons
     }
     if (rc == IXH_ELAUNCH) set_error("gemv: launch failed");
     return rc;
+}
+
+int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, const uint16_t *x, int32_t m,
+             int64_t ldx, uint16_t *y, int64_t ldy, float *y32, void *workspace, size_t workspace_bytes,
+             uint32_t flags, ixh_stream_t stream) {
+    return gemv_any(packed, prefix, chunk, x, m, ldx, y, ldy, y32, workspace, workspace_bytes, flags, stream);
+}
+
+// ---- ixh_gemv for callers that may not allocate: the partial sums go to a buffer that is part of the library ----
+// The array lives in the code object, once per GPU the library runs on, until the process ends.  In host code its
+// name is only a handle for hipGetSymbolAddress: kernels and everything else take the per-device address looked
+// up below, never the name.
+static __device__ __align__(256) unsigned char scratch[IXH_NOALLOC_WORKSPACE_BYTES];
+
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices];  // address of `scratch` on each device, looked up on first use there
+static std::mutex g_scratch_lock;
+
+// the current device's copy of `scratch`
+static int scratch_of_current_device(void **out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("gemv_noalloc: no current device (or its index %d is beyond %d)", dev, kMaxDevices - 1);
+        return IXH_ELAUNCH;
+    }
+    std::lock_guard<std::mutex> guard(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            set_error("gemv_noalloc: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+            return IXH_ELAUNCH;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return IXH_OK;
+}
+
+int ixh_gemv_noalloc(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, const uint16_t *x, int32_t m,
+                     int64_t ldx, uint16_t *y, int64_t ldy, uint32_t flags, ixh_stream_t stream) {
+    if (flags & IXH_GEMV_ATOMIC) {
+        set_error("gemv_noalloc: IXH_GEMV_ATOMIC takes no workspace; call ixh_gemv");
+        return IXH_EINVAL;
+    }
+    const size_t need = ixh_gemv_workspace_bytes(packed, chunk, m, flags);  // 0 also for arguments gemv_any rejects
+    if (need > (size_t)IXH_NOALLOC_WORKSPACE_BYTES) {
+        set_error("gemv_noalloc: this call needs %zu bytes of partial sums, the built-in buffer holds %zu; "
+                  "call ixh_gemv with a workspace of your own", need, (size_t)IXH_NOALLOC_WORKSPACE_BYTES);
+        return IXH_EWORKSPACE;
+    }
+    void *ws = nullptr;
+    const int rc = scratch_of_current_device(&ws);
+    if (rc) return rc;
+    // every partial sum the second kernel reads was written by the first in the same call: nothing to clear
+    return gemv_any(packed, prefix, chunk, x, m, ldx, y, ldy, nullptr, ws, (size_t)IXH_NOALLOC_WORKSPACE_BYTES, flags,
+                    stream);
 }
 
 size_t ixh_gemm_workspace_bytes(const IxhPacked *packed, int32_t m) {

@@ -51,6 +51,18 @@ def test_entries_and_workspace_sizes():
     assert lib.ixh_gemv_workspace_bytes(C.byref(s), 512, 3, _lib.IXH_GEMV_ATOMIC) == 0
 
 
+def test_noalloc_entry_rejects_oversize_on_the_host():
+    """ixh_gemv_noalloc refuses, before any GPU call, a request whose partial sums exceed its built-in buffer, and
+    the atomic mode (which takes no workspace)."""
+    lib = _lib.lib()
+    s = _packed(out_f=1 << 14, in_f=1 << 14, bm0_words=1 << 23)
+    assert lib.ixh_gemv_workspace_bytes(C.byref(s), 512, 16, 0) == 32 * 16 * (1 << 14) * 4 > (16 << 20)
+    rc = lib.ixh_gemv_noalloc(C.byref(s), 0x1000, 512, 0x1000, 16, 1 << 14, 0x1000, 1 << 14, 0, None)
+    assert rc == -4 and b"built-in buffer" in lib.ixh_last_error()
+    rc = lib.ixh_gemv_noalloc(C.byref(s), 0x1000, 512, 0x1000, 1, 1 << 14, 0x1000, 1 << 14, _lib.IXH_GEMV_ATOMIC, None)
+    assert rc == -1
+
+
 @pytest.mark.parametrize("mutate,needle", [
     (lambda s: setattr(s, "n_levels", 1), "n_levels"),
     (lambda s: s.level_bits.__setitem__(2, 7), "last level"),

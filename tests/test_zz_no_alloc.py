@@ -1,0 +1,92 @@
+"""The entry point that allocates nothing (ixh_gemv_noalloc) against ixh_gemv, through the C ABI.
+
+Both run the same kernels; the only difference is where the partial sums of the kernels that need a workspace
+live (the library's built-in buffer instead of a caller's tensor), so the outputs must be equal bit for bit.  Each
+case calls twice in a row, the second time with a smaller tensor, so that what the first call left in the shared
+buffer would show.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import activations, bf16_bits, calibrated_weight, outlier_weight, student_t_weight
+
+pytestmark = pytest.mark.gpu
+
+LIMIT = 16 << 20
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from ixrun_amd import _lib
+
+    assert _lib.lib().ixh_version() >= 100
+    return torch.device("cuda:0")
+
+
+def _layer(recipe, out_f, in_f, dev, level_bits=(3, 5, 8)):
+    from ixrun_amd import _lib
+    from ixrun_amd.quantize import int8x_quantize
+
+    w = {"student_t": lambda: student_t_weight(out_f, in_f, seed=2),
+         "outlier": lambda: outlier_weight(out_f, in_f, seed=2),
+         "calibrated": lambda: calibrated_weight(out_f, in_f, seed=2, scale=0.0123046875)[0]}[recipe]()
+    dp = _lib.DevicePacked.from_dict(int8x_quantize(w, level_bits), dev)
+    return dp, dp.prefix_build(512)
+
+
+def _both(dp, table, x, flags, dev):
+    m = x.shape[0]
+    need = dp.gemv_workspace_bytes(512, m, flags)
+    ws = torch.empty(max(need // 4, 1), dtype=torch.float32, device=dev)
+    y_ref = torch.zeros((m, dp.out_f), dtype=torch.bfloat16, device=dev)
+    dp.gemv(table, 512, x, y=y_ref, workspace=ws, flags=flags)
+    y_new = torch.full((m, dp.out_f), 7.0, dtype=torch.bfloat16, device=dev)
+    dp.gemv_noalloc(table, 512, x, y_new, flags=flags)
+    torch.cuda.synchronize()
+    return bf16_bits(y_ref), bf16_bits(y_new), need
+
+
+@pytest.mark.parametrize("recipe,level_bits", [("calibrated", (3, 5, 8)), ("outlier", (3, 5, 8)), ("student_t", (3, 5, 8)),
+                                               ("outlier", (3, 4, 5, 6, 8))])
+@pytest.mark.parametrize("m", [1, 3, 8, 16])
+def test_noalloc_equals_gemv_twice_in_a_row(dev, recipe, level_bits, m):
+    """Big tensor first, then a smaller one: the second call's partial sums cover only a part of what the first left
+    in the buffer.  Flags: the library's own choice, the column-block kernel and the staged kernel (both always go
+    through the workspace), the wave-per-unit kernel."""
+    from ixrun_amd import _lib
+
+    big, big_t = _layer(recipe, 640, 4608, dev, level_bits)
+    small, small_t = _layer(recipe, 96, 1536, dev, level_bits)
+    used = 0
+    for flags in (0, _lib.IXH_GEMV_COLUMN_KERNEL, _lib.IXH_GEMV_STAGED, _lib.IXH_GEMV_FORCE_GENERIC):
+        for dp, table in ((big, big_t), (small, small_t)):
+            x = activations(m, dp.in_f, seed=3 + m).to(dev)
+            y_ref, y_new, need = _both(dp, table, x, flags, dev)
+            assert need <= LIMIT
+            used = max(used, need)
+            assert np.array_equal(y_ref, y_new), (recipe, level_bits, m, flags, dp.out_f)
+    assert used > 0  # at least one of the routes really went through the buffer
+
+
+def test_noalloc_rejects_what_does_not_fit(dev):
+    """A request whose partial sums exceed the built-in buffer fails with IXH_EWORKSPACE before anything is launched
+    (the table handed in is a real one for that chunk, so even a wrongly accepted call would run validly); the
+    atomic mode, which has no workspace, is refused too."""
+    from ixrun_amd import _lib
+    from ixrun_amd.quantize import int8x_quantize
+
+    dp = _lib.DevicePacked.from_dict(int8x_quantize(outlier_weight(2048, 2048, seed=1)), dev)
+    table = dp.prefix_build(1)
+    assert dp.gemv_workspace_bytes(1, 2) == 2 * 2048 * 2048 * 4 > LIMIT
+    x = activations(2, 2048, seed=1).to(dev)
+    y = torch.full((2, 2048), 7.0, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(_lib.IxhError) as e:
+        dp.gemv_noalloc(table, 1, x, y)
+    assert e.value.code == -4 and "built-in buffer" in str(e.value)
+    with pytest.raises(_lib.IxhError) as e:
+        dp.gemv_noalloc(table, 1, x, y, flags=_lib.IXH_GEMV_ATOMIC)
+    assert e.value.code == -1
+    torch.cuda.synchronize()
+    assert torch.all(y == 7.0)  # nothing ran
