@@ -30,8 +30,11 @@ MFMA_BF16_PEAK = 2.5e15  # FLOP/s dense bf16, MI355X published
 
 # HBM bytes per launch of the dominant kernel, from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then
 # WRITE_SIZE, KiB per dispatch, scaled by what the same counters read for the 256 MiB copy of --calibrate-copy:
-# x 2.0 and x 1.0); the counter summaries are kept under profiles/.  Workloads without a counter run report null.
-MEASURED_TRAFFIC_BYTES = {
+# x 2.0 and x 1.0); the counter summaries are kept under profiles/.  Each figure carries the hash of the kernel
+# sources it was measured on (kernel_sources_sha16) and is reported only while the sources still hash to it;
+# workloads without a counter run, or measured on other sources, report null.
+_TRAFFIC_SOURCES = "unmeasured-on-these-sources"
+MEASURED_TRAFFIC_BYTES_RAW = {
     "down_proj_5120x17408_m1_student_t": 23023.0 * 2.0 * 1024 + 16.0 * 1024,
     "down_proj_5120x17408_m1_calibrated": 33662.0 * 2.0 * 1024 + 40.0 * 1024,
     "prefill_5120x5120_m512_five_level": 50297.9 * 2.0 * 1024 + 30720.0 * 1024,
@@ -43,11 +46,14 @@ MEASURED_TRAFFIC_BYTES = {
     # all kernels of one encode step together (absmax, count, scans, clear, pack)
     "encode_5120x17408_student_t": (87053 + 87092 + 1402 + 15 + 92442) * 2.0 * 1024 + (32 + 2040 + 1362 + 32694 + 63405) * 1024,
 }
+MEASURED_TRAFFIC_BYTES = {k: (v, _TRAFFIC_SOURCES) for k, v in MEASURED_TRAFFIC_BYTES_RAW.items()}
 
 WORKLOADS = {
     # name: (out_f, in_f, m, weight recipe)
     "down_proj_5120x17408_m1_student_t": (5120, 17408, 1, "student_t"),
     "down_proj_5120x17408_m1_calibrated": (5120, 17408, 1, "calibrated"),
+    # the reference tests' own weight recipe (tests/test_fused.py:17-22): N(0, 0.005) with 4 % N(0, 0.05) outliers
+    "down_proj_5120x17408_m1_reference_recipe": (5120, 17408, 1, "outlier"),
     "down_proj_5120x17408_m1_five_level": (5120, 17408, 1, "student_t", (3, 4, 5, 6, 8)),
     "attn_proj_5120x5120_m1_five_level": (5120, 5120, 1, "student_t", (3, 4, 5, 6, 8)),
     "attn_proj_5120x5120_m1_calibrated": (5120, 5120, 1, "calibrated"),
@@ -83,10 +89,12 @@ WORKLOADS = {
 
 
 def make_weight(out_f, in_f, recipe):
-    from helpers import calibrated_weight, student_t_weight
+    from helpers import calibrated_weight, outlier_weight, student_t_weight
 
     if recipe == "student_t":
         return student_t_weight(out_f, in_f, seed=0)
+    if recipe == "outlier":
+        return outlier_weight(out_f, in_f, seed=0)
     return calibrated_weight(out_f, in_f, seed=0)[0]
 
 
@@ -103,27 +111,34 @@ def cpu_baseline(weight, x, level_bits=(3, 5, 8), rows=640):
     sub = int8x_quantize(weight[:rows].contiguous(), level_bits)
     n = sub["N"]
     xs = x[:1]
-    times = []
-    for _ in range(3):
+    xs32 = xs.float()
+    t_dec, t_mm16, t_mm32 = [], [], []
+    for rep in range(3 + 10):  # 3 warm-ups, 10 timed repetitions, medians
         t0 = time.perf_counter()
         w = decode_to_weight(sub, device="cpu")
         t1 = time.perf_counter()
         F.linear(xs, w)
         t2 = time.perf_counter()
-        times.append((t2 - t0, t1 - t0, t2 - t1))
-    total, dec, mm = sorted(times)[1]
+        F.linear(xs32, w.float())  # the fp32 variant: the bf16 weight widened, then the product
+        t3 = time.perf_counter()
+        if rep >= 3:
+            t_dec.append(t1 - t0), t_mm16.append(t2 - t1), t_mm32.append(t3 - t2)
+    dec, mm16, mm32 = float(np.median(t_dec)), float(np.median(t_mm16)), float(np.median(t_mm32))
     pn = oracle.packed_to_numpy(sub)
     xb = xs[0].contiguous().view(torch.int16).numpy().view(np.uint16)
     reps, t0 = 0, time.perf_counter()
-    while reps < 3 or time.perf_counter() - t0 < 3.0:
+    while reps < 10 or time.perf_counter() - t0 < 3.0:
         oracle.fused_gemv_f32(rows, pn["in_f"], pn["level_bits"], pn["bitmaps"], pn["streams"], pn["last"],
                               pn["scale_bits"], xb)
         reps += 1
     t_c = (time.perf_counter() - t0) / reps
     return {
-        "value": n / total / 1e9, "unit": "G weights/s", "cores": torch.get_num_threads(), "kind": "port",
-        "sample": f"first {rows} rows ({n} weights) of the same layer: torch CPU scatter decode {dec:.2f} s + "
-                  f"F.linear {mm * 1e3:.1f} ms, median of 3; host has {os.cpu_count()} logical cores",
+        "value": n / (dec + mm16) / 1e9, "unit": "G weights/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"first {rows} rows ({n} weights) of the same layer: torch CPU scatter decode {dec:.3f} s + "
+                  f"F.linear in bf16 {mm16 * 1e3:.2f} ms (in fp32: {mm32 * 1e3:.2f} ms), medians of 10 after 3 warm-ups; "
+                  f"host has {os.cpu_count()} logical cores, torch uses {torch.get_num_threads()} threads",
+        "fp32_matmul_variant_G_weights_per_s": n / (dec + mm32) / 1e9,
+        "decode_s": dec, "matmul_bf16_s": mm16, "matmul_fp32_s": mm32,
         "oracle_c_single_core_G_weights_per_s": n / t_c / 1e9,
     }
 
@@ -201,7 +216,7 @@ def bench_encode(args, dev):
                    "distinct_copies": copies},
         "us": {"scan_median": float(np.median(t_scan) * 1e3), "pack_median": float(np.median(t_pack) * 1e3)},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": alg_bytes / (ms * 1e-3) / HBM_PEAK, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "frac": alg_bytes / (ms * 1e-3) / HBM_PEAK, "traffic": measured_traffic(args.workload),
                      "note": f"algorithmic bytes = weight read once + packed output + table; the three passes move "
                              f"about {moved / 1e6:.0f} MB ({moved / (ms * 1e-3) / 1e9:.0f} GB/s)"},
         "host_wall_ms_per_step": wall_ms / steps,
@@ -285,23 +300,208 @@ def bench_decode(args, dev):
         "config": {"workload": args.workload, "out_f": out_f, "in_f": in_f, "weights": recipe,
                    "level_fractions": level_fractions, "packed_bytes": packed_bytes, "distinct_copies": copies},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": alg_bytes / (ms * 1e-3) / HBM_PEAK, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "frac": alg_bytes / (ms * 1e-3) / HBM_PEAK, "traffic": measured_traffic(args.workload),
                      "note": "algorithmic bytes = packed layer read + 2 bytes per weight written"},
         "cpu_baseline": {"value": rows * in_f / t_c / 1e9, "unit": "G weights/s", "cores": 1, "kind": "port",
                          "sample": f"first {rows} rows through the oracle's C decoder ({t_c:.2f} s)"},
     }))
 
 
+def kernel_sources_sha16():
+    """sha256 (first 16 hex digits) over the library's kernel sources: counter-derived figures are only reported
+    for the sources they were measured on."""
+    import hashlib
+
+    h = hashlib.sha256()
+    src = os.path.join(ROOT, "ixrun_amd", "csrc")
+    for name in sorted(os.listdir(src)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            h.update(open(os.path.join(src, name), "rb").read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch from the committed counter runs, or None when the kernel sources have changed since."""
+    hit = MEASURED_TRAFFIC_BYTES.get(workload)
+    if hit is None:
+        return None
+    nbytes, sha16 = hit
+    return nbytes if sha16 == kernel_sources_sha16() else None
+
+
+def build_layers(workload, dev, copies=0, unfused=False):
+    """The packed layer of a workload (CPU generator, CPU writer: the literal recipe), `copies` device copies of it
+    as StreamingLinear modules, and its activations."""
+    from ixrun_amd.engine import StreamingLinear
+    from ixrun_amd.quantize import int8x_quantize
+
+    out_f, in_f, m, recipe, *rest = WORKLOADS[workload]
+    level_bits = rest[0] if rest else (3, 5, 8)
+    weight = make_weight(out_f, in_f, recipe)
+    packed = int8x_quantize(weight, level_bits)
+    chained = workload.startswith("graph64")
+    copies = copies or (64 if chained else max(2, -(-600_000_000 // packed["total_bytes"])))
+    layers = [StreamingLinear(packed) for _ in range(copies)]
+    if unfused:
+        shared = torch.empty(packed["N"], dtype=torch.bfloat16, device=dev)
+        for sl in layers:
+            sl._gemm_ok = False
+            sl._set_shared_buf(shared)
+    g = torch.Generator("cpu").manual_seed(1)
+    x_host = torch.randn(m, in_f, generator=g).bfloat16()
+    return weight, packed, layers, x_host, chained
+
+
+def time_layers(layers, x, chained, steps_requested, warmup, min_seconds, eager=False):
+    """Time steps over the layers (round-robin; chained: each output feeds the next layer).  One pass over all
+    copies is captured as a hipGraph and replayed back to back; the timed region covers at least `steps_requested`
+    steps and at least `min_seconds` (a region of a few hundred microseconds ends before the clocks have settled
+    and reads several per cent slow).  Returns (ms per step, steps timed, graph or None, step function)."""
+    copies = len(layers)
+    state = {"h": x}
+
+    def step(i):
+        if not chained:
+            return layers[i % copies](x)
+        if i % copies == 0:
+            state["h"] = x
+        state["h"] = layers[i % copies](state["h"])  # the layer's output is the next layer's input
+        return state["h"]
+
+    for i in range(max(warmup, 1)):
+        step(i)
+    torch.cuda.synchronize()
+    graph = None
+    if not eager:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for i in range(copies):
+                step(i)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            outs = [step(i) for i in range(copies)]  # noqa: F841  (kept alive by the graph's pool)
+
+    def run(n_steps):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        if graph is not None:
+            for _ in range(n_steps // copies):
+                graph.replay()
+        else:
+            for i in range(n_steps):
+                step(i)
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop)
+
+    unit = copies if graph is not None else 1
+    steps = max(unit, -(-steps_requested // unit) * unit)
+    # warm-up the way the timed steps run (back to back, no host gaps), and a first estimate of the step time
+    probe = max(unit, -(-max(warmup, 1) // unit) * unit)
+    est_ms = run(probe) / probe
+    est_ms = min(est_ms, run(probe) / probe)
+    if est_ms * steps < min_seconds * 1e3:
+        steps = -(-int(min_seconds * 1e3 / max(est_ms, 1e-6)) // unit) * unit
+    ms = run(steps)
+    while ms < min_seconds * 1e3 * 0.999:  # the estimate was slow (clocks still rising): lengthen and time again
+        steps = -(-int(steps * 1.1 * min_seconds * 1e3 / max(ms, 1e-6)) // unit) * unit
+        ms = run(steps)
+    return ms / steps, steps, graph, step
+
+
+def also_block(dev, args):
+    """The other shapes of the hot path, each timed for a few hundred milliseconds with the headline's harness
+    (distinct packed copies beyond the last-level cache, hipGraph replay): us per layer, G weights/s and the
+    fraction of the roofline on algorithmic bytes (HBM; bf16 MFMA flops for the many-row workload)."""
+    import gc
+
+    from ixrun_amd import gemm_tuning
+    from ixrun_amd.fused import fused_gemv
+
+    # (workload that names the layer, [(reported name, activation rows, variant)])
+    plan = [
+        ("down_proj_5120x17408_m1_calibrated", [("down_proj_5120x17408_m1_calibrated", 1, "fused")]),
+        ("down_proj_5120x17408_m1_reference_recipe", [("down_proj_5120x17408_m1_reference_recipe", 1, "fused")]),
+        ("down_proj_5120x17408_m1_student_t", [("down_proj_5120x17408_m1_student_t_split_k_call", 1, "split_k"),
+                                               ("down_proj_5120x17408_m1_student_t_split_k_kernel_alone", 1, "split_k_bare")]),
+        ("attn_proj_5120x5120_m1_student_t", [("attn_proj_5120x5120_m1_student_t", 1, "fused")]),
+        ("gate_up_17408x5120_m2_student_t", [(f"gate_up_17408x5120_m{m}_student_t", m, "fused") for m in (2, 4, 8, 16)]),
+        ("graph64_5120x5120_m1_student_t", [("graph64_5120x5120_m1_student_t", 1, "fused")]),
+        ("prefill_5120x17408_m512_five_level", [("prefill_5120x17408_m512_five_level", 512, "fused"),
+                                                ("prefill_5120x17408_m512_five_level", 512, "unfused")]),
+    ]
+    out = {}
+    for key, runs in plan:
+        t0 = time.perf_counter()
+        out_f, in_f = WORKLOADS[key][:2]
+        chained = key.startswith("graph64")
+        _, packed, layers, _, _ = build_layers(key, dev)
+        for name, m, variant in runs:
+            g = torch.Generator("cpu").manual_seed(1)
+            x = torch.randn(m, in_f, generator=g).bfloat16().to(dev)
+            runners = layers
+            if variant == "unfused":  # decode to a bf16 buffer + library GEMM chosen by measurement: what the engine runs
+                shared_w = torch.empty(packed["N"], dtype=torch.bfloat16, device=dev)
+                for sl in layers:
+                    sl._gemm_ok = False
+                    sl._set_shared_buf(shared_w)
+                gemm_tuning.enable()
+            elif variant.startswith("split_k"):
+                # the reference's call of this shape (ixrun/engine.py:148-159): zero the fp32 vector, fused_gemv with
+                # chunk = in_f / 2 adds into it, cast to bf16 (three launches); "bare": the middle one alone
+                y32 = torch.zeros(out_f, dtype=torch.float32, device=dev)
+                whole = variant == "split_k"
+
+                def make(sl):
+                    def call(xin):
+                        if whole:
+                            y32.zero_()
+                        fused_gemv(xin.reshape(-1), sl._b1, sl._b2, sl._l1, sl._l2, sl._l3, sl._q1, sl._q2, sl._scale,
+                                   out_f, in_f, chunk=in_f // 2, y32=y32)
+                        return y32.to(torch.bfloat16) if whole else y32
+                    return call
+
+                runners = [make(sl) for sl in layers]
+            ms, steps, graph, step = time_layers(runners, x, chained, 0, 20, args.also_seconds)
+            r = {"us_per_layer": round(ms * 1e3, 2), "G_weights_per_s": round(out_f * in_f / (ms * 1e-3) / 1e9, 1),
+                 "steps": steps}
+            if m > 16:
+                flops = 2.0 * m * out_f * in_f
+                r["TFLOP_per_s"] = round(flops / (ms * 1e-3) / 1e12, 1)
+                r["frac_mfma"] = round(flops / (ms * 1e-3) / MFMA_BF16_PEAK, 4)
+                out.setdefault(name, {})["ixh_gemm" if variant == "fused" else "decode_plus_tuned_library_gemm"] = r
+            else:
+                alg_bytes = packed["total_bytes"] + m * in_f * 2 + m * out_f * 2
+                r["frac_hbm"] = round(alg_bytes / (ms * 1e-3) / HBM_PEAK, 4)
+                r["level_fractions"] = [round(c / packed["N"], 5) for c in packed["counts"]]
+                r["bits_per_weight"] = round(packed["bits_per_weight"], 3)
+                out[name] = r
+            del graph, step, runners
+            torch.cuda.synchronize()
+        out[runs[-1][0]]["wall_s"] = round(time.perf_counter() - t0, 1)
+        del layers
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # defaults: 0.2 s of timed work after 20 ms of warm-up; a run of a few hundred steps (10 ms) ends before the
-    # clocks have settled and reads about 8 % slower on the headline layer
+    # the timed region is never shorter than --min-seconds, whatever --steps says: a run of a few hundred steps
+    # (10 ms) ends before the clocks have settled and reads about 8 % slower on the headline layer
     ap.add_argument("--steps", type=int, default=9800)
     ap.add_argument("--warmup", type=int, default=980)
+    ap.add_argument("--min-seconds", type=float, default=0.2, help="shortest timed region (0 = exactly --steps)")
     ap.add_argument("--workload", default="down_proj_5120x17408_m1_student_t", choices=list(WORKLOADS))
     ap.add_argument("--copies", type=int, default=0, help="distinct packed copies to rotate over (0 = enough for 600 MB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-also", action="store_true", help="skip the block of other workloads timed beside the headline")
+    ap.add_argument("--also-seconds", type=float, default=0.15, help="timed region of each workload of that block")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of hipGraph replays")
     ap.add_argument("--unfused", action="store_true",
                     help="many-row workloads: decode the bf16 weight to HBM and call the library GEMM instead")
@@ -321,47 +521,21 @@ def main():
     if args.workload.startswith("decode_"):
         return bench_decode(args, dev)
 
-    from ixrun_amd.engine import StreamingLinear
-
     out_f, in_f, m, recipe, *rest = WORKLOADS[args.workload]
     level_bits = rest[0] if rest else (3, 5, 8)
+    headline = args.workload == "down_proj_5120x17408_m1_student_t"
     t0 = time.perf_counter()
-    from ixrun_amd.quantize import int8x_quantize
-
-    weight = make_weight(out_f, in_f, recipe)
-    packed = int8x_quantize(weight, level_bits)
+    weight, packed, layers, x_host, chained = build_layers(args.workload, dev, args.copies, args.unfused)
+    copies = len(layers)
     prep_s = time.perf_counter() - t0
-    chained = args.workload.startswith("graph64")
-    copies = args.copies or (64 if chained else max(2, -(-600_000_000 // packed["total_bytes"])))
-    layers = [StreamingLinear(packed) for _ in range(copies)]
     if args.tune_gemm:
         from ixrun_amd import gemm_tuning
         gemm_tuning.enable()
-    if args.unfused:
-        shared = torch.empty(packed["N"], dtype=torch.bfloat16, device=dev)
-        for sl in layers:
-            sl._gemm_ok = False
-            sl._set_shared_buf(shared)
-    g = torch.Generator("cpu").manual_seed(1)
-    x_host = torch.randn(m, in_f, generator=g).bfloat16()
     x = x_host.to(dev)
     table_bytes = layers[0]._table.numel() * 4
     # algorithmic bytes of one step: the packed layer, the activations in, the outputs out
     alg_bytes = packed["total_bytes"] + m * in_f * 2 + m * out_f * 2
 
-    state = {"h": x}
-
-    def step(i):
-        if not chained:
-            return layers[i % copies](x)
-        if i % copies == 0:
-            state["h"] = x
-        state["h"] = layers[i % copies](state["h"])  # the layer's output is the next layer's input
-        return state["h"]
-
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
     if args.calibrate_copy:
         src = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -370,40 +544,10 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # One pass over all copies is captured as a hipGraph (the per-layer launches
-    # of a decode step are replayed the same way); the timed region replays it.
-    rounds = max(1, -(-args.steps // copies))
-    steps = rounds * copies if not args.eager else args.steps
-    graph = None
-    if not args.eager:
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for i in range(copies):
-                step(i)
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            outs = [step(i) for i in range(copies)]
-        # the warm-up steps once more the way the timed steps run (back to back, no host gaps)
-        for _ in range(max(1, -(-args.warmup // copies))):
-            graph.replay()
-        torch.cuda.synchronize()
-
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t_wall = time.perf_counter()
-    start.record()
-    if graph is not None:
-        for _ in range(rounds):
-            graph.replay()
-    else:
-        for i in range(steps):
-            step(i)
-    stop.record()
-    torch.cuda.synchronize()
+    ms_per_step, steps, graph, step = time_layers(layers, x, chained, args.steps, args.warmup, args.min_seconds,
+                                                   eager=args.eager)
     wall_ms = (time.perf_counter() - t_wall) * 1e3
-    ms_per_step = start.elapsed_time(stop) / steps
 
     # eager launches with an event pair around every call, for the spread and the host cost
     n_ev = min(steps, 240)
@@ -420,7 +564,8 @@ def main():
     achieved = alg_bytes / (ms_per_step * 1e-3)
     out = {
         "metric": "fused decode+GEMV G weights/s & % HBM peak (5120x17408, batch 1); us/layer",
-        "value": weights_per_s / 1e9, "unit": "G weights/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "value": weights_per_s / 1e9, "unit": "G weights/s", "n_gpus": 1, "steps": steps,
+        "steps_requested": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "us_per_layer": us, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16 activations x int8 codes, fp32 accumulate", "data": "synthetic",
         "config": {
@@ -431,11 +576,14 @@ def main():
         },
         "roofline": {
             "bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "frac": achieved / HBM_PEAK, "traffic": measured_traffic(args.workload),
             "note": "algorithmic bytes = packed layer + x + y per launch; time = HIP-event time of the timed region / "
-                    "steps; traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script",
+                    "steps; traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script "
+                    "(null when the kernel sources have changed since those runs)",
         },
-        "launch": "eager" if graph is None else f"hipGraph of {copies} layer launches, replayed {rounds}x",
+        "launch": "eager" if graph is None else f"hipGraph of {copies} layer launches, replayed {steps // copies}x",
+        "timed_region": f"{steps} steps = {ms_per_step * steps:.1f} ms: at least --steps ({args.steps}) and at least "
+                        f"--min-seconds ({args.min_seconds} s) of back-to-back replays",
         "eager_per_call_us": {"median": float(np.median(per_call)), "min": float(per_call.min()),
                         "p90": float(np.percentile(per_call, 90))},
         "host_wall_ms_per_step": wall_ms / steps,
@@ -446,13 +594,20 @@ def main():
         out["roofline"] = {
             "bound": "mfma", "achieved": flops / (ms_per_step * 1e-3) / 1e12, "peak": MFMA_BF16_PEAK / 1e12,
             "unit": "TFLOP/s", "frac": flops / (ms_per_step * 1e-3) / MFMA_BF16_PEAK,
-            "traffic": None if args.unfused else MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic": None if args.unfused else measured_traffic(args.workload),
             "note": "2*M*N*K flops per launch pair (GEMM + slice reduce); the kernel is bound by the VALU decode "
                     "that feeds the matrix cores, not by MFMA issue",
         }
         out["path"] = "decode to HBM + library GEMM" if args.unfused else "fused decode + MFMA (ixh_gemm)"
         if args.unfused and args.tune_gemm:
             out["path"] += ", GEMM kernel chosen by measurement (torch.cuda.tunable)"
+    del graph, step, layers
+    import gc
+
+    gc.collect()
+    torch.cuda.empty_cache()
+    if headline and not args.no_also and not args.eager:
+        out["also"] = also_block(dev, args)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(weight, x_host, level_bits)
         out["cpu_baseline"]["speedup_vs_cpu"] = out["value"] / out["cpu_baseline"]["value"]
