@@ -54,6 +54,8 @@ WORKLOADS = {
     "down_proj_5120x17408_m1_calibrated": (5120, 17408, 1, "calibrated"),
     # the reference tests' own weight recipe (tests/test_fused.py:17-22): N(0, 0.005) with 4 % N(0, 0.05) outliers
     "down_proj_5120x17408_m1_reference_recipe": (5120, 17408, 1, "outlier"),
+    # no element above level 1 (but one): what the record queue and its resolution cost shows against the headline
+    "down_proj_5120x17408_m1_level1_only": (5120, 17408, 1, "level1_only"),
     "down_proj_5120x17408_m1_five_level": (5120, 17408, 1, "student_t", (3, 4, 5, 6, 8)),
     "attn_proj_5120x5120_m1_five_level": (5120, 5120, 1, "student_t", (3, 4, 5, 6, 8)),
     "attn_proj_5120x5120_m1_calibrated": (5120, 5120, 1, "calibrated"),
@@ -95,6 +97,8 @@ def make_weight(out_f, in_f, recipe):
         return student_t_weight(out_f, in_f, seed=0)
     if recipe == "outlier":
         return outlier_weight(out_f, in_f, seed=0)
+    if recipe == "level1_only":  # every value within the first level but the one +-127 that fixes the scale
+        return calibrated_weight(out_f, in_f, seed=0, fractions=(1.0, 0.0, 0.0))[0]
     return calibrated_weight(out_f, in_f, seed=0)[0]
 
 
@@ -507,6 +511,8 @@ def main():
                     help="many-row workloads: decode the bf16 weight to HBM and call the library GEMM instead")
     ap.add_argument("--tune-gemm", action="store_true",
                     help="with --unfused: let the library GEMM of the many-row path be chosen by measurement")
+    ap.add_argument("--set-option", action="append", default=[], metavar="NAME=VALUE",
+                    help="library switch for comparisons (ixh_set_option), e.g. gemv_strips=-1")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 256 MiB device copies (known traffic) so that counter runs can be scaled")
     args = ap.parse_args()
@@ -515,6 +521,11 @@ def main():
                  "run with --gpus 1")
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     dev = torch.device("cuda:0")
+    for item in args.set_option:
+        from ixrun_amd import _lib
+
+        name, _, value = item.partition("=")
+        _lib.set_option(name, int(value))
 
     if args.workload.startswith("encode_"):
         return bench_encode(args, dev)

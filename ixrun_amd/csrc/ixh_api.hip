@@ -16,6 +16,7 @@ static thread_local char g_error[512] = "";
 
 std::atomic<int> g_opt_decode_kernel{kDecodeAuto};
 std::atomic<int> g_opt_gemv_shared_x{8};
+std::atomic<int> g_opt_gemv_strips{0};
 
 void set_error(const char *fmt, ...) {
     va_list ap;
@@ -98,6 +99,11 @@ int ixh_set_option(const char *name, int64_t value) {
     if (strcmp(name, "gemv_shared_x") == 0) {
         if (value < 0 || value > 8) { set_error("gemv_shared_x %lld not in 0..8", (long long)value); return IXH_EINVAL; }
         g_opt_gemv_shared_x.store((int)value, std::memory_order_relaxed);
+        return IXH_OK;
+    }
+    if (strcmp(name, "gemv_strips") == 0) {
+        if (value < -1 || value > 6) { set_error("gemv_strips %lld not in -1..6", (long long)value); return IXH_EINVAL; }
+        g_opt_gemv_strips.store((int)value, std::memory_order_relaxed);
         return IXH_OK;
     }
     set_error("unknown option '%s'", name);
@@ -225,21 +231,28 @@ static int gemv_any(const IxhPacked *packed, const int32_t *prefix, int64_t chun
     const bool fast_any = !fast && !is_358(d) && d.n_levels >= 2 && d.bits[0] == 3 &&
                           !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED | IXH_GEMV_DENSE | IXH_GEMV_COLUMN_KERNEL)) &&
                           fast358_supports(d, (uint32_t)chunk, m) && (mostly_l1 || (flags & IXH_GEMV_FORCE_358));
-    if ((fast || fast_any) && !(flags & IXH_GEMV_COLUMN_KERNEL) && (!atomic || m <= 8)) {
-        if (m <= 8) {
-            // up to four rows: one of the row-block kernels; five to eight: the shared-x row-block kernel where the
-            // activation rows fit in LDS, else (IXH_EUNSUPPORTED) the column-block kernel below.  A workgroup owns
-            // whole rows, so the split-K contract (add into the caller's fp32 vector) costs it one addition per output.
-            rc = launch_gemv_358_rows(d, prefix, x, m, ldx, atomic ? nullptr : y, ldy, atomic ? y32 : nullptr,
-                                      (hipStream_t)stream);
-        } else {
-            // 9..16 rows: the row-block kernels eight or four rows at a time beat the column-block kernel's 16-row
-            // version (175 us on 17408 x 5120)
+    if ((fast || fast_any) && !(flags & IXH_GEMV_COLUMN_KERNEL)) {
+        // The row-block kernels: a workgroup owns whole rows, so the split-K contract (add into the caller's fp32
+        // vector) costs them one addition per output.  First the strip kernel (products on the matrix pipe, up to 16
+        // activation rows where they fit LDS beside the tables), then the kernels that multiply lane by lane: up to
+        // four rows, five to eight with the activations shared in LDS, nine to sixteen eight or four rows at a time
+        // (atomic mode excepted: a later group that does not fit must not leave an earlier one added).
+        uint16_t *const yb = atomic ? nullptr : y;
+        float *const yf = atomic ? y32 : nullptr;
+        rc = launch_gemv_358_strips(d, prefix, x, m, ldx, yb, ldy, yf, (hipStream_t)stream);
+        if (rc == IXH_EUNSUPPORTED && m <= 8)
+            rc = launch_gemv_358_rows(d, prefix, x, m, ldx, yb, ldy, yf, (hipStream_t)stream);
+        if (rc == IXH_EUNSUPPORTED && m > 8 && !atomic) {
             for (int group = 8; group >= 4 && rc == IXH_EUNSUPPORTED; group -= 4) {
                 rc = IXH_OK;
-                for (int j = 0; j < m && rc == IXH_OK; j += group)
-                    rc = launch_gemv_358_rows(d, prefix, x + (int64_t)j * ldx, m - j < group ? m - j : group, ldx,
-                                              y + (int64_t)j * ldy, ldy, nullptr, (hipStream_t)stream);
+                for (int j = 0; j < m && rc == IXH_OK; j += group) {
+                    const int mj = m - j < group ? m - j : group;
+                    rc = launch_gemv_358_strips(d, prefix, x + (int64_t)j * ldx, mj, ldx, y + (int64_t)j * ldy, ldy, nullptr,
+                                                (hipStream_t)stream);
+                    if (rc == IXH_EUNSUPPORTED)
+                        rc = launch_gemv_358_rows(d, prefix, x + (int64_t)j * ldx, mj, ldx, y + (int64_t)j * ldy, ldy,
+                                                  nullptr, (hipStream_t)stream);
+                }
             }
         }
     }

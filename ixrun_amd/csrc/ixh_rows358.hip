@@ -40,28 +40,10 @@
 
 #include <mutex>
 
-#include "ixh_fast358.h"
+#include "ixh_rows_common.h"
 
 namespace ixh {
 
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) void *lds_ptr_t;
-
-constexpr int kRStages = 3;              // unit-quads in flight per wave
-constexpr uint32_t kRStageBytes = 1280;  // 1024 stream + 256 bitmap
-constexpr uint32_t kRQueue = 128;        // records per wave
-constexpr uint32_t kRTasks = 192;        // elements above level 1 of 64 records that are spread over the lanes
-constexpr uint32_t kRSlots = 64;         // rows per workgroup at most
-constexpr int kRMaxWaves = 12;           // waves per workgroup at most: 3 per SIMD, up to 168 VGPRs each
-constexpr uint32_t kRLutBytes = 64 * 32 * 4;
-constexpr uint32_t kRSpliceBytes = 33 * 32;
-// staged share of the other streams: bitmap 1 (1 KB), 5-bit stream (2 KB), 8-bit stream (1 KB)
-constexpr uint32_t kRSideB2 = 0, kRSideL2 = 1024, kRSideL3 = 3072, kRSideBytes = 4096;
-
-constexpr uint32_t kFlagStageSide = 2u;  // the 8-bit stream is dword aligned, the side streams may be staged
-
-constexpr uint32_t kZeroCodes0 = 0xDB6DB6DBu, kZeroCodes1 = 0xB6DB6DB6u, kZeroCodes2 = 0x6DB6DB6Du;
 
 // a wave's region: ring, record queue, row sums, task list, and a copy of the activations of its own column
 // blocks (c blocks x mt rows x 512 bf16) for the elements above level 1
@@ -86,239 +68,6 @@ __host__ __device__ inline RowsLds rows_layout(uint32_t rows_cap, uint32_t n_chu
     return L;
 }
 
-__device__ __forceinline__ uint32_t dpp_shr(uint32_t v, int n) {
-    switch (n) {
-        case 1: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, true);
-        case 2: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, true);
-        case 4: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, true);
-        default: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, true);
-    }
-}
-
-__device__ __forceinline__ uint32_t row_scan(uint32_t v) {
-    v += dpp_shr(v, 1);
-    v += dpp_shr(v, 2);
-    v += dpp_shr(v, 4);
-    v += dpp_shr(v, 8);
-    return v;
-}
-
-__device__ __forceinline__ float row_sum(float v) {
-    v += __uint_as_float(dpp_shr(__float_as_uint(v), 1));
-    v += __uint_as_float(dpp_shr(__float_as_uint(v), 2));
-    v += __uint_as_float(dpp_shr(__float_as_uint(v), 4));
-    v += __uint_as_float(dpp_shr(__float_as_uint(v), 8));
-    return v;
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vmem() {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
-__device__ __forceinline__ uint32_t lds_u32(uint32_t addr) {
-    return *reinterpret_cast<const __attribute__((address_space(3))) uint32_t *>((uintptr_t)addr);
-}
-__device__ __forceinline__ uint32_t lds_u16(uint32_t addr) {
-    return *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>((uintptr_t)addr);
-}
-__device__ __forceinline__ uint32_t lds_u8(uint32_t addr) {
-    return *reinterpret_cast<const __attribute__((address_space(3))) uint8_t *>((uintptr_t)addr);
-}
-__device__ __forceinline__ u32x4 lds_u128(uint32_t addr) {
-    return *reinterpret_cast<const __attribute__((address_space(3))) u32x4 *>((uintptr_t)addr);
-}
-
-// where the elements above level 1 of this workgroup's rows live
-struct SideView {
-    bool staged;             // true: in LDS at `base`; false: read from global memory
-    uint32_t base;           // LDS address of the staged region
-    uint32_t b2w0, l2w0, l3w0;  // first staged word of bitmap 1 / 5-bit stream / 8-bit stream
-};
-
-// A store through a restrict-qualified parameter: once inlined it carries alias-scope information, which is
-// what keeps the compiler from putting "wait for every LDS-DMA copy in flight" (s_waitcnt vmcnt(0)) in front
-// of an LDS access that has nothing to do with the ring the copies land in.
-__device__ __forceinline__ void push_record(uint4 *__restrict__ q, uint32_t idx, uint4 v) { q[idx] = v; }
-
-// Two LDS operations issued outside the compiler's memory model, for the code that runs while the wave has
-// LDS-DMA copies in flight: in front of a merged two-word LDS read and of an LDS atomic the compiler puts
-// "wait for every copy" (it cannot tell that they do not touch the ring), which would stall the ring.
-__device__ __forceinline__ uint64_t lds_read2_raw(uint32_t addr) {  // words at addr and addr + 4
-    uint64_t v;
-    asm volatile("ds_read2_b32 %0, %1 offset1:1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
-    return v;
-}
-__device__ __forceinline__ void lds_add_f32_raw(uint32_t addr, float v) {  // complete after s_waitcnt lgkmcnt(0)
-    asm volatile("ds_add_f32 %0, %1" ::"v"(addr), "v"(v) : "memory");
-}
-
-// inclusive sum over the lanes at or below this one
-__device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
-    v = row_scan(v);
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1, 3
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2, 3
-    return v;
-}
-
-// Resolve queued records: every record is one bitmap word with elements above level 1.  The elements of 64
-// records are first spread over the lanes (one element per lane and round, through a task list in LDS), so
-// that the dependent reads of an element (bitmap 1, its code, x) are paid once per round and not once per
-// element of the fullest record; a batch with more than kRTasks elements is walked record by record instead.
-// STAGED: the workgroup's share of bitmap 1 and of the 5-bit / 8-bit streams is in LDS; that version reads
-// no global memory at all (the activations come from the wave's LDS copy), so nothing in it waits for the
-// copies the wave has in flight: a load from global memory returns behind all of them.
-// ANY: any scheme whose first level has 3 bits: the element is followed down the nested bitmaps (level i: rank among
-// the elements in no level below i), every rank counted from the unit's start, where the table holds it (read
-// from global memory; tq2 and the staged side streams are not used).
-// XSW: the activations are the workgroup's shared, swizzled copy of the whole x rows (xs_row bytes apart): 16-byte
-// piece p of the 64 bytes that lane l of a 16-lane row owns in a column block sits at piece p * 16 + l of the block.
-template <int MT, bool STAGED, bool ANY = false, bool XSW = false>
-__device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, uint32_t tq1_addr, uint32_t tq2_addr,
-                                             uint32_t unit0, const uint4 *__restrict__ queue, uint32_t count,
-                                             uint32_t rowacc_addr, uint16_t *__restrict__ tasks,
-                                             uint32_t xs_addr, uint32_t xs_row, uint32_t k_first,
-                                             int m, float scale, uint32_t lane,
-                                             const int32_t *__restrict__ prefix = nullptr, uint32_t entries = 0) {
-    const uint32_t *__restrict__ b2 = P.bm[1];
-    const uint32_t b2_words = P.bm_words[1];
-    // value of the element at rank r of bitmap 1's domain, unit `unit`, any scheme
-    auto value_any = [&](uint32_t unit, uint32_t r) {
-        uint32_t ru = unit * kFastChunk - lds_u32(tq1_addr + (unit - unit0) * 4);  // the unit's first rank at level i
-        for (int i = 1; i + 1 < P.n_levels; ++i) {
-            const uint32_t *__restrict__ bm = P.bm[i];
-            const uint32_t words = P.bm_words[i];
-            const uint32_t qu = (uint32_t)prefix[(size_t)i * entries + unit];  // level-i elements before the unit
-            const uint32_t wf = ru >> 5, wl = min(r >> 5, wf + 17u);
-            const uint32_t first_mask = ~0u << (ru & 31);
-            uint32_t cnt = 0;
-            for (uint32_t w = wf; w < wl; ++w) {
-                uint32_t bits = w < words ? bm[w] : 0u;
-                if (w == wf) bits &= first_mask;
-                cnt += __popc(bits);
-            }
-            const uint32_t bits = wl < words ? bm[wl] : 0u;
-            uint32_t low = (1u << (r & 31)) - 1u;
-            if (wl == wf) low &= first_mask;
-            cnt += __popc(bits & low);
-            if ((bits >> (r & 31)) & 1u) {
-                const uint32_t nb = (uint32_t)P.bits[i];
-                const uint64_t bitpos = (uint64_t)(qu + cnt) * nb;
-                const uint32_t wi = (uint32_t)(bitpos >> 5), sh = (uint32_t)bitpos & 31u;
-                const uint32_t lo = wi < P.st_words[i] ? P.st[i][wi] : 0u;
-                const uint32_t hi = (sh + nb > 32 && wi + 1 < P.st_words[i]) ? P.st[i][wi + 1] : 0u;
-                return (int)((uint32_t)((((uint64_t)hi << 32) | lo) >> sh) & ((1u << nb) - 1u)) - threshold_of((int)nb);
-            }
-            r -= qu + cnt;
-            ru -= qu;
-        }
-        return r < P.last_bytes ? (int)P.last[r] - 127 : 0;
-    };
-    // element `e` (bit of the record's word), the nth element above level 1 of its record
-    auto one = [&](const uint4 rec, uint32_t nth, uint32_t e) {
-        uint32_t r0_lane = rec.y, unit = rec.z, k0 = rec.w & 0xFFFFu;
-        const uint32_t slot = rec.w >> 16;
-        if (XSW) {  // the shared-x kernel's records: rank offset in the unit, LDS address of the unit's table
-                    // entry, column block << 4 | lane
-            const uint32_t in_unit = (rec.w & 15u) * 32u;
-            unit = unit0 + ((rec.z - tq1_addr) >> 2);
-            r0_lane = unit * kFastChunk + in_unit - (lds_u32(rec.z) + rec.y);
-            k0 = ((rec.w >> 4) & 0xFFFu) * kFastChunk + in_unit;
-        }
-        uint32_t xe[MT];  // the activations this element meets
-#pragma unroll
-        for (int j = 0; j < MT; ++j)
-            xe[j] = XSW ? lds_u16(xs_addr + (uint32_t)j * xs_row + (k0 >> 9) * (kFastChunk * 2) +
-                                  (((e >> 3) * 16u + ((k0 >> 5) & 15u)) * 16u) + (e & 7u) * 2u)
-                        : lds_u16(xs_addr + ((uint32_t)j * xs_row + k0 - k_first + e) * 2u);
-        if (ANY) {
-            const float w = dequant(value_any(unit, r0_lane + nth), scale);
-#pragma unroll
-            for (int j = 0; j < MT; ++j)
-                if (j < m) lds_add_f32_raw(rowacc_addr + (slot * MT + j) * 4, bf16_bits_to_f32(xe[j]) * w);
-            return;
-        }
-        const uint32_t r0u = unit * kFastChunk - lds_u32(tq1_addr + (unit - unit0) * 4);
-        const uint32_t q2u = lds_u32(tq2_addr + (unit - unit0) * 4);
-        const uint32_t wf = r0u >> 5;
-        const uint32_t first_mask = ~0u << (r0u & 31);
-        const uint32_t r = r0_lane + nth;
-        // level-2 elements among bitmap-1 bits [r0u, r) (a unit spans at most 17 words), and the bit at r
-        const uint32_t wl = min(r >> 5, wf + 17u);
-        uint32_t cnt = 0;
-        for (uint32_t w = wf; w < wl; ++w) {
-            uint32_t bits = STAGED ? lds_u32(sv.base + kRSideB2 + (w - sv.b2w0) * 4) : (w < b2_words ? b2[w] : 0u);
-            if (w == wf) bits &= first_mask;
-            cnt += __popc(bits);
-        }
-        const uint32_t bits = STAGED ? lds_u32(sv.base + kRSideB2 + (wl - sv.b2w0) * 4)
-                                     : (wl < b2_words ? b2[wl] : 0u);
-        uint32_t low = (1u << (r & 31)) - 1u;
-        if (wl == wf) low &= first_mask;
-        cnt += __popc(bits & low);
-        int v = 0;
-        if ((bits >> (r & 31)) & 1u) {
-            const uint64_t bitpos = (uint64_t)(q2u + cnt) * 5u;
-            const uint32_t wi = (uint32_t)(bitpos >> 5), sh = (uint32_t)bitpos & 31u;
-            uint32_t lo, hi;
-            if (STAGED) {
-                const uint64_t pair = lds_read2_raw(sv.base + kRSideL2 + (wi - sv.l2w0) * 4);
-                lo = (uint32_t)pair;
-                hi = (uint32_t)(pair >> 32);
-            } else {
-                lo = wi < P.st_words[1] ? P.st[1][wi] : 0u;
-                hi = (sh > 27 && wi + 1 < P.st_words[1]) ? P.st[1][wi + 1] : 0u;
-            }
-            v = (int)((uint32_t)((((uint64_t)hi << 32) | lo) >> sh) & 31u) - 15;
-        } else {
-            const uint32_t i3 = r - (q2u + cnt);
-            if (STAGED) v = i3 < P.last_bytes ? (int)lds_u8(sv.base + kRSideL3 + (i3 - sv.l3w0 * 4)) - 127 : 0;
-            else v = i3 < P.last_bytes ? (int)P.last[i3] - 127 : 0;
-        }
-        const float w = dequant(v, scale);
-#pragma unroll
-        for (int j = 0; j < MT; ++j)
-            if (j < m) lds_add_f32_raw(rowacc_addr + (slot * MT + j) * 4, bf16_bits_to_f32(xe[j]) * w);
-    };
-    for (uint32_t base = 0; base < count; base += kWave) {
-        const uint32_t idx = base + lane;
-        const bool has = idx < count;
-        uint4 rec = make_uint4(0, 0, 0, 0);
-        if (has) rec = queue[idx];
-        uint32_t zeros = rec.x;
-        const uint32_t mine = (uint32_t)__popc(zeros);
-        const uint32_t incl = wave_scan(mine);
-        const uint32_t n_tasks = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
-        if (n_tasks <= kRTasks) {
-            uint32_t t = incl - mine, nth = 0;
-            while (zeros != 0) {
-                tasks[t++] = (uint16_t)((lane << 10) | (nth++ << 5) | (uint32_t)__builtin_ctz(zeros));
-                zeros &= zeros - 1;
-            }
-            for (uint32_t tb = 0; tb < n_tasks; tb += kWave) {
-                if (tb + lane < n_tasks) {
-                    const uint32_t task = tasks[tb + lane];
-                    one(queue[base + (task >> 10)], (task >> 5) & 31u, task & 31u);
-                }
-            }
-        } else {
-            uint32_t nth = 0;
-            while (zeros != 0) {
-                const uint32_t e = (uint32_t)__builtin_ctz(zeros);
-                zeros &= zeros - 1;
-                one(rec, nth++, e);
-            }
-        }
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the row sums have taken the additions
-}
-
-// s_setprio takes an immediate
-__device__ __forceinline__ void set_wave_priority(uint32_t p) {
-    if (p == 0) __builtin_amdgcn_s_setprio(0);
-    else if (p == 1) __builtin_amdgcn_s_setprio(1);
-    else __builtin_amdgcn_s_setprio(2);
-}
 
 template <int MT, int C, bool ANY = false>
 __global__ void __launch_bounds__(kRMaxWaves * kWave)
@@ -933,13 +682,13 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
     auto resolve = [&]() {
         if (ANY)
-            resolve_rows<MT, false, true, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
+            resolve_rows<MT, false, true, 1>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
                                                xs_addr, xs_row, 0, m, scale, lane, prefix, entries);
         else if (sv.staged)
-            resolve_rows<MT, true, false, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
+            resolve_rows<MT, true, false, 1>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
                                                xs_addr, xs_row, 0, m, scale, lane);
         else
-            resolve_rows<MT, false, false, true>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
+            resolve_rows<MT, false, false, 1>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rowacc_addr, tasks,
                                                 xs_addr, xs_row, 0, m, scale, lane);
         qcount = 0;
     };

@@ -31,3 +31,20 @@ def force_decoder():
 
     yield force
     _lib.set_option("decode_kernel", "auto")
+
+
+@pytest.fixture
+def gemv_option():
+    """Set a kernel-selection switch of ixh_gemv for the duration of a test (``ixh_set_option``)."""
+    from ixrun_amd import _lib
+
+    defaults = {"gemv_strips": 0, "gemv_shared_x": 8}
+    touched = []
+
+    def set_(name: str, value: int) -> None:
+        touched.append(name)
+        _lib.set_option(name, value)
+
+    yield set_
+    for name in touched:
+        _lib.set_option(name, defaults[name])

@@ -291,6 +291,29 @@ def test_gemv_shared_x_kernel_lds_limits(oracle, dev, kind, shape):
 
 
 @pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("shape", [(8, 512), (64, 512), (40, 1536), (20, 17408), (68, 5120), (256, 4608), (1024, 2048), (4, 33792)])
+@pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8)])
+def test_gemv_strip_kernel(oracle, dev, gemv_option, kind, shape, level_bits):
+    """The strip kernel (every lane walks 128 weights of one row, products on the matrix pipe), forced for every
+    mix and for one and two activation rows, which it leaves to the other kernels by itself: 1..16 rows (one, two and
+    four groups of four), bf16 output and the fp32 accumulate contract, one and several tasks per DPP row, workgroups
+    with fewer tasks than DPP rows, dense mixes that overflow the shared task list."""
+    from ixrun_amd import _lib
+
+    out_f, in_f = shape
+    p = make_packed(kind, out_f, in_f, level_bits)
+    dp = device_packed(p, dev)
+    w_bits = oracle.decode_packed_bf16(p)
+    gemv_option("gemv_strips", 1)
+    for m in (1, 2, 3, 4, 5, 8, 11, 16):
+        x = activations(m, in_f, seed=m)
+        y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
+        for atomic in (False, True):
+            y = run_gemv(dp, 512, x, m, dev, flags=_lib.IXH_GEMV_FORCE_358, atomic=atomic)
+            check_outputs(y, y64, f"{kind} {shape} {level_bits} m={m} atomic={atomic}")
+
+
+@pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("shape", [(64, 512), (37, 1024), (130, 2048), (24, 8704), (5, 25600)])
 @pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8), (5, 8)])
 def test_gemv_staged(oracle, dev, kind, shape, level_bits):
@@ -353,6 +376,24 @@ def test_gemv_one_hot_is_exact(oracle, dev, kind):
         x[0, k] = 1.0
         for chunk in (512, in_f):
             assert np.array_equal(run_gemv(dp, chunk, x, 1, dev)[0], w_want[:, k]), (kind, k, chunk)
+
+
+@pytest.mark.parametrize("kind", ["student_t", "rare_other"])
+def test_gemv_strip_kernel_one_hot_is_exact(oracle, dev, gemv_option, kind):
+    """One-hot activation rows through the strip kernel: every output equals a decoded weight, exactly (the matrix
+    pipe multiplies by 1.0 and adds zeros)."""
+    out_f, in_f = 96, 1024
+    p = make_packed(kind, out_f, in_f)
+    dp = device_packed(p, dev)
+    w_want = oracle.decode_packed_bf16(p)
+    gemv_option("gemv_strips", 1)
+    cols = (0, 3, 4, 31, 32, 127, 128, 511, 512, 1023)
+    x = torch.zeros(len(cols), in_f, dtype=torch.bfloat16)
+    for i, k in enumerate(cols):
+        x[i, k] = 1.0
+    y = run_gemv(dp, 512, x, len(cols), dev)
+    for i, k in enumerate(cols):
+        assert np.array_equal(y[i], w_want[:, k]), (kind, k)
 
 
 def test_gemv_is_reproducible(oracle, dev):
