@@ -133,6 +133,7 @@ k_gemv358_strips(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, u
     const uint32_t n_workers = n_waves * 4;
     const uint32_t worker = wave * 4 + drow;
     const uint32_t wave_iters = wave * 4 < n_tasks ? (n_tasks - wave * 4 + n_workers - 1) / n_workers : 0u;
+    const bool quads_fastest = m > 4 && n_groups >= 4;
 
     // what a lane needs for one task: requested first, so that it travels while the workgroup sets up
     struct TaskIn {
@@ -148,7 +149,18 @@ k_gemv358_strips(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, u
         const uint32_t t = worker + it * n_workers;
         T.valid = t < n_tasks;
         const uint32_t tt = T.valid ? t : 0u;
-        const uint32_t g = tt / n_chunks, c = tt - g * n_chunks;
+        // Column blocks run fastest for up to four activation rows: the wave's four tasks then read neighbouring
+        // pieces of the same rows (fewer cache lines per load).  Beyond that row quads run fastest: the four tasks are
+        // four different row quads, their row sums never meet in one LDS addition, and what that saves per
+        // activation row is worth more.
+        uint32_t g, c;
+        if (quads_fastest) {
+            c = tt / n_groups;
+            g = tt - c * n_groups;
+        } else {
+            g = tt / n_chunks;
+            c = tt - g * n_chunks;
+        }
         T.col = c * kFastChunk + q * 128u;
         T.strip = c * 4u + q;
 #pragma unroll
@@ -388,20 +400,37 @@ k_gemv358_strips(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, u
             }
         }
         // The strips of a unit are four lanes apart: lanes q == 3 end up with the unit's sums and add them to the wave's
-        // row sums, one DPP row after the other (two of them may hold the same matrix row, for different column
-        // blocks: taking turns keeps the order of the additions fixed).
+        // row sums.  Where the wave's four tasks are four different row quads: one addition; otherwise two of them may
+        // hold the same matrix row (for different column blocks) and the DPP rows take turns, which keeps the order of
+        // the additions fixed.
 #pragma unroll
         for (int r = 0; r < R; ++r) {
+            float sums[MT];
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
+                sums[i] = 0.0f;
                 if (i < m) {
                     float v = acc[r][i >> 2][i & 3];
                     v += __uint_as_float(dpp_shr(__float_as_uint(v), 4));
                     v += __uint_as_float(dpp_shr(__float_as_uint(v), 8));
-                    const uint32_t at = rowacc_addr + (S.lrow[r] * (uint32_t)m + i) * 4u;
+                    sums[i] = v;
+                }
+            }
+            const uint32_t at = rowacc_addr + S.lrow[r] * (uint32_t)m * 4u;
+            if (quads_fastest) {
+                if (q == 3 && S.live[r]) {
 #pragma unroll
-                    for (uint32_t dd = 0; dd < 4; ++dd)
-                        if (q == 3 && S.live[r] && drow == dd) lds_add_f32_raw(at, v);
+                    for (int i = 0; i < MT; ++i)
+                        if (i < m) lds_add_f32_raw(at + (uint32_t)i * 4u, sums[i]);
+                }
+            } else {
+#pragma unroll
+                for (uint32_t dd = 0; dd < 4; ++dd) {
+                    if (q == 3 && S.live[r] && drow == dd) {
+#pragma unroll
+                        for (int i = 0; i < MT; ++i)
+                            if (i < m) lds_add_f32_raw(at + (uint32_t)i * 4u, sums[i]);
+                    }
                 }
             }
         }
