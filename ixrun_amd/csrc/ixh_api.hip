@@ -17,6 +17,7 @@ static thread_local char g_error[512] = "";
 std::atomic<int> g_opt_decode_kernel{kDecodeAuto};
 std::atomic<int> g_opt_gemv_shared_x{8};
 std::atomic<int> g_opt_gemv_strips{0};
+std::atomic<int> g_opt_gemv_tiles{0};
 
 void set_error(const char *fmt, ...) {
     va_list ap;
@@ -99,6 +100,11 @@ int ixh_set_option(const char *name, int64_t value) {
     if (strcmp(name, "gemv_shared_x") == 0) {
         if (value < 0 || value > 8) { set_error("gemv_shared_x %lld not in 0..8", (long long)value); return IXH_EINVAL; }
         g_opt_gemv_shared_x.store((int)value, std::memory_order_relaxed);
+        return IXH_OK;
+    }
+    if (strcmp(name, "gemv_tiles") == 0) {
+        if (value < -1 || value > 1) { set_error("gemv_tiles %lld not in -1..1", (long long)value); return IXH_EINVAL; }
+        g_opt_gemv_tiles.store((int)value, std::memory_order_relaxed);
         return IXH_OK;
     }
     if (strcmp(name, "gemv_strips") == 0) {
@@ -239,7 +245,8 @@ static int gemv_any(const IxhPacked *packed, const int32_t *prefix, int64_t chun
         // (atomic mode excepted: a later group that does not fit must not leave an earlier one added).
         uint16_t *const yb = atomic ? nullptr : y;
         float *const yf = atomic ? y32 : nullptr;
-        rc = launch_gemv_358_strips(d, prefix, x, m, ldx, yb, ldy, yf, (hipStream_t)stream);
+        rc = launch_gemv_358_tiles(d, prefix, x, m, ldx, yb, ldy, yf, (hipStream_t)stream);
+        if (rc == IXH_EUNSUPPORTED) rc = launch_gemv_358_strips(d, prefix, x, m, ldx, yb, ldy, yf, (hipStream_t)stream);
         if (rc == IXH_EUNSUPPORTED && m <= 8)
             rc = launch_gemv_358_rows(d, prefix, x, m, ldx, yb, ldy, yf, (hipStream_t)stream);
         if (rc == IXH_EUNSUPPORTED && m > 8 && !atomic) {

@@ -142,6 +142,7 @@ void set_error(const char *fmt, ...);
 enum DecodeKernel : int { kDecodeAuto = 0, kDecodeRows = 1, kDecodeDense = 2, kDecodeStaged = 3, kDecodeGeneric = 4 };
 extern std::atomic<int> g_opt_decode_kernel;   // a DecodeKernel
 extern std::atomic<int> g_opt_gemv_shared_x;   // most activation rows the shared-x row-block kernel serves (0..8)
+extern std::atomic<int> g_opt_gemv_tiles;      // the tile kernel: -1 = never, 0 = where it pays, 1 = wherever it fits
 extern std::atomic<int> g_opt_gemv_strips;     // the strip kernel: -1 = never, 0 = where it fits, 1..6 = with that many chains
 
 }  // namespace ixh

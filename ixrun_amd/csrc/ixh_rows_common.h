@@ -112,7 +112,8 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
 // XL, where the activations are: 0 = the wave's own copy of the rows of its column blocks (xs_row elements apart,
 // first column k_first); 1 = the workgroup's shared, swizzled copy of the whole x rows (xs_row bytes apart): 16-byte
 // piece p of the 64 bytes that lane l of a 16-lane row owns in a column block sits at piece p * 16 + l of the block;
-// 2 = the workgroup's shared copy in strips of 128 columns, kStripBytes apart (xs_row bytes between rows).
+// 2 = the workgroup's shared copy, from column k_first (a multiple of 128) on, in strips of 128 columns, kStripBytes
+// apart (xs_row bytes between rows).
 constexpr uint32_t kStripBytes = 264;  // 128 bf16 + 8: neighbouring strips start two LDS banks apart
 
 // POOL: the elements come from a task list that the waves of the workgroup filled together (entry = wave << 18 |
@@ -176,25 +177,32 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
             r0_lane = unit * kFastChunk + in_unit - (lds_u32(rec.z) + rec.y);
             k0 = ((rec.w >> 4) & 0xFFFu) * kFastChunk + in_unit;
         }
-        uint32_t xe[MT];  // the activations this element meets
+        // XL == 2 (up to 16 activation rows): the activations are read in a loop at the end, one register at a time
+        auto add_all = [&](float w) {
+            const uint32_t xa = xs_addr + ((k0 - k_first) >> 7) * kStripBytes + ((k0 & 127u) + e) * 2u;
+            const uint32_t ra = rowacc_addr + slot * (uint32_t)m * 4u;
+#pragma unroll 1
+            for (int j = 0; j < m; ++j)
+                lds_add_f32_raw(ra + (uint32_t)j * 4u, bf16_bits_to_f32(lds_u16(xa + (uint32_t)j * xs_row)) * w);
+        };
+        uint32_t xe[XL == 2 ? 1 : MT];  // the activations this element meets
 #pragma unroll
-        for (int j = 0; j < MT; ++j) {
+        for (int j = 0; j < (XL == 2 ? 0 : MT); ++j) {
             if (XL == 1)
                 xe[j] = lds_u16(xs_addr + (uint32_t)j * xs_row + (k0 >> 9) * (kFastChunk * 2) +
                                 (((e >> 3) * 16u + ((k0 >> 5) & 15u)) * 16u) + (e & 7u) * 2u);
-            else if (XL == 2) {
-                xe[j] = 0u;
-                if (j < m)  // m is the same for every lane: a branch, not a select
-                    xe[j] = lds_u16(xs_addr + (uint32_t)j * xs_row + (k0 >> 7) * kStripBytes + ((k0 & 127u) + e) * 2u);
-            }
             else
                 xe[j] = lds_u16(xs_addr + ((uint32_t)j * xs_row + k0 - k_first + e) * 2u);
         }
         if (ANY) {
             const float w = dequant(value_any(unit, r0_lane + nth), scale);
+            if (XL == 2) {
+                add_all(w);
+                return;
+            }
 #pragma unroll
             for (int j = 0; j < MT; ++j)
-                if (j < m) lds_add_f32_raw(rowacc_addr + (slot * (XL == 2 ? (uint32_t)m : (uint32_t)MT) + j) * 4, bf16_bits_to_f32(xe[j]) * w);
+                if (j < m) lds_add_f32_raw(rowacc_addr + (slot * MT + j) * 4, bf16_bits_to_f32(xe[j]) * w);
             return;
         }
         const uint32_t r0u = unit * kFastChunk - lds_u32(tq1_addr + (unit - unit0) * 4);
@@ -235,9 +243,13 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
             else v = i3 < P.last_bytes ? (int)P.last[i3] - 127 : 0;
         }
         const float w = dequant(v, scale);
+        if (XL == 2) {
+            add_all(w);
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < MT; ++j)
-            if (j < m) lds_add_f32_raw(rowacc_addr + (slot * (XL == 2 ? (uint32_t)m : (uint32_t)MT) + j) * 4, bf16_bits_to_f32(xe[j]) * w);
+            if (j < m) lds_add_f32_raw(rowacc_addr + (slot * MT + j) * 4, bf16_bits_to_f32(xe[j]) * w);
     };
     if (POOL) {
         for (uint32_t r = pool.first_round; r * kWave < pool.total; r += pool.round_stride) {

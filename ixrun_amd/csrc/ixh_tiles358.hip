@@ -1,0 +1,472 @@
+// (3,5,8) fused decode + skinny GEMM for gfx950, tile variant: 16 weight rows x 16 activation rows per matrix
+// instruction, so that up to 16 activation rows cost what one costs.
+//
+// Work split.  A workgroup owns whole rows.  Its rows are cut into tiles of 16; a wave belongs to one tile and to one
+// share of the column blocks for its whole life, so its 16 x 16 accumulator never leaves its registers: wave =
+// tile * n_sub + sub, and the column blocks (512 wide) of a part are dealt in runs to the n_sub waves of a tile.
+// Lane (n, kg), n = lane % 16, kg = lane / 16, decodes strip kg (128 columns) of row n of the tile, word by word, exactly
+// as in ixh_strips358.hip: bitmap words and table entry into registers, ranks from popcounts (the strips of a unit are
+// 16 lanes apart: their counts travel through ds_bpermute), 16 stream bytes per word, v_alignbit, splice, pair table.
+//
+// Products.  v_mfma_f32_16x16x32_bf16 takes eight weights of every lane (B: column n, k group kg) and eight activations
+// of every lane (A: activation row n, the same eight columns of strip kg) and adds into D[4 kg + i][n], i = 0..3:
+// four instructions per 32-column word whatever the number of activation rows.  Activation rows that do not exist
+// read a strip of zeros.
+//
+// Activations.  In LDS, in padded strips as in the strip kernel, 16 bytes of shift between rows; when all rows do not
+// fit beside the tables they are held one part of the columns at a time, and the workgroup walks the parts in turn
+// (a barrier, the next part's copy, a barrier).
+//
+// Elements above level 1 go to the wave's record queue and are resolved by the wave itself (it owns its tile) into a
+// 16-row array of its own.  At the end every wave stores its accumulators; after one barrier the outputs are summed
+// over the sub-ranges in order.  Every addition has a fixed place, apart from the order in which the LDS adds the lanes
+// of one instruction that hit the same sum.
+#include <math.h>
+
+#include "ixh_rows_common.h"
+
+namespace ixh {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kTMaxWaves = 16;
+constexpr uint32_t kTMaxRows = 128;  // rows per workgroup at most (8 tiles)
+constexpr int kTMaxM = 16;
+constexpr size_t kTLdsLimit = 160 * 1024;
+
+struct TilesLds {
+    uint32_t tq1, tq2, side, xs, xs_row, zero, partial, waves, wave_bytes, rare_off, tasks_off, total;
+};
+
+// x_blocks: column blocks of the activation rows that LDS holds at a time
+__host__ __device__ inline TilesLds tiles_layout(uint32_t rows_cap, uint32_t n_chunks, uint32_t x_blocks, uint32_t n_sub,
+                                                 uint32_t n_waves, int m, uint32_t qcap) {
+    TilesLds L;
+    const uint32_t tbl = ((rows_cap * n_chunks + 1u + 3u) & ~3u) * 4u;  // one entry past the slice: its end ranks
+    L.tq1 = kRLutBytes + kRSpliceBytes;
+    L.tq2 = L.tq1 + tbl;
+    L.side = L.tq2 + tbl;
+    L.xs = L.side + kRSideBytes;
+    // bytes between activation rows: the padded strips, then 16 bytes so that the 16 rows a b128 read takes
+    // start four banks apart
+    L.xs_row = ((x_blocks * 4u * kStripBytes + 127u) & ~127u) + 16u;
+    L.zero = L.xs + (uint32_t)m * L.xs_row;  // a strip of zeros: what the lanes of absent activation rows read
+    L.partial = (L.zero + kStripBytes + 15u) & ~15u;  // [n_sub][rows_cap][m] fp32: the waves' accumulators at the end
+    L.waves = L.partial + n_sub * rows_cap * (uint32_t)m * 4u;
+    L.rare_off = qcap * 16u;  // behind the queue: [16 rows][m] fp32 for the elements above level 1
+    L.tasks_off = L.rare_off + 16u * (uint32_t)m * 4u;
+    L.wave_bytes = (L.tasks_off + kRTasks * 2u + 15u) & ~15u;
+    L.total = L.waves + n_waves * L.wave_bytes;
+    return L;
+}
+
+template <bool ANY>
+__global__ void __launch_bounds__(kTMaxWaves * kWave)
+k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t rows_per_wg, uint32_t n_sub,
+                uint32_t x_blocks, uint32_t qcap, uint32_t flags, const uint16_t *__restrict__ x, int m, int64_t ldx,
+                uint16_t *__restrict__ y, int64_t ldy, float *__restrict__ y32) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t n_waves = blockDim.x >> 6;
+    const uint32_t n = lane & 15u, kg = lane >> 4;
+
+    const uint32_t row0 = blockIdx.x * rows_per_wg;
+    const uint32_t rows_here = min(rows_per_wg, P.out_f - row0), rows_cap = rows_per_wg;
+    const TilesLds L = tiles_layout(rows_cap, n_chunks, x_blocks, n_sub, n_waves, m, qcap);
+
+    // the pair table is addressed with (index bits | lane bits): it must sit at LDS address 0
+    if ((uint32_t)(uintptr_t)(lds_ptr_t)smem != 0) {
+        for (uint32_t t = tid; t < rows_here * (uint32_t)m; t += blockDim.x) {
+            if (y32) y32[(size_t)(t % m) * P.out_f + row0 + t / m] = __uint_as_float(0x7FC00000u);  // NaN
+            else y[(int64_t)(t % m) * ldy + row0 + t / m] = 0x7FC0;
+        }
+        return;
+    }
+    uint32_t *const lut = reinterpret_cast<uint32_t *>(smem);            // [64][32]
+    uint4 *const splice = reinterpret_cast<uint4 *>(smem + kRLutBytes);  // [33][2]
+    uint32_t *const tq1 = reinterpret_cast<uint32_t *>(smem + L.tq1);
+    uint32_t *const tq2 = reinterpret_cast<uint32_t *>(smem + L.tq2);
+    uint8_t *const wave_base = smem + L.waves + wave * L.wave_bytes;
+    uint4 *const queue = reinterpret_cast<uint4 *>(wave_base);
+    float *const rare = reinterpret_cast<float *>(wave_base + L.rare_off);
+    uint16_t *const tasks = reinterpret_cast<uint16_t *>(wave_base + L.tasks_off);
+
+    const uint32_t unit0 = row0 * n_chunks;
+    const uint32_t entries = P.out_f * n_chunks + 1;
+    const uint32_t n_local = rows_here * n_chunks;
+
+    const __amdgpu_buffer_rsrc_t b1_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[0], 0, (int)(P.bm_words[0] * 4u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t l1_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[0], 0, (int)(P.st_words[0] * 4u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t tb_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)prefix, 0, (int)(entries * 4u), 0x00020000);
+
+    // ---- this wave's tile and its share of the column blocks of a part ----
+    const uint32_t tile = wave / n_sub, sub = wave - tile * n_sub;
+    const uint32_t trow0 = tile * 16u;
+    const bool tile_live = trow0 < rows_here;                      // a wave beyond the workgroup's rows has nothing to do
+    const bool live = trow0 + n < rows_here;                       // this lane's row exists
+    const uint32_t lrow = min(trow0 + n, rows_here - 1);           // clamped: a lane without a row decodes and is dropped
+    const uint32_t n_parts = (n_chunks + x_blocks - 1) / x_blocks;
+    uint32_t part_first = 0, part_count = min(x_blocks, n_chunks);  // the part's column blocks
+    uint32_t c_begin = 0, c_end = 0;                                // this wave's run of them
+    auto take_share = [&]() {
+        const uint32_t base = part_count / n_sub, rem = part_count - base * n_sub;
+        c_begin = part_first + sub * base + min(sub, rem);
+        c_end = tile_live ? c_begin + base + (sub < rem ? 1u : 0u) : c_begin;
+    };
+    take_share();
+
+    // what a lane needs for one task (its tile x one column block): requested first, so that it travels early
+    struct TaskIn {
+        uint32_t col;    // first column of the lane's strip
+        uint32_t strip;  // strip index in the part of the activation rows in LDS
+        uint32_t q1u;    // rank table entry of the row's unit
+        u32x4 bm;        // the four bitmap words of the lane's strip
+    };
+    auto request = [&](uint32_t c, TaskIn &T) {
+        T.col = c * kFastChunk + kg * 128u;
+        T.strip = (c - part_first) * 4u + kg;
+        T.q1u = __builtin_amdgcn_raw_buffer_load_b32(tb_rsrc, (int)((unit0 + lrow * n_chunks + c) * 4u), 0, 0);
+        T.bm = __builtin_amdgcn_raw_buffer_load_b128(b1_rsrc, (int)((((row0 + lrow) * P.in_f + T.col) >> 5) * 4u), 0, 0);
+    };
+    TaskIn T;
+    if (c_begin < c_end) request(c_begin, T);
+
+    // ---- workgroup set-up: activations, table slices, side streams, pair table, splice masks ----
+    // activation rows of the part's columns into padded strips: 16-byte piece p of row i holds columns 8p .. 8p+7
+    auto load_activations = [&]() {
+        const uint32_t pieces = part_count * (kFastChunk / 8), first_piece = part_first * (kFastChunk / 8);
+        for (uint32_t t = tid; t < (uint32_t)m * pieces; t += blockDim.x) {
+            const uint32_t i = t / pieces, p = t - i * pieces;
+            const uint4 v = *reinterpret_cast<const uint4 *>(x + (int64_t)i * ldx + (first_piece + p) * 8u);
+            // strips start on multiples of 8 bytes: two 8-byte stores
+            uint2 *dst = reinterpret_cast<uint2 *>(smem + L.xs + i * L.xs_row + (p >> 4) * kStripBytes + (p & 15u) * 16u);
+            dst[0] = make_uint2(v.x, v.y);
+            dst[1] = make_uint2(v.z, v.w);
+        }
+    };
+    load_activations();
+    for (uint32_t t = tid; t < kStripBytes / 4; t += blockDim.x) reinterpret_cast<uint32_t *>(smem + L.zero)[t] = 0u;
+    for (uint32_t i = tid; i <= n_local; i += blockDim.x) {
+        tq1[i] = (uint32_t)prefix[unit0 + i];
+        if (!ANY) tq2[i] = (uint32_t)prefix[entries + unit0 + i];
+    }
+    // this workgroup's share of bitmap 1 and of the 5-bit / 8-bit streams: small when few elements are above level 1,
+    // then it is staged in LDS and resolving them touches no global memory
+    SideView sv;
+    sv.staged = false;
+    sv.base = L.side;
+    sv.b2w0 = sv.l2w0 = sv.l3w0 = 0;
+    if (!ANY) {
+        const uint32_t q1b = (uint32_t)prefix[unit0], q2b = (uint32_t)prefix[entries + unit0];
+        const uint32_t q1e = (uint32_t)prefix[unit0 + n_local], q2e = (uint32_t)prefix[entries + unit0 + n_local];
+        const uint32_t nl1b = row0 * P.in_f - q1b, nl1e = (row0 + rows_here) * P.in_f - q1e;
+        sv.b2w0 = nl1b >> 5;
+        sv.l2w0 = (uint32_t)(((uint64_t)q2b * 5u) >> 5);
+        sv.l3w0 = (nl1b - q2b) >> 2;
+        const uint32_t n_b2 = ((nl1e + 31) >> 5) - sv.b2w0;
+        const uint32_t n_l2 = (uint32_t)((((uint64_t)q2e * 5u) + 31) >> 5) - sv.l2w0;
+        const uint32_t n_l3 = ((nl1e - q2e + 3) >> 2) - sv.l3w0;
+        // one word of slack each: the resolver reads the word after a code's first word unconditionally
+        sv.staged = (flags & kFlagStageSide) && n_b2 < 256 && n_l2 < 511 && n_l3 <= 256;
+        if (sv.staged) {
+            uint32_t *side = reinterpret_cast<uint32_t *>(smem + L.side);
+            const uint32_t *last32 = reinterpret_cast<const uint32_t *>(P.last);
+            const uint32_t last_words = (P.last_bytes + 3u) >> 2;  // whole dwords (allocations are 256-byte granular)
+            for (uint32_t t = tid; t < kRSideBytes / 4; t += blockDim.x) {
+                uint32_t v = 0;
+                if (t < 256) {
+                    const uint32_t w = sv.b2w0 + t;
+                    if (w < P.bm_words[1]) v = P.bm[1][w];
+                } else if (t < 768) {
+                    const uint32_t w = sv.l2w0 + (t - 256);
+                    if (w < P.st_words[1]) v = P.st[1][w];
+                } else {
+                    const uint32_t w = sv.l3w0 + (t - 768);
+                    if (w < last_words) v = last32[w];
+                }
+                side[t] = v;
+            }
+        }
+    }
+    const float scale = bf16_bits_to_f32(*P.scale);
+    for (uint32_t i = tid; i < 64 * 32; i += blockDim.x) {
+        const int c0 = (i >> 5) & 7, c1 = i >> 8;
+        const uint32_t w0 = c0 < 7 ? f32_to_bf16_bits((float)(c0 - 3) * scale) : 0u;
+        const uint32_t w1 = c1 < 7 ? f32_to_bf16_bits((float)(c1 - 3) * scale) : 0u;
+        lut[i] = w0 | (w1 << 16);
+    }
+    if (tid <= 32) {
+        // entry e < 32: masks for a zero at element e (code bits 3e..3e+2): the bits below it, and its field;
+        // entry 32: the identity (nothing to splice)
+        const uint32_t pos = 3 * tid;
+        uint32_t lm[3], f[3];
+#pragma unroll
+        for (int dd = 0; dd < 3; ++dd) {
+            const uint32_t base = 32u * dd;
+            lm[dd] = pos <= base ? 0u : (pos >= base + 32 ? ~0u : (1u << (pos - base)) - 1u);
+            f[dd] = (pos + 3 <= base || pos >= base + 32) ? 0u : (pos >= base ? 7u << (pos - base) : 7u >> (base - pos));
+        }
+        splice[2 * tid] = make_uint4(lm[0], lm[1], lm[2], 0u);
+        splice[2 * tid + 1] = make_uint4(f[0], f[1], f[2], 0u);
+    }
+    for (uint32_t t = lane; t < 16u * (uint32_t)m; t += kWave) rare[t] = 0.0f;
+
+    const uint32_t lut_lane = (lane & 31u) << 2;
+    const uint32_t splice_addr = kRLutBytes;
+    const uint32_t tq1_addr = L.tq1, tq2_addr = L.tq2;
+    // the resolver adds into rowacc + (local row * m + activation row) * 4: the wave's 16-row array, shifted by its tile
+    const uint32_t rare_addr = (uint32_t)(uintptr_t)(lds_ptr_t)rare - trow0 * (uint32_t)m * 4u;
+    const uint32_t xs_addr = L.xs;
+    // lane n of each k group feeds activation row n (absent rows read zeros)
+    const bool x_real = n < (uint32_t)m;
+    const uint32_t x_lane = x_real ? L.xs + n * L.xs_row : L.zero;
+
+    uint32_t qcount = 0;  // wave-uniform
+    auto resolve = [&]() {
+        if (ANY)
+            resolve_rows<kTMaxM, false, true, 2>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rare_addr, tasks, xs_addr,
+                                                L.xs_row, part_first * kFastChunk, m, scale, lane, prefix, entries);
+        else if (sv.staged)
+            resolve_rows<kTMaxM, true, false, 2>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rare_addr, tasks, xs_addr,
+                                                L.xs_row, part_first * kFastChunk, m, scale, lane);
+        else
+            resolve_rows<kTMaxM, false, false, 2>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rare_addr, tasks,
+                                                 xs_addr, L.xs_row, part_first * kFastChunk, m, scale, lane);
+        qcount = 0;
+    };
+
+    auto splice_once = [&](uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &zrem) {
+        const uint32_t e = zrem != 0 ? (uint32_t)__builtin_ctz(zrem) : 32u;
+        zrem &= zrem - 1;
+        const u32x4 lm = lds_u128(splice_addr + e * 32), fm = lds_u128(splice_addr + e * 32 + 16);
+        const uint32_t s0 = w0 << 3;
+        const uint32_t s1 = __builtin_amdgcn_alignbit(w1, w0, 29);
+        const uint32_t s2 = __builtin_amdgcn_alignbit(w2, w1, 29);
+        w0 = (w0 & lm.x) | (s0 & ~lm.x);
+        w1 = (w1 & lm.y) | (s1 & ~lm.y);
+        w2 = (w2 & lm.z) | (s2 & ~lm.z);
+        w0 = (w0 & ~fm.x) | (kZeroCodes0 & fm.x);
+        w1 = (w1 & ~fm.y) | (kZeroCodes1 & fm.y);
+        w2 = (w2 & ~fm.z) | (kZeroCodes2 & fm.z);
+    };
+
+    __syncthreads();
+
+    // A task in flight: the ranks at which its words start and the stream bytes asked for with them.
+    struct Stage {
+        uint32_t word[4];  // bitmap words
+        uint32_t rank[4];  // level-1 elements before each word (global rank)
+        u32x4 code[4];     // the 16 stream bytes that hold each word's codes (address = 3 x rank)
+        uint32_t col, x_strip;
+    };
+    // second step of a task: from table entry and bitmap words to the ranks, and the requests for the codes
+    auto launch_codes = [&](const TaskIn &T, Stage &S) {
+        S.col = T.col;
+        S.x_strip = x_lane + (x_real ? T.strip * kStripBytes : 0u);
+        u32x4 b = T.bm;
+        if (!live) b = u32x4{~0u, ~0u, ~0u, ~0u};  // a lane without a row decodes what it finds and is dropped
+        S.word[0] = b.x; S.word[1] = b.y; S.word[2] = b.z; S.word[3] = b.w;
+        const uint32_t p1 = __popc(b.x), p2 = p1 + __popc(b.y), p3 = p2 + __popc(b.z), p4 = p3 + __popc(b.w);
+        // level-1 elements of the unit's strips before this one: they are 16, 32 and 48 lanes down
+        const uint32_t d1 = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((lane - 16u) * 4u), (int)p4);
+        const uint32_t d2 = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((lane - 32u) * 4u), (int)p4);
+        const uint32_t d3 = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((lane - 48u) * 4u), (int)p4);
+        const uint32_t before = (kg >= 1 ? d1 : 0u) + (kg >= 2 ? d2 : 0u) + (kg >= 3 ? d3 : 0u);
+        const uint32_t first = T.q1u + before;
+        S.rank[0] = first; S.rank[1] = first + p1; S.rank[2] = first + p2; S.rank[3] = first + p3;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            S.code[k] = __builtin_amdgcn_raw_buffer_load_b128(l1_rsrc, (int)(((S.rank[k] * 3u) >> 5) * 4u), 0, 0);
+    };
+
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};  // D[4 kg + i][n]: activation rows 4 kg .. 4 kg + 3 x this lane's weight row
+
+    // third step: decode and multiply the task's words
+    auto compute = [&](Stage &S) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const u32x4 dq = S.code[k];
+            const uint32_t rk = S.rank[k];
+            const uint32_t off = rk * 3u;  // v_alignbit takes the low five bits
+            uint32_t w0 = __builtin_amdgcn_alignbit(dq.y, dq.x, off);
+            uint32_t w1 = __builtin_amdgcn_alignbit(dq.z, dq.y, off);
+            uint32_t w2 = __builtin_amdgcn_alignbit(dq.w, dq.z, off);
+            uint32_t zrem = ~S.word[k];
+            const uint64_t any = __ballot(zrem != 0);
+            if (any != 0) {  // lanes with elements above level 1 leave a record
+                if (qcount > qcap - kWave) resolve();
+                if (zrem != 0) {
+                    const uint32_t kcol = S.col + 32u * (uint32_t)k;
+                    const uint32_t unit = unit0 + lrow * n_chunks + (S.col >> 9);
+                    const uint32_t r0 = (row0 + lrow) * P.in_f + kcol - rk;
+                    push_record(queue, qcount + lanes_below(any), make_uint4(zrem, r0, unit, (lrow << 16) | kcol));
+                }
+                qcount += (uint32_t)__popcll(any);
+                do splice_once(w0, w1, w2, zrem);
+                while (__ballot(zrem != 0) != 0);
+            }
+            // the word's activations: four steps of eight columns
+            u32x4 xa[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) xa[s] = lds_u128(S.x_strip + (uint32_t)k * 64u + (uint32_t)s * 16u);
+            // sixteen code pairs through the pair table, eight weights per matrix instruction
+            uint32_t wp[16];
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const int bit = 6 * t, ob = bit & 31, dd = bit >> 5;
+                const uint32_t lo = dd == 0 ? w0 : (dd == 1 ? w1 : w2);
+                const uint32_t hi = dd == 0 ? w1 : w2;
+                uint32_t a;  // pair index at bits 12..7
+                if (ob > 26) a = __builtin_amdgcn_alignbit(hi, lo, ob - 7);
+                else if (ob >= 7) a = lo >> (ob - 7);
+                else a = lo << (7 - ob);
+                wp[t] = lds_u32((a & 0x1F80u) | lut_lane);
+            }
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const u32x4 b4 = u32x4{wp[4 * s], wp[4 * s + 1], wp[4 * s + 2], wp[4 * s + 3]};
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[s]),
+                                                             __builtin_bit_cast(bf16x8, b4), acc, 0, 0, 0);
+            }
+        }
+    };
+
+    // Three steps per task, each one task ahead of the next: table entry + bitmap words (request), ranks and code
+    // requests (launch_codes), decode (compute).  Two stages take turns, so nothing is copied between iterations.
+    for (uint32_t part = 0;;) {
+        if (c_begin < c_end) {
+            Stage A, B;
+            launch_codes(T, A);
+            if (c_begin + 1 < c_end) request(c_begin + 1, T);
+            for (uint32_t c = c_begin; c < c_end; c += 2) {
+                if (c + 1 < c_end) {
+                    launch_codes(T, B);
+                    if (c + 2 < c_end) request(c + 2, T);
+                }
+                compute(A);
+                if (c + 1 < c_end) {
+                    if (c + 2 < c_end) {
+                        launch_codes(T, A);
+                        if (c + 3 < c_end) request(c + 3, T);
+                    }
+                    compute(B);
+                }
+            }
+        }
+        if (++part == n_parts) break;
+        // the next part of the columns: this part's elements above level 1 meet its activations while they are there
+        resolve();
+        part_first = part * x_blocks;
+        part_count = min(x_blocks, n_chunks - part_first);
+        take_share();
+        if (c_begin < c_end) request(c_begin, T);
+        __syncthreads();  // nobody reads the old part any more
+        load_activations();
+        __syncthreads();
+    }
+    resolve();
+
+    // ---- the wave's accumulators into the sub-range's slot; after the barrier the outputs are summed over the
+    // sub-ranges, each with what its wave added for the elements above level 1 ----
+    if (live) {
+        float *const partial = reinterpret_cast<float *>(smem + L.partial) + (sub * rows_cap + trow0 + n) * (uint32_t)m;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (4u * kg + i < (uint32_t)m) partial[4u * kg + i] = acc[i];
+    }
+    __syncthreads();
+    for (uint32_t t = tid; t < rows_here * (uint32_t)m; t += blockDim.x) {
+        const uint32_t slot = t / (uint32_t)m, i = t - slot * (uint32_t)m;
+        const uint32_t tl = slot >> 4;
+        float sum = 0.0f;
+        for (uint32_t s = 0; s < n_sub; ++s) {
+            sum += reinterpret_cast<const float *>(smem + L.partial)[(s * rows_cap + slot) * (uint32_t)m + i];
+            sum += reinterpret_cast<const float *>(smem + L.waves + (tl * n_sub + s) * L.wave_bytes + L.rare_off)
+                       [(slot & 15u) * (uint32_t)m + i];
+        }
+        if (y32) atomicAdd(&y32[(size_t)i * P.out_f + row0 + slot], sum);
+        else y[(int64_t)i * ldy + row0 + slot] = (uint16_t)f32_to_bf16_bits(sum);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+struct TilesPlan {
+    uint32_t rows, n_sub, x_blocks, qcap, waves;
+};
+
+// Rows per workgroup (whole rounds of one workgroup per CU, a multiple of four), waves per tile and the part of the
+// activation rows LDS holds at a time: as many waves per tile as fit (16 waves, LDS), the activations in as few parts
+// as leave room for at least two waves per tile.
+static TilesPlan plan_tiles(uint32_t out_f, uint32_t n_chunks, uint32_t n_cu, int m) {
+    const uint32_t n_quads = (out_f + 3) / 4, max_quads = kTMaxRows / 4;
+    const uint32_t rounds = (n_quads + n_cu * max_quads - 1) / (n_cu * max_quads);
+    const uint32_t rows = 4u * max(1u, min(max_quads, (n_quads + rounds * n_cu - 1) / (rounds * n_cu)));
+    const uint32_t tiles = (rows + 15) / 16;
+    for (uint32_t parts = 1; parts <= n_chunks; ++parts) {
+        const uint32_t x_blocks = (n_chunks + parts - 1) / parts;
+        if ((n_chunks + x_blocks - 1) / x_blocks != parts) continue;  // the same parts with fewer blocks each: seen
+        for (uint32_t n_sub = min((uint32_t)kTMaxWaves / tiles, x_blocks); n_sub >= 1; --n_sub) {
+            if (n_sub < 2 && x_blocks > 1 && parts < n_chunks) break;  // rather more parts than one wave per tile
+            for (uint32_t qcap : {256u, 128u}) {
+                if (tiles_layout(rows, n_chunks, x_blocks, n_sub, tiles * n_sub, m, qcap).total > kTLdsLimit) continue;
+                // no more waves than shorten the longest run of blocks
+                const uint32_t run = (x_blocks + n_sub - 1) / n_sub;
+                const uint32_t subs = (x_blocks + run - 1) / run;
+                return TilesPlan{rows, subs, x_blocks, qcap, tiles * subs};
+            }
+        }
+    }
+    return TilesPlan{0, 0, 0, 0, 0};
+}
+
+template <bool ANY>
+static int launch_tiles(const Dev &P, const int32_t *prefix, uint32_t n_chunks, const TilesPlan &plan, const uint16_t *x,
+                        int m, int64_t ldx, uint16_t *y, int64_t ldy, float *y32, hipStream_t s) {
+    static const bool raised =  // per instantiation
+        hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_tiles<ANY>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTLdsLimit) == hipSuccess;
+    if (!raised) return IXH_EUNSUPPORTED;
+    const uint32_t groups = (P.out_f + plan.rows - 1) / plan.rows;
+    const size_t lds = tiles_layout(plan.rows, n_chunks, plan.x_blocks, plan.n_sub, plan.waves, m, plan.qcap).total;
+    if (lds > kTLdsLimit) return IXH_EUNSUPPORTED;
+    uint32_t flags = 0;
+    if (((uintptr_t)P.last & 3u) == 0) flags |= kFlagStageSide;
+    hipLaunchKernelGGL((k_gemv358_tiles<ANY>), dim3(groups), dim3(plan.waves * kWave), lds, s, P, prefix, n_chunks,
+                       plan.rows, plan.n_sub, plan.x_blocks, plan.qcap, flags, x, m, ldx, y, ldy, y32);
+    return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
+}
+
+// The tile kernel: up to 16 activation rows, rows of whole 512-column blocks, row counts that are multiples of four;
+// IXH_EUNSUPPORTED sends the caller on to the other row-block kernels.
+int launch_gemv_358_tiles(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
+                          int64_t ldy, float *y32, hipStream_t s) {
+    if (m < 1 || m > kTMaxM || P.out_f % 4u != 0 || P.in_f % kFastChunk != 0 || P.in_f > 65536u) return IXH_EUNSUPPORTED;
+    if (((uintptr_t)x & 15u) != 0 || (m > 1 && (ldx & 7) != 0)) return IXH_EUNSUPPORTED;
+    const int opt = g_opt_gemv_tiles.load(std::memory_order_relaxed);  // ixh_set_option("gemv_tiles")
+    if (opt < 0) return IXH_EUNSUPPORTED;
+    const bool any = !(P.n_levels == 3 && P.bits[1] == 5);  // not (3,5,8): the resolver that walks the nested bitmaps
+    static const int n_cu = [] {
+        int dev = 0, v = 256;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
+        return v;
+    }();
+    const uint32_t n_chunks = P.in_f / kFastChunk;
+    const TilesPlan plan = plan_tiles(P.out_f, n_chunks, (uint32_t)n_cu, m);
+    if (plan.waves == 0) return IXH_EUNSUPPORTED;
+    // by itself only for more than eight activation rows (up to eight the strip kernel is faster: 17408 x 5120, M = 8:
+    // 42 us against 49 us; M = 16: 82 us in two passes against 62 us) and where most of a tile's 16 rows exist (a
+    // workgroup's rows fill its tiles to three quarters); forced (option 1) wherever it fits
+    if (opt == 0 && (m <= 8 || plan.rows * 4u < ((plan.rows + 15u) / 16u) * 16u * 3u)) return IXH_EUNSUPPORTED;
+    return any ? launch_tiles<true>(P, prefix, n_chunks, plan, x, m, ldx, y, ldy, y32, s)
+               : launch_tiles<false>(P, prefix, n_chunks, plan, x, m, ldx, y, ldy, y32, s);
+}
+
+}  // namespace ixh

@@ -293,11 +293,13 @@ def test_gemv_shared_x_kernel_lds_limits(oracle, dev, kind, shape):
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("shape", [(8, 512), (64, 512), (40, 1536), (20, 17408), (68, 5120), (256, 4608), (1024, 2048), (4, 33792)])
 @pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8)])
-def test_gemv_strip_kernel(oracle, dev, gemv_option, kind, shape, level_bits):
-    """The strip kernel (every lane walks 128 weights of one row, products on the matrix pipe), forced for every
-    mix and for one and two activation rows, which it leaves to the other kernels by itself: 1..16 rows (one, two and
-    four groups of four), bf16 output and the fp32 accumulate contract, one and several tasks per DPP row, workgroups
-    with fewer tasks than DPP rows, dense mixes that overflow the shared task list."""
+@pytest.mark.parametrize("kernel", ["strips", "tiles"])
+def test_gemv_strip_and_tile_kernels(oracle, dev, gemv_option, kind, shape, level_bits, kernel):
+    """The two kernels that take their products on the matrix pipe, each forced for every mix and every number of
+    activation rows (by themselves the strip kernel takes 3..8 rows, the tile kernel 9..16 where a workgroup's rows
+    fill its 16-row tiles): 1..16 rows, bf16 output and the fp32 accumulate contract, one and several tasks per worker,
+    workgroups with fewer tasks than workers, tiles with fewer than 16 rows, activations held in LDS one part of the
+    columns at a time (tile kernel, wide rows), dense mixes that overflow the record queues and the shared task list."""
     from ixrun_amd import _lib
 
     out_f, in_f = shape
@@ -305,12 +307,13 @@ def test_gemv_strip_kernel(oracle, dev, gemv_option, kind, shape, level_bits):
     dp = device_packed(p, dev)
     w_bits = oracle.decode_packed_bf16(p)
     gemv_option("gemv_strips", 1)
+    gemv_option("gemv_tiles", 1 if kernel == "tiles" else -1)
     for m in (1, 2, 3, 4, 5, 8, 11, 16):
         x = activations(m, in_f, seed=m)
         y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
         for atomic in (False, True):
             y = run_gemv(dp, 512, x, m, dev, flags=_lib.IXH_GEMV_FORCE_358, atomic=atomic)
-            check_outputs(y, y64, f"{kind} {shape} {level_bits} m={m} atomic={atomic}")
+            check_outputs(y, y64, f"{kernel} {kind} {shape} {level_bits} m={m} atomic={atomic}")
 
 
 @pytest.mark.parametrize("kind", KINDS)
@@ -379,15 +382,17 @@ def test_gemv_one_hot_is_exact(oracle, dev, kind):
 
 
 @pytest.mark.parametrize("kind", ["student_t", "rare_other"])
-def test_gemv_strip_kernel_one_hot_is_exact(oracle, dev, gemv_option, kind):
-    """One-hot activation rows through the strip kernel: every output equals a decoded weight, exactly (the matrix
-    pipe multiplies by 1.0 and adds zeros)."""
+@pytest.mark.parametrize("kernel", ["strips", "tiles"])
+def test_gemv_matrix_pipe_kernels_one_hot_is_exact(oracle, dev, gemv_option, kind, kernel):
+    """One-hot activation rows through the strip and the tile kernel: every output equals a decoded weight, exactly
+    (the matrix pipe multiplies by 1.0 and adds zeros)."""
     out_f, in_f = 96, 1024
     p = make_packed(kind, out_f, in_f)
     dp = device_packed(p, dev)
     w_want = oracle.decode_packed_bf16(p)
     gemv_option("gemv_strips", 1)
-    cols = (0, 3, 4, 31, 32, 127, 128, 511, 512, 1023)
+    gemv_option("gemv_tiles", 1 if kernel == "tiles" else -1)
+    cols = (0, 3, 4, 7, 8, 31, 32, 127, 128, 511, 512, 1023)
     x = torch.zeros(len(cols), in_f, dtype=torch.bfloat16)
     for i, k in enumerate(cols):
         x[i, k] = 1.0
