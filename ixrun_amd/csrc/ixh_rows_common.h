@@ -112,7 +112,7 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
 // XL, where the activations are: 0 = the wave's own copy of the rows of its column blocks (xs_row elements apart,
 // first column k_first); 1 = the workgroup's shared, swizzled copy of the whole x rows (xs_row bytes apart): 16-byte
 // piece p of the 64 bytes that lane l of a 16-lane row owns in a column block sits at piece p * 16 + l of the block;
-// 2 = the workgroup's shared copy, from column k_first (a multiple of 128) on, in strips of 128 columns, kStripBytes
+// 2 = the workgroup's shared copy, from column k_first (a multiple of 128) on, in strips of 128 columns, STRIP bytes
 // apart (xs_row bytes between rows).
 constexpr uint32_t kStripBytes = 264;  // 128 bf16 + 8: neighbouring strips start two LDS banks apart
 
@@ -124,7 +124,7 @@ struct TaskPool {
     uint32_t addr, total, first_round, round_stride, queues_addr, queue_stride;
 };
 
-template <int MT, bool STAGED, bool ANY = false, int XL = 0, bool POOL = false>
+template <int MT, bool STAGED, bool ANY = false, int XL = 0, bool POOL = false, uint32_t STRIP = kStripBytes>
 __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, uint32_t tq1_addr, uint32_t tq2_addr,
                                              uint32_t unit0, const uint4 *__restrict__ queue, uint32_t count,
                                              uint32_t rowacc_addr, uint16_t *__restrict__ tasks,
@@ -179,7 +179,7 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
         }
         // XL == 2 (up to 16 activation rows): the activations are read in a loop at the end, one register at a time
         auto add_all = [&](float w) {
-            const uint32_t xa = xs_addr + ((k0 - k_first) >> 7) * kStripBytes + ((k0 & 127u) + e) * 2u;
+            const uint32_t xa = xs_addr + ((k0 - k_first) >> 7) * STRIP + ((k0 & 127u) + e) * 2u;
             const uint32_t ra = rowacc_addr + slot * (uint32_t)m * 4u;
 #pragma unroll 1
             for (int j = 0; j < m; ++j)

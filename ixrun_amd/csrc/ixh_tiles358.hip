@@ -34,6 +34,9 @@ constexpr int kTMaxWaves = 16;
 constexpr uint32_t kTMaxRows = 128;  // rows per workgroup at most (8 tiles)
 constexpr int kTMaxM = 16;
 constexpr size_t kTLdsLimit = 160 * 1024;
+// bytes between the 128-column strips of an activation row: 16-byte reads need 16-byte aligned strips, and 272 = 68
+// dwords puts the four strips of a column block four banks apart, as the 16-byte shift between rows does for the rows
+constexpr uint32_t kTStripBytes = 272;
 
 struct TilesLds {
     uint32_t tq1, tq2, side, xs, xs_row, zero, partial, waves, wave_bytes, rare_off, tasks_off, total;
@@ -50,9 +53,9 @@ __host__ __device__ inline TilesLds tiles_layout(uint32_t rows_cap, uint32_t n_c
     L.xs = L.side + kRSideBytes;
     // bytes between activation rows: the padded strips, then 16 bytes so that the 16 rows a b128 read takes
     // start four banks apart
-    L.xs_row = ((x_blocks * 4u * kStripBytes + 127u) & ~127u) + 16u;
+    L.xs_row = ((x_blocks * 4u * kTStripBytes + 127u) & ~127u) + 16u;
     L.zero = L.xs + (uint32_t)m * L.xs_row;  // a strip of zeros: what the lanes of absent activation rows read
-    L.partial = (L.zero + kStripBytes + 15u) & ~15u;  // [n_sub][rows_cap][m] fp32: the waves' accumulators at the end
+    L.partial = (L.zero + kTStripBytes + 15u) & ~15u;  // [n_sub][rows_cap][m] fp32: the waves' accumulators at the end
     L.waves = L.partial + n_sub * rows_cap * (uint32_t)m * 4u;
     L.rare_off = qcap * 16u;  // behind the queue: [16 rows][m] fp32 for the elements above level 1
     L.tasks_off = L.rare_off + 16u * (uint32_t)m * 4u;
@@ -144,14 +147,11 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         for (uint32_t t = tid; t < (uint32_t)m * pieces; t += blockDim.x) {
             const uint32_t i = t / pieces, p = t - i * pieces;
             const uint4 v = *reinterpret_cast<const uint4 *>(x + (int64_t)i * ldx + (first_piece + p) * 8u);
-            // strips start on multiples of 8 bytes: two 8-byte stores
-            uint2 *dst = reinterpret_cast<uint2 *>(smem + L.xs + i * L.xs_row + (p >> 4) * kStripBytes + (p & 15u) * 16u);
-            dst[0] = make_uint2(v.x, v.y);
-            dst[1] = make_uint2(v.z, v.w);
+            *reinterpret_cast<uint4 *>(smem + L.xs + i * L.xs_row + (p >> 4) * kTStripBytes + (p & 15u) * 16u) = v;
         }
     };
     load_activations();
-    for (uint32_t t = tid; t < kStripBytes / 4; t += blockDim.x) reinterpret_cast<uint32_t *>(smem + L.zero)[t] = 0u;
+    for (uint32_t t = tid; t < kTStripBytes / 4; t += blockDim.x) reinterpret_cast<uint32_t *>(smem + L.zero)[t] = 0u;
     for (uint32_t i = tid; i <= n_local; i += blockDim.x) {
         tq1[i] = (uint32_t)prefix[unit0 + i];
         if (!ANY) tq2[i] = (uint32_t)prefix[entries + unit0 + i];
@@ -230,13 +230,13 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     uint32_t qcount = 0;  // wave-uniform
     auto resolve = [&]() {
         if (ANY)
-            resolve_rows<kTMaxM, false, true, 2>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rare_addr, tasks, xs_addr,
+            resolve_rows<kTMaxM, false, true, 2, false, kTStripBytes>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rare_addr, tasks, xs_addr,
                                                 L.xs_row, part_first * kFastChunk, m, scale, lane, prefix, entries);
         else if (sv.staged)
-            resolve_rows<kTMaxM, true, false, 2>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rare_addr, tasks, xs_addr,
+            resolve_rows<kTMaxM, true, false, 2, false, kTStripBytes>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rare_addr, tasks, xs_addr,
                                                 L.xs_row, part_first * kFastChunk, m, scale, lane);
         else
-            resolve_rows<kTMaxM, false, false, 2>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rare_addr, tasks,
+            resolve_rows<kTMaxM, false, false, 2, false, kTStripBytes>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rare_addr, tasks,
                                                  xs_addr, L.xs_row, part_first * kFastChunk, m, scale, lane);
         qcount = 0;
     };
@@ -268,7 +268,7 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     // second step of a task: from table entry and bitmap words to the ranks, and the requests for the codes
     auto launch_codes = [&](const TaskIn &T, Stage &S) {
         S.col = T.col;
-        S.x_strip = x_lane + (x_real ? T.strip * kStripBytes : 0u);
+        S.x_strip = x_lane + (x_real ? T.strip * kTStripBytes : 0u);
         u32x4 b = T.bm;
         if (!live) b = u32x4{~0u, ~0u, ~0u, ~0u};  // a lane without a row decodes what it finds and is dropped
         S.word[0] = b.x; S.word[1] = b.y; S.word[2] = b.z; S.word[3] = b.w;
@@ -461,10 +461,9 @@ int launch_gemv_358_tiles(const Dev &P, const int32_t *prefix, const uint16_t *x
     const uint32_t n_chunks = P.in_f / kFastChunk;
     const TilesPlan plan = plan_tiles(P.out_f, n_chunks, (uint32_t)n_cu, m);
     if (plan.waves == 0) return IXH_EUNSUPPORTED;
-    // by itself only for more than eight activation rows (up to eight the strip kernel is faster: 17408 x 5120, M = 8:
-    // 42 us against 49 us; M = 16: 82 us in two passes against 62 us) and where most of a tile's 16 rows exist (a
-    // workgroup's rows fill its tiles to three quarters); forced (option 1) wherever it fits
-    if (opt == 0 && (m <= 8 || plan.rows * 4u < ((plan.rows + 15u) / 16u) * 16u * 3u)) return IXH_EUNSUPPORTED;
+    // by itself from three activation rows on (one or two: the kernels that multiply lane by lane are as fast or faster)
+    // and where a workgroup's rows fill its tiles of 16 at least half; forced (option 1) wherever it fits
+    if (opt == 0 && (m <= 2 || plan.rows * 2u < ((plan.rows + 15u) / 16u) * 16u)) return IXH_EUNSUPPORTED;
     return any ? launch_tiles<true>(P, prefix, n_chunks, plan, x, m, ldx, y, ldy, y32, s)
                : launch_tiles<false>(P, prefix, n_chunks, plan, x, m, ldx, y, ldy, y32, s);
 }
