@@ -55,8 +55,10 @@ __host__ __device__ inline TilesLds tiles_layout(uint32_t rows_cap, uint32_t n_c
     // start four banks apart
     L.xs_row = ((x_blocks * 4u * kTStripBytes + 127u) & ~127u) + 16u;
     L.zero = L.xs + (uint32_t)m * L.xs_row;  // a strip of zeros: what the lanes of absent activation rows read
-    L.partial = (L.zero + kTStripBytes + 15u) & ~15u;  // [n_sub][rows_cap][m] fp32: the waves' accumulators at the end
-    L.waves = L.partial + n_sub * rows_cap * (uint32_t)m * 4u;
+    // [n_sub][rows_cap][m] fp32, the waves' accumulators at the end: over the activations, which nobody reads any more
+    // then (n_sub * rows_cap <= 256, so a row of them is shorter than a row of activations)
+    L.partial = L.xs;
+    L.waves = (L.zero + kTStripBytes + 15u) & ~15u;
     L.rare_off = qcap * 16u;  // behind the queue: [16 rows][m] fp32 for the elements above level 1
     L.tasks_off = L.rare_off + 16u * (uint32_t)m * 4u;
     L.wave_bytes = (L.tasks_off + kRTasks * 2u + 15u) & ~15u;
@@ -374,6 +376,7 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
     // ---- the wave's accumulators into the sub-range's slot; after the barrier the outputs are summed over the
     // sub-ranges, each with what its wave added for the elements above level 1 ----
+    __syncthreads();  // the accumulators go where the activations were
     if (live) {
         float *const partial = reinterpret_cast<float *>(smem + L.partial) + (sub * rows_cap + trow0 + n) * (uint32_t)m;
 #pragma unroll
@@ -403,28 +406,33 @@ struct TilesPlan {
 };
 
 // Rows per workgroup (whole rounds of one workgroup per CU, a multiple of four), waves per tile and the part of the
-// activation rows LDS holds at a time: as many waves per tile as fit (16 waves, LDS), the activations in as few parts
-// as leave room for at least two waves per tile.
+// activation rows LDS holds at a time.  Every part costs the workgroup two barriers and a copy, every missing wave
+// costs latency that nobody covers: the plan with the fewest parts among those with ten waves or more, else the one
+// with the most waves.
 static TilesPlan plan_tiles(uint32_t out_f, uint32_t n_chunks, uint32_t n_cu, int m) {
     const uint32_t n_quads = (out_f + 3) / 4, max_quads = kTMaxRows / 4;
     const uint32_t rounds = (n_quads + n_cu * max_quads - 1) / (n_cu * max_quads);
     const uint32_t rows = 4u * max(1u, min(max_quads, (n_quads + rounds * n_cu - 1) / (rounds * n_cu)));
     const uint32_t tiles = (rows + 15) / 16;
+    TilesPlan best{0, 0, 0, 0, 0};
     for (uint32_t parts = 1; parts <= n_chunks; ++parts) {
         const uint32_t x_blocks = (n_chunks + parts - 1) / parts;
         if ((n_chunks + x_blocks - 1) / x_blocks != parts) continue;  // the same parts with fewer blocks each: seen
-        for (uint32_t n_sub = min((uint32_t)kTMaxWaves / tiles, x_blocks); n_sub >= 1; --n_sub) {
-            if (n_sub < 2 && x_blocks > 1 && parts < n_chunks) break;  // rather more parts than one wave per tile
+        TilesPlan here{0, 0, 0, 0, 0};
+        for (uint32_t n_sub = min((uint32_t)kTMaxWaves / tiles, x_blocks); n_sub >= 1 && here.waves == 0; --n_sub) {
             for (uint32_t qcap : {256u, 128u}) {
                 if (tiles_layout(rows, n_chunks, x_blocks, n_sub, tiles * n_sub, m, qcap).total > kTLdsLimit) continue;
                 // no more waves than shorten the longest run of blocks
                 const uint32_t run = (x_blocks + n_sub - 1) / n_sub;
                 const uint32_t subs = (x_blocks + run - 1) / run;
-                return TilesPlan{rows, subs, x_blocks, qcap, tiles * subs};
+                here = TilesPlan{rows, subs, x_blocks, qcap, tiles * subs};
+                break;
             }
         }
+        if (here.waves > best.waves) best = here;
+        if (best.waves >= 10u || best.waves >= tiles * min((uint32_t)kTMaxWaves / tiles, n_chunks)) break;
     }
-    return TilesPlan{0, 0, 0, 0, 0};
+    return best;
 }
 
 template <bool ANY>
