@@ -33,20 +33,22 @@ MFMA_BF16_PEAK = 2.5e15  # FLOP/s dense bf16, MI355X published
 # x 2.0 and x 1.0); the counter summaries are kept under profiles/.  Each figure carries the hash of the kernel
 # sources it was measured on (kernel_sources_sha16) and is reported only while the sources still hash to it;
 # workloads without a counter run, or measured on other sources, report null.
-_TRAFFIC_SOURCES = "unmeasured-on-these-sources"
-MEASURED_TRAFFIC_BYTES_RAW = {
-    "down_proj_5120x17408_m1_student_t": 23023.0 * 2.0 * 1024 + 16.0 * 1024,
-    "down_proj_5120x17408_m1_calibrated": 33662.0 * 2.0 * 1024 + 40.0 * 1024,
-    "prefill_5120x5120_m512_five_level": 50297.9 * 2.0 * 1024 + 30720.0 * 1024,
-    "attn_proj_5120x5120_m1_student_t": 7118.0 * 2.0 * 1024 + 16.0 * 1024,
-    "gate_up_17408x5120_m4_student_t": 23193.0 * 2.0 * 1024 + 181.0 * 1024,
-    "decode_5120x17408_student_t": 23268.0 * 2.0 * 1024 + 179524.0 * 1024,
-    "decode_5120x17408_calibrated": 36308.0 * 2.0 * 1024 + 174080.0 * 1024,
-    "decode_gs_5120x17408_student_t": 33559.0 * 2.0 * 1024 + 174080.0 * 1024,
+_SHA_A = "eee09a2280566be3"  # kernel sources of the counter runs summarised in profiles/gemv358_rowsx_*, gemv358_tiles_*
+_SHA_OLD = "measured-on-earlier-sources"  # figures kept for the record; reported as null
+MEASURED_TRAFFIC_BYTES = {
+    "down_proj_5120x17408_m1_student_t": (23020.0 * 2.0 * 1024 + 16.0 * 1024, _SHA_A),
+    "down_proj_5120x17408_m1_calibrated": (33832.0 * 2.0 * 1024 + 40.0 * 1024, _SHA_A),
+    "attn_proj_5120x5120_m1_student_t": (7110.0 * 2.0 * 1024 + 16.0 * 1024, _SHA_A),
+    "gate_up_17408x5120_m4_student_t": (28079.0 * 2.0 * 1024 + 160.0 * 1024, _SHA_A),
+    "gate_up_17408x5120_m16_student_t": (26457.0 * 2.0 * 1024 + 640.0 * 1024, _SHA_A),
+    "prefill_5120x5120_m512_five_level": (50297.9 * 2.0 * 1024 + 30720.0 * 1024, _SHA_OLD),
+    "decode_5120x17408_student_t": (23268.0 * 2.0 * 1024 + 179524.0 * 1024, _SHA_OLD),
+    "decode_5120x17408_calibrated": (36308.0 * 2.0 * 1024 + 174080.0 * 1024, _SHA_OLD),
+    "decode_gs_5120x17408_student_t": (33559.0 * 2.0 * 1024 + 174080.0 * 1024, _SHA_OLD),
     # all kernels of one encode step together (absmax, count, scans, clear, pack)
-    "encode_5120x17408_student_t": (87053 + 87092 + 1402 + 15 + 92442) * 2.0 * 1024 + (32 + 2040 + 1362 + 32694 + 63405) * 1024,
+    "encode_5120x17408_student_t": ((87053 + 87092 + 1402 + 15 + 92442) * 2.0 * 1024 + (32 + 2040 + 1362 + 32694 + 63405) * 1024,
+                                    _SHA_OLD),
 }
-MEASURED_TRAFFIC_BYTES = {k: (v, _TRAFFIC_SOURCES) for k, v in MEASURED_TRAFFIC_BYTES_RAW.items()}
 
 WORKLOADS = {
     # name: (out_f, in_f, m, weight recipe)
@@ -512,7 +514,7 @@ def main():
     ap.add_argument("--tune-gemm", action="store_true",
                     help="with --unfused: let the library GEMM of the many-row path be chosen by measurement")
     ap.add_argument("--set-option", action="append", default=[], metavar="NAME=VALUE",
-                    help="library switch for comparisons (ixh_set_option), e.g. gemv_strips=-1")
+                    help="library switch for comparisons (ixh_set_option), e.g. gemv_tiles=-1 or decode_kernel=staged")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 256 MiB device copies (known traffic) so that counter runs can be scaled")
     args = ap.parse_args()
@@ -525,7 +527,7 @@ def main():
         from ixrun_amd import _lib
 
         name, _, value = item.partition("=")
-        _lib.set_option(name, int(value))
+        _lib.set_option(name, value if name == "decode_kernel" and not value.lstrip("-").isdigit() else int(value))
 
     if args.workload.startswith("encode_"):
         return bench_encode(args, dev)

@@ -85,9 +85,10 @@ const char *ixh_last_error(void);
  *   "gemv_shared_x"  most activation rows (0..8, default 8) that ixh_gemv gives to the row-block kernel that
  *                    shares the activations through on-chip memory; 0 = never
  *   "gemv_tiles"     the tile kernel (16 weight rows x up to 16 activation rows per matrix instruction): -1 = never,
- *                    0 = where it pays (more than eight activation rows, tiles mostly full; default), 1 = wherever it fits
- *   "gemv_strips"    the strip kernel (1..4 activation rows): -1 = never, 0 = where the shape fits it (default),
- *                    1..6 = where it fits, with that many independent chains per lane
+ *                    0 = where it pays (three activation rows or more, tiles at least half full; default),
+ *                    1 = wherever it fits
+ *   "gemv_strips"    the strip kernel (up to eight activation rows a pass): -1 = never, 0 = for three rows or more
+ *                    where the tile kernel does not run and the shape fits (default), 1..6 = wherever it fits
  * Returns IXH_EINVAL for an unknown name or a value out of range.  Calls already running are not affected.
  */
 int ixh_set_option(const char *name, int64_t value);
