@@ -466,12 +466,33 @@ def gate_up_layer(oracle, dev):
 @pytest.mark.parametrize("m", [2, 4, 8, 16])
 def test_full_size_config4_every_batch(oracle, dev, gate_up_layer, m):
     """BASELINE config 4 as stated: 17408 x 5120 with M in {2, 4, 8, 16} activation rows, each through the kernel the
-    library picks for it (2 and 4 rows: 16 waves; 8 rows: the eight-wave variant; 16 rows: more than one launch)."""
+    library picks for it (2 rows: the row-block kernel; 4, 8 and 16 rows: the tile kernel, at 16 rows with the
+    activations in two column parts)."""
     sl, w_bits = gate_up_layer
     x = activations(m, 5120, seed=1)
     y = sl(x.to(dev))
     assert y.shape == (m, 17408)
     check_outputs(bf16_bits(y), oracle.gemm_f64(w_bits, bf16_bits(x)), f"config 4 m={m}")
+
+
+@pytest.fixture(scope="module")
+def down_proj_layer(oracle, dev):
+    """The headline layer, 5120 x 17408 Student-t, packed once for several batch sizes."""
+    from ixrun_amd.engine import StreamingLinear
+
+    p = quantize(student_t_weight(5120, 17408, seed=0))
+    return StreamingLinear(p), oracle.decode_packed_bf16(p)
+
+
+@pytest.mark.parametrize("m", [3, 8, 12, 16])
+def test_full_size_down_proj_many_rows(oracle, dev, down_proj_layer, m):
+    """5120 x 17408 with 3..16 activation rows: 20 rows per workgroup (one tile of 16 and a quarter of one) and
+    activation rows that LDS holds two to six column parts at a time."""
+    sl, w_bits = down_proj_layer
+    x = activations(m, 17408, seed=m)
+    y = sl(x.to(dev))
+    assert y.shape == (m, 5120)
+    check_outputs(bf16_bits(y), oracle.gemm_f64(w_bits, bf16_bits(x)), f"5120x17408 m={m}")
 
 
 def test_full_size_split_k_contract(oracle, dev):
