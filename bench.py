@@ -33,21 +33,25 @@ MFMA_BF16_PEAK = 2.5e15  # FLOP/s dense bf16, MI355X published
 # x 2.0 and x 1.0); the counter summaries are kept under profiles/.  Each figure carries the hash of the kernel
 # sources it was measured on (kernel_sources_sha16) and is reported only while the sources still hash to it;
 # workloads without a counter run, or measured on other sources, report null.
-_SHA_A = "eee09a2280566be3"  # kernel sources of the counter runs summarised in profiles/gemv358_rowsx_*, gemv358_tiles_*
-_SHA_OLD = "measured-on-earlier-sources"  # figures kept for the record; reported as null
+# (bytes per launch, the sources the kernel is compiled from, their kernel_sources_sha16 at the counter run)
+_ROWS = ("ixh_rows358.hip", "ixh_rows_common.h", "ixh_dev.h")
+_TILES = ("ixh_tiles358.hip", "ixh_rows_common.h", "ixh_dev.h")
+_DENSE = ("ixh_dense358.hip", "ixh_dev.h")
+_DENSE5 = ("ixh_dense5.hip", "ixh_dev.h")
+_OLD = ((), "measured-on-earlier-sources")  # figures kept for the record; reported as null
 MEASURED_TRAFFIC_BYTES = {
-    "down_proj_5120x17408_m1_student_t": (23020.0 * 2.0 * 1024 + 16.0 * 1024, _SHA_A),
-    "down_proj_5120x17408_m1_calibrated": (33832.0 * 2.0 * 1024 + 40.0 * 1024, _SHA_A),
-    "attn_proj_5120x5120_m1_student_t": (7110.0 * 2.0 * 1024 + 16.0 * 1024, _SHA_A),
-    "gate_up_17408x5120_m4_student_t": (28079.0 * 2.0 * 1024 + 160.0 * 1024, _SHA_A),
-    "gate_up_17408x5120_m16_student_t": (26457.0 * 2.0 * 1024 + 640.0 * 1024, _SHA_A),
-    "prefill_5120x5120_m512_five_level": (50297.9 * 2.0 * 1024 + 30720.0 * 1024, _SHA_OLD),
-    "decode_5120x17408_student_t": (23268.0 * 2.0 * 1024 + 179524.0 * 1024, _SHA_OLD),
-    "decode_5120x17408_calibrated": (36308.0 * 2.0 * 1024 + 174080.0 * 1024, _SHA_OLD),
-    "decode_gs_5120x17408_student_t": (33559.0 * 2.0 * 1024 + 174080.0 * 1024, _SHA_OLD),
+    "down_proj_5120x17408_m1_student_t": (23020.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "bdc69284735fd9fa"),
+    "attn_proj_5120x5120_m1_student_t": (7110.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "bdc69284735fd9fa"),
+    "down_proj_5120x17408_m1_calibrated": (33832.0 * 2.0 * 1024 + 40.0 * 1024, _DENSE, "4c194d30b116b40a"),
+    "down_proj_5120x17408_m1_five_level_calibrated": (49706.0 * 2.0 * 1024 + 1334.0 * 1024, _DENSE5, "7cf97245e07e3bf5"),
+    "gate_up_17408x5120_m4_student_t": (28079.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "3ceb514690dd072e"),
+    "gate_up_17408x5120_m16_student_t": (26457.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "3ceb514690dd072e"),
+    "prefill_5120x5120_m512_five_level": (50297.9 * 2.0 * 1024 + 30720.0 * 1024,) + _OLD,
+    "decode_5120x17408_student_t": (23268.0 * 2.0 * 1024 + 179524.0 * 1024,) + _OLD,
+    "decode_5120x17408_calibrated": (36308.0 * 2.0 * 1024 + 174080.0 * 1024,) + _OLD,
+    "decode_gs_5120x17408_student_t": (33559.0 * 2.0 * 1024 + 174080.0 * 1024,) + _OLD,
     # all kernels of one encode step together (absmax, count, scans, clear, pack)
-    "encode_5120x17408_student_t": ((87053 + 87092 + 1402 + 15 + 92442) * 2.0 * 1024 + (32 + 2040 + 1362 + 32694 + 63405) * 1024,
-                                    _SHA_OLD),
+    "encode_5120x17408_student_t": ((87053 + 87092 + 1402 + 15 + 92442) * 2.0 * 1024 + (32 + 2040 + 1362 + 32694 + 63405) * 1024,) + _OLD,
 }
 
 WORKLOADS = {
@@ -59,6 +63,8 @@ WORKLOADS = {
     # no element above level 1 (but one): what the record queue and its resolution cost shows against the headline
     "down_proj_5120x17408_m1_level1_only": (5120, 17408, 1, "level1_only"),
     "down_proj_5120x17408_m1_five_level": (5120, 17408, 1, "student_t", (3, 4, 5, 6, 8)),
+    # the fraction-calibrated weights in the five-level scheme: every level populated
+    "down_proj_5120x17408_m1_five_level_calibrated": (5120, 17408, 1, "calibrated", (3, 4, 5, 6, 8)),
     "attn_proj_5120x5120_m1_five_level": (5120, 5120, 1, "student_t", (3, 4, 5, 6, 8)),
     "attn_proj_5120x5120_m1_calibrated": (5120, 5120, 1, "calibrated"),
     "graph64_5120x5120_m1_calibrated": (5120, 5120, 1, "calibrated"),
@@ -313,27 +319,27 @@ def bench_decode(args, dev):
     }))
 
 
-def kernel_sources_sha16():
-    """sha256 (first 16 hex digits) over the library's kernel sources: counter-derived figures are only reported
-    for the sources they were measured on."""
+def kernel_sources_sha16(files=None):
+    """sha256 (first 16 hex digits) over kernel sources of the library (all of them, or the named ones):
+    counter-derived figures are only reported for the sources they were measured on."""
     import hashlib
 
     h = hashlib.sha256()
     src = os.path.join(ROOT, "ixrun_amd", "csrc")
-    for name in sorted(os.listdir(src)):
-        if name.endswith((".hip", ".h")):
-            h.update(name.encode())
-            h.update(open(os.path.join(src, name), "rb").read())
+    names = sorted(files) if files is not None else sorted(n for n in os.listdir(src) if n.endswith((".hip", ".h")))
+    for name in names:
+        h.update(name.encode())
+        h.update(open(os.path.join(src, name), "rb").read())
     return h.hexdigest()[:16]
 
 
 def measured_traffic(workload):
-    """HBM bytes per launch from the committed counter runs, or None when the kernel sources have changed since."""
+    """HBM bytes per launch from the committed counter runs, or None when the kernel's sources have changed since."""
     hit = MEASURED_TRAFFIC_BYTES.get(workload)
     if hit is None:
         return None
-    nbytes, sha16 = hit
-    return nbytes if sha16 == kernel_sources_sha16() else None
+    nbytes, files, sha16 = hit
+    return nbytes if files and sha16 == kernel_sources_sha16(files) else None
 
 
 def build_layers(workload, dev, copies=0, unfused=False):

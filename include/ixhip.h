@@ -41,7 +41,7 @@ extern "C" {
 #define IXH_GEMV_COLUMN_KERNEL 4u /* of the (3,5,8) kernels, take the column-block one with the workspace */
 #define IXH_GEMV_FORCE_358 8u /* use the (3,5,8) kernels even when less than 97 % of the elements are level 1 */
 #define IXH_GEMV_STAGED 16u /* skip the (3,5,8) kernels: the any-scheme kernel that stages the streams in LDS */
-#define IXH_GEMV_DENSE 32u /* (3,5,8), M <= 8: the level-by-level kernels even when almost all elements are level 1 */
+#define IXH_GEMV_DENSE 32u /* (3,5,8) with M <= 8, (3,4,5,6,8) with M = 1: the level-by-level kernels even when almost all elements are level 1 */
 
 typedef void *ixh_stream_t; /* a hipStream_t */
 

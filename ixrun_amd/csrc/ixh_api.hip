@@ -270,6 +270,10 @@ static int gemv_any(const IxhPacked *packed, const int32_t *prefix, int64_t chun
         (!mostly_l1 || (flags & IXH_GEMV_DENSE)) && gemv_dense358_supports(d, (uint32_t)chunk, m, x))
         // (3,5,8), one activation row, many elements above level 1: level-by-level products over compacted x
         rc = launch_gemv_dense358(d, prefix, x, y, y32, (float *)workspace, atomic, (hipStream_t)stream);
+    if (rc == IXH_EUNSUPPORTED && !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED)) &&
+        (!mostly_l1 || (flags & IXH_GEMV_DENSE)) && gemv_dense34568_supports(d, (uint32_t)chunk, m, x))
+        // the same for the five-level scheme (3,4,5,6,8)
+        rc = launch_gemv_dense34568(d, prefix, x, y, y32, (float *)workspace, atomic, (hipStream_t)stream);
     if (rc == IXH_EUNSUPPORTED && !atomic && !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED)) &&
         (!mostly_l1 || (flags & IXH_GEMV_DENSE)) && gemv_dense358_rows_supports(d, (uint32_t)chunk, m, x, ldx))
         // (3,5,8), 2..8 activation rows, many elements above level 1: weights gathered to position order per span

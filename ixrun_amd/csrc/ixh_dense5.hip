@@ -1,0 +1,396 @@
+// (3,4,5,6,8) fused decode + GEMV for one activation row when the levels above the first are well populated (the
+// reference's five-level scheme on real weights: about 5.3 bits per weight): the level-by-level method of
+// ixh_dense358.hip with five levels.
+//
+//     sum_k w_k x_k = sum over the levels of (sum_{k in level} w_k x_k)
+// The codes of a level are dense in their stream, so each level's sum is taken over whole codes at fixed positions,
+// and what depends on the bitmaps is moved to the activations: the x values of a span are scattered into five arrays
+// in LDS, one per level, in the order of that level's codes.
+//
+// A wave takes spans of up to 2048 consecutive elements of one weight row (four 512-element table units).  The rank
+// table gives the span's first code in every stream and its level counts.  Lane l owns word l of the first bitmap (32
+// elements, 16 x pairs in registers).  The nested bitmaps of the span (at most 2048 bits each) are copied to LDS from
+// addresses that follow from the table alone; a lane's window into each of them starts at its number of elements that
+// no earlier level claimed, which comes from one wave prefix sum per level.  The scatter walks two elements per step
+// (t and t + 16) with all running slots and bitmap cursors in packed 16-bit halves.  The dense passes split each
+// level's codes evenly over the 64 lanes (a multiple of four per lane), read them through buffer descriptors, and
+// meet the compacted x pairs in v_dot2_f32_bf16: level 1 through the table of dequantised pairs, the others as
+// fma(code, scale, -T * scale), exact in fp32, rounded to bf16 as the reference's decoder does
+// (ixrun/triton_kernels.py:168-177).  Every array is padded with zeros up to 64 x codes-per-lane.
+#include "ixh_fast358.h"
+
+namespace ixh {
+
+typedef uint32_t e_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t e_u32x3 __attribute__((ext_vector_type(3)));
+typedef uint32_t e_u32x2 __attribute__((ext_vector_type(2)));
+typedef uint16_t e_u16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 e_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float e_f32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kD5Waves = 4;                       // waves per workgroup
+constexpr uint32_t kD5Span = 2048;                // elements per span: four table units of one row
+constexpr uint32_t kD5Slots = kD5Span + 5 * 256;  // compacted x slots per wave: five arrays, each padded to 64 * E
+constexpr uint32_t kD5BmWords = 68;               // staged words of a nested bitmap: 2048 bits from any bit of a word on
+constexpr uint32_t kD5LutBytes = 64 * 32 * 4;     // pair table: 64 code pairs x 32 lane copies
+
+enum : int { kD5Direct = 0, kD5Atomic = 1, kD5Workspace = 2 };
+
+#define IXH_D5_DPP_ADD(v, ctrl, row_mask, bound) \
+    v += __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), ctrl, row_mask, 0xf, bound))
+// sum over the wave, valid in lane 63
+__device__ __forceinline__ float d5_wave_sum(float v) {
+    IXH_D5_DPP_ADD(v, 0x111, 0xf, true);
+    IXH_D5_DPP_ADD(v, 0x112, 0xf, true);
+    IXH_D5_DPP_ADD(v, 0x114, 0xf, true);
+    IXH_D5_DPP_ADD(v, 0x118, 0xf, true);
+    IXH_D5_DPP_ADD(v, 0x142, 0xa, false);
+    IXH_D5_DPP_ADD(v, 0x143, 0xc, false);
+    return v;
+}
+#undef IXH_D5_DPP_ADD
+
+__device__ __forceinline__ uint32_t d5_pack(float lo, float hi) {
+    const e_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, e_bf16x2));
+}
+
+__device__ __forceinline__ float d5_dot2(uint32_t w, uint32_t x, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(e_bf16x2, w), __builtin_bit_cast(e_bf16x2, x), acc, false);
+}
+
+// the low `n` bits set (n = 0 .. 32)
+__device__ __forceinline__ uint32_t d5_low_mask(uint32_t n) { return (uint32_t)(0xFFFFFFFFull >> (32u - n)); }
+
+// A lane's window of a code stream: B + 1 dwords from the dword that holds code `first` on, shifted so that the code
+// starts at bit 0 of w[0].  A dword past the stream's end reads as zero.
+template <int B>
+__device__ __forceinline__ void d5_window(__amdgpu_buffer_rsrc_t rsrc, uint64_t first_bit, uint32_t (&w)[B]) {
+    const uint32_t at = (uint32_t)(first_bit >> 5) * 4u, sh = (uint32_t)first_bit & 31u;
+    uint32_t d[B + 1];
+#pragma unroll
+    for (int j = 0; j + 4 <= B + 1; j += 4) {
+        const e_u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(at + 4u * j), 0, 0);
+        d[j] = v[0]; d[j + 1] = v[1]; d[j + 2] = v[2]; d[j + 3] = v[3];
+    }
+    constexpr int done = ((B + 1) / 4) * 4, rest = B + 1 - done;
+    if constexpr (rest == 1) {
+        d[done] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(at + 4u * done), 0, 0);
+    } else if constexpr (rest == 2) {
+        const e_u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)(at + 4u * done), 0, 0);
+        d[done] = v[0]; d[done + 1] = v[1];
+    } else if constexpr (rest == 3) {
+        const e_u32x3 v = __builtin_amdgcn_raw_buffer_load_b96(rsrc, (int)(at + 4u * done), 0, 0);
+        d[done] = v[0]; d[done + 1] = v[1]; d[done + 2] = v[2];
+    }
+#pragma unroll
+    for (int j = 0; j < B; ++j) w[j] = __builtin_amdgcn_alignbit(d[j + 1], d[j], sh);
+}
+
+// code t (a compile-time index) of a window of B-bit codes
+template <int B>
+__device__ __forceinline__ uint32_t d5_code(const uint32_t (&w)[B], int t) {
+    const int bit = B * t, ob = bit & 31, d = bit >> 5;
+    constexpr uint32_t mask = (1u << B) - 1u;
+    if (ob + B <= 32) return (w[d] >> ob) & mask;
+    return __builtin_amdgcn_alignbit(d + 1 < B ? w[d + 1] : 0u, w[d], ob) & mask;
+}
+
+// one level's dense pass: e codes of this lane (a multiple of four, at most 32) against its row of compacted x pairs.
+// Groups of two pairs; a group is entered only if the level has codes for it (the empty asm statements keep the
+// group tests branches: as selects, all eight groups would run for every span).
+template <int B>
+__device__ __forceinline__ float d5_pass(const uint32_t (&w)[B], const uint32_t *xp, uint32_t e, float scale,
+                                         float minus_t_scale, float acc) {
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+        if (e > 4u * g) {
+            asm volatile("");
+#pragma unroll
+            for (int t = 2 * g; t < 2 * g + 2; ++t) {
+                // (c - T) * scale as c * scale - T * scale: both products and their difference are exact in fp32
+                // (codes and T have at most 8 significant bits, the bf16 scale 8): nothing is rounded twice
+                const uint32_t c0 = d5_code<B>(w, 2 * t), c1 = d5_code<B>(w, 2 * t + 1);
+                const uint32_t wp = d5_pack(__fmaf_rn((float)c0, scale, minus_t_scale), __fmaf_rn((float)c1, scale, minus_t_scale));
+                acc = d5_dot2(wp, xp[t], acc);
+            }
+        }
+    }
+    return acc;
+}
+
+__global__ void __launch_bounds__(kWave *kD5Waves)
+k_gemv34568_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t spans_per_row, uint32_t n_spans,
+                  const uint16_t *__restrict__ x, uint16_t *__restrict__ y, float *__restrict__ y32,
+                  float *__restrict__ ws, int out_mode, bool by_rows) {
+    __shared__ __attribute__((aligned(16))) uint32_t lut[kD5LutBytes / 4];
+    __shared__ __attribute__((aligned(16))) uint16_t xc_all[kD5Waves][kD5Slots];
+    __shared__ uint32_t bm_all[kD5Waves][3][kD5BmWords];
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const float scale = bf16_bits_to_f32(*P.scale);
+    const float m7 = -7.0f * scale, m15 = -15.0f * scale, m31 = -31.0f * scale, m127 = -127.0f * scale;  // exact
+
+    // pair table: entry (c0 | c1 << 3) = the two dequantised level-1 weights, one copy per bank
+    for (uint32_t e = tid; e < 64 * 32; e += kWave * kD5Waves) {
+        const uint32_t idx = e >> 5;
+        lut[e] = d5_pack(dequant((int)(idx & 7u) - 3, scale), dequant((int)(idx >> 3) - 3, scale));
+    }
+    __syncthreads();
+
+    uint16_t *const xc = xc_all[wave];
+    uint32_t(*const bmw)[kD5BmWords] = bm_all[wave];
+    const uint32_t lut_lane = (lane & 31u) << 2;
+    const uint32_t entries = P.out_f * n_chunks + 1;
+    const uint32_t *__restrict__ b1 = P.bm[0];
+    const __amdgpu_buffer_rsrc_t st_rsrc[4] = {
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[0], 0, (int)(P.st_words[0] * 4u), 0x00020000),
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[1], 0, (int)(P.st_words[1] * 4u), 0x00020000),
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[2], 0, (int)(P.st_words[2] * 4u), 0x00020000),
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[3], 0, (int)(P.st_words[3] * 4u), 0x00020000)};
+    // whole dwords of the byte stream (device allocations are 256-byte granular, the last dword is there to read)
+    const __amdgpu_buffer_rsrc_t last_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.last, 0, (int)((P.last_bytes + 3u) & ~3u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t bm_rsrc[3] = {
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[1], 0, (int)(P.bm_words[1] * 4u), 0x00020000),
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[2], 0, (int)(P.bm_words[2] * 4u), 0x00020000),
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[3], 0, (int)(P.bm_words[3] * 4u), 0x00020000)};
+
+    // Work is dealt to the waves of the launch in turn; the launch is resident as a whole.  An item is a whole row (its
+    // spans are summed in the wave and the result leaves as it is) or, when rows would not spread evenly, one span
+    // (partial sums meet in the workspace).
+    const uint32_t n_waves = gridDim.x * kD5Waves;
+    const uint32_t n_items = by_rows ? P.out_f : n_spans;
+    for (uint32_t item = blockIdx.x * kD5Waves + wave; item < n_items; item += n_waves) {
+      const uint32_t row = by_rows ? item : item / spans_per_row;
+      const uint32_t k_first = by_rows ? 0u : item - row * spans_per_row;
+      const uint32_t k_end = by_rows ? spans_per_row : k_first + 1u;
+      float row_total = 0.0f;  // meaningful in lane 63
+      for (uint32_t k = k_first; k < k_end; ++k) {
+        {   // the waves that share a SIMD take turns at the issue priority, one span each
+            const uint32_t turn = (wave + k) % 3u;  // s_setprio takes an immediate
+            if (turn == 0) __builtin_amdgcn_s_setprio(0);
+            else if (turn == 1) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(2);
+        }
+        const uint32_t c0 = 4 * k, nb = min(4u, n_chunks - c0);
+        const uint32_t u0 = row * n_chunks + c0;
+        const uint32_t n_el = nb * kFastChunk, p0 = u0 * kFastChunk;
+        // codes of each level before the span, and in it
+        uint32_t qa[4], cnt[5];
+        {
+            uint32_t rest = n_el;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                qa[i] = (uint32_t)prefix[(size_t)i * entries + u0];
+                cnt[i] = (uint32_t)prefix[(size_t)i * entries + u0 + nb] - qa[i];
+                rest -= cnt[i];
+            }
+            cnt[4] = rest;
+        }
+        // codes per lane in the dense passes (a multiple of four), and where each level's compacted array starts
+        uint32_t e[5], base[5];
+        {
+            uint32_t at = 0;
+#pragma unroll
+            for (int i = 0; i < 5; ++i) {
+                e[i] = 4 * ((cnt[i] + 255) / 256);
+                base[i] = at;
+                at += 64 * e[i];
+            }
+        }
+        // first bit of the span in each nested bitmap's domain: its elements that no earlier level claimed
+        const uint32_t g1 = p0 - qa[0], g2 = g1 - qa[1], g3 = g2 - qa[2], at_last = g3 - qa[3];
+
+        // ---- loads whose addresses follow from the table alone ----
+        const bool valid = 32 * lane < n_el;
+        const uint32_t w1 = valid ? b1[(p0 >> 5) + lane] : 0u;
+        uint32_t xr[16];
+        if (valid) {
+            const uint4 *xp = reinterpret_cast<const uint4 *>(x + c0 * kFastChunk + 32 * lane);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint4 v = xp[t];
+                xr[4 * t] = v.x; xr[4 * t + 1] = v.y; xr[4 * t + 2] = v.z; xr[4 * t + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 16; ++t) xr[t] = 0u;
+        }
+        // the span's part of the nested bitmaps: 65 words each from the word that holds its first bit
+        {
+            const uint32_t gs[3] = {g1, g2, g3};
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                const uint32_t w0 = gs[j] >> 5;
+                bmw[j][lane] = __builtin_amdgcn_raw_buffer_load_b32(bm_rsrc[j], (int)((w0 + lane) * 4u), 0, 0);
+                if (lane < 4) bmw[j][64 + lane] = __builtin_amdgcn_raw_buffer_load_b32(bm_rsrc[j], (int)((w0 + 64u + lane) * 4u), 0, 0);
+            }
+        }
+        // The code streams, read through buffer descriptors: a dword past a stream's end reads as zero, so no lane
+        // needs a bounds test; lanes whose share lies past the level's last code read codes of the next span, which
+        // then meet the zero pads of the compacted arrays.
+        uint32_t c1w[3], c2w[4], c3w[5], c4w[6], c5w[8];
+        d5_window<3>(st_rsrc[0], (uint64_t)(qa[0] + lane * e[0]) * 3u, c1w);
+        d5_window<4>(st_rsrc[1], (uint64_t)(qa[1] + lane * e[1]) * 4u, c2w);
+        d5_window<5>(st_rsrc[2], (uint64_t)(qa[2] + lane * e[2]) * 5u, c3w);
+        d5_window<6>(st_rsrc[3], (uint64_t)(qa[3] + lane * e[3]) * 6u, c4w);
+        d5_window<8>(last_rsrc, (uint64_t)(at_last + lane * e[4]) * 8u, c5w);
+
+        // ---- clear the compacted arrays (the pads must read as zero) ----
+        for (uint32_t j = lane; j < kD5Slots / 8; j += kWave) reinterpret_cast<e_u32x4 *>(xc)[j] = e_u32x4{0, 0, 0, 0};
+
+        // ---- ranks: first slot of this lane in each array ----
+        // a lane's window into nested bitmap j starts at the span's first bit there plus the elements of the lanes
+        // below that no earlier level claimed
+        auto window = [&](int j, uint32_t g, uint32_t first, uint32_t alive) {
+            const uint32_t o = (g & 31u) + first;
+            const uint32_t lo = bmw[j][o >> 5], hi = bmw[j][(o >> 5) + 1];
+            return __builtin_amdgcn_alignbit(hi, lo, o & 31u) & d5_low_mask(alive);
+        };
+        const uint32_t cnt1 = (uint32_t)__popc(w1);
+        const uint32_t alive1 = valid ? 32u - cnt1 : 0u;
+        const uint32_t sc1 = wave_scan_inclusive(cnt1 | (alive1 << 16));
+        const uint32_t first1 = (sc1 & 0xffffu) - cnt1, first_a1 = (sc1 >> 16) - alive1;
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const uint32_t bits2 = window(0, g1, first_a1, alive1);  // bit j: the lane's j-th element above level 1 is level 2
+        const uint32_t cnt2 = (uint32_t)__popc(bits2), alive2 = alive1 - cnt2;
+        const uint32_t sc2 = wave_scan_inclusive(cnt2 | (alive2 << 16));
+        const uint32_t first2 = (sc2 & 0xffffu) - cnt2, first_a2 = (sc2 >> 16) - alive2;
+        const uint32_t bits3 = window(1, g2, first_a2, alive2);
+        const uint32_t cnt3 = (uint32_t)__popc(bits3), alive3 = alive2 - cnt3;
+        const uint32_t sc3 = wave_scan_inclusive(cnt3 | (alive3 << 16));
+        const uint32_t first3 = (sc3 & 0xffffu) - cnt3, first_a3 = (sc3 >> 16) - alive3;
+        const uint32_t bits4 = window(2, g3, first_a3, alive3);
+        const uint32_t cnt4 = (uint32_t)__popc(bits4);
+        const uint32_t first4 = wave_scan_inclusive(cnt4) - cnt4;
+        const uint32_t first5 = first_a3 - first4;
+
+        // ---- scatter the lane's 32 activations to their levels' arrays ----
+        // Two elements per step, t and t + 16, with their counters in the two halves of one register (packed 16-bit
+        // arithmetic): each half holds "LDS byte address / 2" of the next slot of its level.  The second half starts
+        // where the first one will end: behind the level counts of the lane's first 16 elements.  in1 .. in5 are 0 or
+        // 1 per half; the slot is picked by multiply-add.  ja, jb, jc count the elements that levels 1, 1..2 and 1..3
+        // have passed on: the cursors into the three nested windows.
+        {
+            const uint32_t xc_half = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)xc >> 1;
+            const uint32_t low1 = (uint32_t)__popc(w1 & 0xffffu);  // level-1 elements among the first 16
+            const uint32_t low_a1 = valid ? 16u - low1 : 0u;          // elements above level 1 among them
+            const uint32_t low2 = (uint32_t)__popc(bits2 & d5_low_mask(low_a1)), low_a2 = low_a1 - low2;
+            const uint32_t low3 = (uint32_t)__popc(bits3 & d5_low_mask(low_a2)), low_a3 = low_a2 - low3;
+            const uint32_t low4 = (uint32_t)__popc(bits4 & d5_low_mask(low_a3)), low5 = low_a3 - low4;
+            const uint32_t a1 = xc_half + base[0] + first1, a2 = xc_half + base[1] + first2, a3 = xc_half + base[2] + first3;
+            const uint32_t a4 = xc_half + base[3] + first4, a5 = xc_half + base[4] + first5;
+            e_u16x2 s1 = __builtin_bit_cast(e_u16x2, a1 | ((a1 + low1) << 16));
+            e_u16x2 s2 = __builtin_bit_cast(e_u16x2, a2 | ((a2 + low2) << 16));
+            e_u16x2 s3 = __builtin_bit_cast(e_u16x2, a3 | ((a3 + low3) << 16));
+            e_u16x2 s4 = __builtin_bit_cast(e_u16x2, a4 | ((a4 + low4) << 16));
+            e_u16x2 s5 = __builtin_bit_cast(e_u16x2, a5 | ((a5 + low5) << 16));
+            // the flags each half walks through: from bit 0, and from where the first 16 elements will have got to
+            // (a 64-bit shift: 32 is a legal count when no element of the first half gets that far)
+            const e_u16x2 f2 = __builtin_bit_cast(e_u16x2, (bits2 & 0xffffu) | ((uint32_t)((uint64_t)bits2 >> low_a1) << 16));
+            const e_u16x2 f3 = __builtin_bit_cast(e_u16x2, (bits3 & 0xffffu) | ((uint32_t)((uint64_t)bits3 >> low_a2) << 16));
+            const e_u16x2 f4 = __builtin_bit_cast(e_u16x2, (bits4 & 0xffffu) | ((uint32_t)((uint64_t)bits4 >> low_a3) << 16));
+            e_u16x2 ja = {0, 0}, jb = {0, 0}, jc = {0, 0};
+            const e_u16x2 one = {1, 1};
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const e_u16x2 in1 = __builtin_bit_cast(e_u16x2, (w1 >> t) & 0x00010001u);
+                const e_u16x2 out1 = in1 ^ one;
+                const e_u16x2 in2 = (f2 >> ja) & out1;
+                const e_u16x2 out2 = out1 ^ in2;
+                const e_u16x2 in3 = (f3 >> jb) & out2;
+                const e_u16x2 out3 = out2 ^ in3;
+                const e_u16x2 in4 = (f4 >> jc) & out3;
+                const e_u16x2 in5 = out3 ^ in4;
+                const e_u16x2 at = in1 * (s1 - s5) + (in2 * (s2 - s5) + (in3 * (s3 - s5) + (in4 * (s4 - s5) + s5)));
+                const uint32_t at32 = __builtin_bit_cast(uint32_t, at);
+                const uint32_t x_lo = xr[t >> 1], x_hi = xr[8 + (t >> 1)];
+                // lanes past the span scatter zeros behind the last array's entries
+                *reinterpret_cast<__attribute__((address_space(3))) uint16_t *>((uintptr_t)((at32 & 0xffffu) << 1)) =
+                    (uint16_t)((t & 1) ? x_lo >> 16 : x_lo);
+                *reinterpret_cast<__attribute__((address_space(3))) uint16_t *>((uintptr_t)((at32 >> 16) << 1)) =
+                    (uint16_t)((t & 1) ? x_hi >> 16 : x_hi);
+                s1 += in1; s2 += in2; s3 += in3; s4 += in4; s5 += in5;
+                ja += out1; jb += out2; jc += out3;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+
+        // ---- dense passes ----
+        float acc = 0.0f;
+        {   // level 1: pairs of 3-bit codes through the pair table
+            const uint32_t *xp = reinterpret_cast<const uint32_t *>(xc) + (lane * e[0]) / 2;
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                if (e[0] > 4u * g) {
+                    asm volatile("");
+#pragma unroll
+                    for (int t = 2 * g; t < 2 * g + 2; ++t) {
+                        const int bit = 6 * t, ob = bit & 31, d = bit >> 5;
+                        const uint32_t lo = c1w[d];
+                        const uint32_t hi = d < 2 ? c1w[d + 1] : 0u;
+                        uint32_t a;  // pair index at bits 12..7
+                        if (ob > 26) a = __builtin_amdgcn_alignbit(hi, lo, ob - 7);
+                        else if (ob >= 7) a = lo >> (ob - 7);
+                        else a = lo << (7 - ob);
+                        const uint32_t wp = lut[((a & 0x1F80u) | lut_lane) >> 2];
+                        acc = d5_dot2(wp, xp[t], acc);
+                    }
+                }
+            }
+        }
+        acc = d5_pass<4>(c2w, reinterpret_cast<const uint32_t *>(xc) + (base[1] + lane * e[1]) / 2, e[1], scale, m7, acc);
+        acc = d5_pass<5>(c3w, reinterpret_cast<const uint32_t *>(xc) + (base[2] + lane * e[2]) / 2, e[2], scale, m15, acc);
+        acc = d5_pass<6>(c4w, reinterpret_cast<const uint32_t *>(xc) + (base[3] + lane * e[3]) / 2, e[3], scale, m31, acc);
+        acc = d5_pass<8>(c5w, reinterpret_cast<const uint32_t *>(xc) + (base[4] + lane * e[4]) / 2, e[4], scale, m127, acc);
+        row_total += d5_wave_sum(acc);
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      }
+      if (lane == 63) {
+          if (out_mode == kD5Direct) y[row] = (uint16_t)f32_to_bf16_bits(row_total);
+          else if (out_mode == kD5Atomic) atomicAdd(y32 + row, row_total);
+          else ws[(size_t)k_first * P.out_f + row] = row_total;
+      }
+    }
+}
+
+bool gemv_dense34568_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x) {
+    return P.n_levels == 5 && P.bits[0] == 3 && P.bits[1] == 4 && P.bits[2] == 5 && P.bits[3] == 6 && P.bits[4] == 8 &&
+           chunk == kFastChunk && m == 1 && P.in_f % kFastChunk == 0 && P.in_f != 0 && ((uintptr_t)x & 15u) == 0 &&
+           ((uintptr_t)P.last & 3u) == 0;
+}
+
+int launch_gemv_dense34568(const Dev &P, const int32_t *prefix, const uint16_t *x, uint16_t *y, float *y32, float *ws,
+                           bool atomic, hipStream_t s) {
+    const uint32_t n_chunks = P.in_f / kFastChunk;
+    const uint32_t spans_per_row = (n_chunks + 3) / 4;
+    const uint32_t n_spans = P.out_f * spans_per_row;
+    if (n_spans == 0) return IXH_OK;
+    // one resident set of workgroups; each wave walks its items with the stride of the launch
+    static const uint32_t resident = [] {
+        int dev = 0, n_cu = 256, per_cu = 0;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv34568_dense, kWave * kD5Waves, 0) != hipSuccess || per_cu < 1)
+            per_cu = 3;
+        return (uint32_t)n_cu * (uint32_t)per_cu;
+    }();
+    // Whole rows per wave when they spread over the resident waves within 12 %: one launch, no workspace, each
+    // output summed in one register.  Otherwise spans are dealt out and a second kernel adds a row's partial sums.
+    const uint32_t waves_res = resident * kD5Waves;
+    const uint32_t rounds = (P.out_f + waves_res - 1) / waves_res;
+    const bool by_rows = spans_per_row == 1 || (uint64_t)rounds * waves_res * 100u <= (uint64_t)P.out_f * 112u;
+    const uint32_t n_items = by_rows ? P.out_f : n_spans;
+    const uint32_t blocks = min(resident, (n_items + kD5Waves - 1) / kD5Waves);
+    const int out_mode = atomic ? kD5Atomic : (by_rows ? kD5Direct : kD5Workspace);
+    hipLaunchKernelGGL(k_gemv34568_dense, dim3(blocks), dim3(kWave * kD5Waves), 0, s, P, prefix, n_chunks, spans_per_row,
+                       n_spans, x, y, y32, ws, out_mode, by_rows);
+    if (hipGetLastError() != hipSuccess) return IXH_ELAUNCH;
+    if (out_mode == kD5Workspace) return launch_reduce_chunks(ws, spans_per_row, 1, P.out_f, y, P.out_f, s);
+    return IXH_OK;
+}
+
+}  // namespace ixh

@@ -26,6 +26,10 @@ int launch_gemv_358_tiles(const Dev &P, const int32_t *prefix, const uint16_t *x
 bool gemv_dense358_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x);
 int launch_gemv_dense358(const Dev &P, const int32_t *prefix, const uint16_t *x, uint16_t *y, float *y32, float *ws,
                          bool atomic, hipStream_t s);
+// the same for the five-level scheme (3,4,5,6,8), one activation row (ixh_dense5.hip)
+bool gemv_dense34568_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x);
+int launch_gemv_dense34568(const Dev &P, const int32_t *prefix, const uint16_t *x, uint16_t *y, float *y32, float *ws,
+                           bool atomic, hipStream_t s);
 bool gemv_dense358_rows_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x, int64_t ldx);
 int launch_gemv_dense358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
                               int64_t ldy, float *ws, hipStream_t s);

@@ -102,4 +102,11 @@ def int8_mix(kind: str, n: int, seed: int = 0) -> np.ndarray:
         v[hit] = (np.where(rng.random(hit.sum()) < 0.7, rng.integers(4, 16, size=hit.sum()),
                            rng.integers(16, 128, size=hit.sum())) * sign[hit])
         return v.astype(np.int8)
+    if kind == "five_dense":  # every level of (3,4,5,6,8) well populated: 40 / 25 / 20 / 10 / 5 %
+        u = rng.random(n)
+        mag = np.where(u < 0.40, rng.integers(0, 4, size=n),
+              np.where(u < 0.65, rng.integers(4, 8, size=n),
+              np.where(u < 0.85, rng.integers(8, 16, size=n),
+              np.where(u < 0.95, rng.integers(16, 32, size=n), rng.integers(32, 128, size=n)))))
+        return (mag * sign).astype(np.int8)
     raise KeyError(kind)

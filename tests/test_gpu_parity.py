@@ -336,6 +336,24 @@ def test_gemv_staged(oracle, dev, kind, shape, level_bits):
             check_outputs(y, y64, f"{kind} {shape} {level_bits} m={m} atomic={atomic}")
 
 
+@pytest.mark.parametrize("kind", KINDS + ["five_dense"])
+@pytest.mark.parametrize("shape", [(64, 512), (37, 1024), (130, 2048), (300, 1536), (24, 8704), (5, 25600)])
+def test_gemv_five_level_dense_kernel(oracle, dev, kind, shape):
+    """The level-by-level kernel of the five-level scheme (3,4,5,6,8), one activation row: what the library picks for
+    dense mixes, forced for the others; whole rows per wave and spans through the workspace, and the split-K call."""
+    from ixrun_amd import _lib
+
+    out_f, in_f = shape
+    p = make_packed(kind, out_f, in_f, (3, 4, 5, 6, 8))
+    dp = device_packed(p, dev)
+    x = activations(1, in_f, seed=3)
+    y64 = oracle.gemm_f64(oracle.decode_packed_bf16(p), bf16_bits(x))
+    for flags in (0, _lib.IXH_GEMV_DENSE):
+        for atomic in (False, True):
+            y = run_gemv(dp, 512, x, 1, dev, flags=flags, atomic=atomic)
+            check_outputs(y, y64, f"{kind} {shape} five-level flags={flags} atomic={atomic}")
+
+
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("shape", [(64, 512), (37, 1024), (130, 1536), (24, 8704), (9, 25600)])
 @pytest.mark.parametrize("level_bits", [(3, 4, 5, 6, 8), (3, 8), (3, 3, 8), (3, 5, 6, 7, 8)])
