@@ -438,6 +438,7 @@ def also_block(dev, args):
     plan = [
         ("down_proj_5120x17408_m1_calibrated", [("down_proj_5120x17408_m1_calibrated", 1, "fused")]),
         ("down_proj_5120x17408_m1_reference_recipe", [("down_proj_5120x17408_m1_reference_recipe", 1, "fused")]),
+        ("down_proj_5120x17408_m1_five_level_calibrated", [("down_proj_5120x17408_m1_five_level_calibrated", 1, "fused")]),
         ("down_proj_5120x17408_m1_student_t", [("down_proj_5120x17408_m1_student_t_split_k_call", 1, "split_k"),
                                                ("down_proj_5120x17408_m1_student_t_split_k_kernel_alone", 1, "split_k_bare")]),
         ("attn_proj_5120x5120_m1_student_t", [("attn_proj_5120x5120_m1_student_t", 1, "fused")]),
