@@ -43,9 +43,10 @@ MEASURED_TRAFFIC_BYTES = {
     "down_proj_5120x17408_m1_student_t": (23020.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "bdc69284735fd9fa"),
     "attn_proj_5120x5120_m1_student_t": (7110.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "bdc69284735fd9fa"),
     "down_proj_5120x17408_m1_calibrated": (33832.0 * 2.0 * 1024 + 40.0 * 1024, _DENSE, "4c194d30b116b40a"),
-    "down_proj_5120x17408_m1_five_level_calibrated": (49706.0 * 2.0 * 1024 + 1334.0 * 1024, _DENSE5, "7cf97245e07e3bf5"),
+    "down_proj_5120x17408_m1_five_level_calibrated": (49711.0 * 2.0 * 1024 + 1338.0 * 1024, _DENSE5, "25b0f9e2ddc3a686"),
     "gate_up_17408x5120_m4_student_t": (28079.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "3ceb514690dd072e"),
     "gate_up_17408x5120_m16_student_t": (26457.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "3ceb514690dd072e"),
+    "decode_5120x17408_five_level_calibrated": (48964.0 * 2.0 * 1024 + 174080.0 * 1024, _DENSE5, "25b0f9e2ddc3a686"),
     "prefill_5120x5120_m512_five_level": (50297.9 * 2.0 * 1024 + 30720.0 * 1024,) + _OLD,
     "decode_5120x17408_student_t": (23268.0 * 2.0 * 1024 + 179524.0 * 1024,) + _OLD,
     "decode_5120x17408_calibrated": (36308.0 * 2.0 * 1024 + 174080.0 * 1024,) + _OLD,
@@ -94,6 +95,7 @@ WORKLOADS = {
     # full decode to bf16 in HBM (m is unused): the per-tensor format and the group-scale sibling format
     "decode_5120x17408_student_t": (5120, 17408, 0, "student_t"),
     "decode_5120x17408_calibrated": (5120, 17408, 0, "calibrated"),
+    "decode_5120x17408_five_level_calibrated": (5120, 17408, 0, "calibrated", (3, 4, 5, 6, 8)),
     "decode_gs_5120x17408_student_t": (5120, 17408, 0, "student_t"),
 }
 
@@ -261,7 +263,8 @@ def bench_decode(args, dev):
     else:
         from ixrun_amd.quantize import int8x_quantize
 
-        packed = int8x_quantize(weight, (3, 5, 8))
+        level_bits = tuple(rest[0]) if rest else (3, 5, 8)
+        packed = int8x_quantize(weight, level_bits)
         packed_bytes = packed["total_bytes"]
         mk = lambda: (_lib.DevicePacked.from_dict(packed, dev), None)
     copies = args.copies or max(2, -(-600_000_000 // packed_bytes))
@@ -300,7 +303,7 @@ def bench_decode(args, dev):
     else:
         from ixrun_amd.quantize import int8x_quantize
 
-        sub = int8x_quantize(weight[:rows].contiguous(), (3, 5, 8))
+        sub = int8x_quantize(weight[:rows].contiguous(), level_bits)
         t0 = time.perf_counter()
         oracle.decode_packed_bf16(sub)
         t_c = time.perf_counter() - t0

@@ -154,6 +154,9 @@ static int decode_any(const IxhPacked *packed, const int32_t *prefix, int64_t ch
     else if (allowed(kDecodeDense) && (forced || !mostly_l1) && decode_dense358_supports(d, (uint32_t)chunk, out_i8, out_bf16, gs))
         // (3,5,8) with many elements above level 1: the level-by-level decoder (ixh_dense358.hip)
         rc = launch_decode_dense358(d, prefix, out_bf16, gs, (hipStream_t)stream);
+    else if (allowed(kDecodeDense) && (forced || !mostly_l1) && !gs.fp16 && decode_dense34568_supports(d, (uint32_t)chunk, out_i8, out_bf16))
+        // the same for the five-level scheme (3,4,5,6,8) (ixh_dense5.hip)
+        rc = launch_decode_dense34568(d, prefix, out_bf16, (hipStream_t)stream);
     else if ((allowed(kDecodeStaged) || allowed(kDecodeRows) || allowed(kDecodeDense)) &&
              decode_staged_supports(d, (uint32_t)chunk, out_i8, out_bf16, gs))
         rc = launch_decode_staged(d, prefix, out_bf16, gs, (hipStream_t)stream);

@@ -358,6 +358,267 @@ k_gemv34568_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, 
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The full decode by the same route turned round (for dense mixes): the codes of each level are dequantised where they
+// lie (dense, fixed positions) into five LDS arrays of bf16 weights, and every lane then gathers the weights of its 32
+// positions from the slots that the scatter above would have written to.  Spans are 2048 consecutive flat elements,
+// dealt to the waves of the launch in turn.  A lane's 64 output bytes go through LDS once more (rows 80 bytes apart),
+// so that a store instruction writes 1 KB of consecutive bytes.
+// ---------------------------------------------------------------------------------------------------------------
+template <int B>
+__device__ __forceinline__ void d5_dequant(const uint32_t (&w)[B], uint32_t *dst, uint32_t e, float scale, float minus_t_scale) {
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+        if (e > 4u * g) {
+            asm volatile("");
+#pragma unroll
+            for (int t = 2 * g; t < 2 * g + 2; ++t) {
+                const uint32_t c0 = d5_code<B>(w, 2 * t), c1 = d5_code<B>(w, 2 * t + 1);
+                dst[t] = d5_pack(__fmaf_rn((float)c0, scale, minus_t_scale), __fmaf_rn((float)c1, scale, minus_t_scale));
+            }
+        }
+    }
+}
+
+__global__ void __launch_bounds__(kWave *kD5Waves)
+k_decode34568_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, uint32_t n_spans, uint16_t *__restrict__ out) {
+    __shared__ __attribute__((aligned(16))) uint32_t lut[kD5LutBytes / 4];
+    __shared__ __attribute__((aligned(16))) uint16_t wc_all[kD5Waves][kD5Slots];
+    __shared__ uint32_t bm_all[kD5Waves][3][kD5BmWords];
+    static_assert(kD5Slots * 2 >= 64 * 80 && (kD5Slots * 2) % 16 == 0, "a wave's slots are re-used as 64 rows of 80 bytes");
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const float scale = bf16_bits_to_f32(*P.scale);
+    const float m7 = -7.0f * scale, m15 = -15.0f * scale, m31 = -31.0f * scale, m127 = -127.0f * scale;  // exact
+    for (uint32_t e = tid; e < 64 * 32; e += kWave * kD5Waves) {
+        const uint32_t idx = e >> 5;
+        lut[e] = d5_pack(dequant((int)(idx & 7u) - 3, scale), dequant((int)(idx >> 3) - 3, scale));
+    }
+    // Positions past the tensor's end walk on through the arrays; what they read is not stored but must be there to
+    // read: start from zeros.
+    for (uint32_t j = lane; j < kD5Slots / 8; j += kWave) reinterpret_cast<e_u32x4 *>(wc_all[wave])[j] = e_u32x4{0, 0, 0, 0};
+    __syncthreads();
+
+    uint16_t *const wc = wc_all[wave];
+    uint32_t *const wc32 = reinterpret_cast<uint32_t *>(wc);
+    uint32_t(*const bmw)[kD5BmWords] = bm_all[wave];
+    const uint32_t lut_lane = (lane & 31u) << 2;
+    const uint32_t entries = n_units + 1;
+    const uint32_t *__restrict__ b1 = P.bm[0];
+    const __amdgpu_buffer_rsrc_t st_rsrc[4] = {
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[0], 0, (int)(P.st_words[0] * 4u), 0x00020000),
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[1], 0, (int)(P.st_words[1] * 4u), 0x00020000),
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[2], 0, (int)(P.st_words[2] * 4u), 0x00020000),
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[3], 0, (int)(P.st_words[3] * 4u), 0x00020000)};
+    const __amdgpu_buffer_rsrc_t last_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.last, 0, (int)((P.last_bytes + 3u) & ~3u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t bm_rsrc[3] = {
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[1], 0, (int)(P.bm_words[1] * 4u), 0x00020000),
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[2], 0, (int)(P.bm_words[2] * 4u), 0x00020000),
+        __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[3], 0, (int)(P.bm_words[3] * 4u), 0x00020000)};
+
+    const uint32_t stride = gridDim.x * kD5Waves;
+    uint32_t turn = wave;
+    for (uint32_t sp = blockIdx.x * kD5Waves + wave; sp < n_spans; sp += stride, ++turn) {
+        {   // the waves that share a SIMD take turns at the issue priority, one span each
+            const uint32_t pr = turn % 3u;  // s_setprio takes an immediate
+            if (pr == 0) __builtin_amdgcn_s_setprio(0);
+            else if (pr == 1) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(2);
+        }
+        const uint32_t u0 = 4 * sp, u1 = min(u0 + 4, n_units);
+        const uint32_t p0 = u0 * kFastChunk, n_el = min(kD5Span, P.n - p0);
+        uint32_t qa[4], cnt[5];
+        {
+            uint32_t rest = n_el;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                qa[i] = (uint32_t)prefix[(size_t)i * entries + u0];
+                cnt[i] = (uint32_t)prefix[(size_t)i * entries + u1] - qa[i];
+                rest -= cnt[i];
+            }
+            cnt[4] = rest;
+        }
+        uint32_t e[5], base[5];
+        {
+            uint32_t at = 0;
+#pragma unroll
+            for (int i = 0; i < 5; ++i) {
+                e[i] = 4 * ((cnt[i] + 255) / 256);
+                base[i] = at;
+                at += 64 * e[i];
+            }
+        }
+        const uint32_t g1 = p0 - qa[0], g2 = g1 - qa[1], g3 = g2 - qa[2], at_last = g3 - qa[3];
+
+        // positions of this lane inside the span, and its bitmap word
+        const uint32_t n_here = 32 * lane < n_el ? min(32u, n_el - 32 * lane) : 0u;
+        const uint32_t w1 = n_here ? b1[(p0 >> 5) + lane] & d5_low_mask(n_here) : 0u;
+        {
+            const uint32_t gs[3] = {g1, g2, g3};
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                const uint32_t w0 = gs[j] >> 5;
+                bmw[j][lane] = __builtin_amdgcn_raw_buffer_load_b32(bm_rsrc[j], (int)((w0 + lane) * 4u), 0, 0);
+                if (lane < 4) bmw[j][64 + lane] = __builtin_amdgcn_raw_buffer_load_b32(bm_rsrc[j], (int)((w0 + 64u + lane) * 4u), 0, 0);
+            }
+        }
+        uint32_t c1w[3], c2w[4], c3w[5], c4w[6], c5w[8];
+        d5_window<3>(st_rsrc[0], (uint64_t)(qa[0] + lane * e[0]) * 3u, c1w);
+        d5_window<4>(st_rsrc[1], (uint64_t)(qa[1] + lane * e[1]) * 4u, c2w);
+        d5_window<5>(st_rsrc[2], (uint64_t)(qa[2] + lane * e[2]) * 5u, c3w);
+        d5_window<6>(st_rsrc[3], (uint64_t)(qa[3] + lane * e[3]) * 6u, c4w);
+        d5_window<8>(last_rsrc, (uint64_t)(at_last + lane * e[4]) * 8u, c5w);
+
+        // ---- dequantise every level where its codes lie ----
+        {
+            uint32_t *dst = wc32 + (lane * e[0]) / 2;
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                if (e[0] > 4u * g) {
+                    asm volatile("");
+#pragma unroll
+                    for (int t = 2 * g; t < 2 * g + 2; ++t) {
+                        const int bit = 6 * t, ob = bit & 31, d = bit >> 5;
+                        const uint32_t lo = c1w[d];
+                        const uint32_t hi = d < 2 ? c1w[d + 1] : 0u;
+                        uint32_t a;  // pair index at bits 12..7
+                        if (ob > 26) a = __builtin_amdgcn_alignbit(hi, lo, ob - 7);
+                        else if (ob >= 7) a = lo >> (ob - 7);
+                        else a = lo << (7 - ob);
+                        dst[t] = lut[((a & 0x1F80u) | lut_lane) >> 2];
+                    }
+                }
+            }
+        }
+        d5_dequant<4>(c2w, wc32 + (base[1] + lane * e[1]) / 2, e[1], scale, m7);
+        d5_dequant<5>(c3w, wc32 + (base[2] + lane * e[2]) / 2, e[2], scale, m15);
+        d5_dequant<6>(c4w, wc32 + (base[3] + lane * e[3]) / 2, e[3], scale, m31);
+        d5_dequant<8>(c5w, wc32 + (base[4] + lane * e[4]) / 2, e[4], scale, m127);
+
+        // ---- ranks: first slot of this lane in each array ----
+        auto window = [&](int j, uint32_t g, uint32_t first, uint32_t alive) {
+            const uint32_t o = (g & 31u) + first;
+            const uint32_t lo = bmw[j][o >> 5], hi = bmw[j][(o >> 5) + 1];
+            return __builtin_amdgcn_alignbit(hi, lo, o & 31u) & d5_low_mask(alive);
+        };
+        const uint32_t cnt1 = (uint32_t)__popc(w1);
+        const uint32_t alive1 = n_here - cnt1;
+        const uint32_t sc1 = wave_scan_inclusive(cnt1 | (alive1 << 16));
+        const uint32_t first1 = (sc1 & 0xffffu) - cnt1, first_a1 = (sc1 >> 16) - alive1;
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const uint32_t bits2 = window(0, g1, first_a1, alive1);
+        const uint32_t cnt2 = (uint32_t)__popc(bits2), alive2 = alive1 - cnt2;
+        const uint32_t sc2 = wave_scan_inclusive(cnt2 | (alive2 << 16));
+        const uint32_t first2 = (sc2 & 0xffffu) - cnt2, first_a2 = (sc2 >> 16) - alive2;
+        const uint32_t bits3 = window(1, g2, first_a2, alive2);
+        const uint32_t cnt3 = (uint32_t)__popc(bits3), alive3 = alive2 - cnt3;
+        const uint32_t sc3 = wave_scan_inclusive(cnt3 | (alive3 << 16));
+        const uint32_t first3 = (sc3 & 0xffffu) - cnt3, first_a3 = (sc3 >> 16) - alive3;
+        const uint32_t bits4 = window(2, g3, first_a3, alive3);
+        const uint32_t cnt4 = (uint32_t)__popc(bits4);
+        const uint32_t first4 = wave_scan_inclusive(cnt4) - cnt4;
+        const uint32_t first5 = first_a3 - first4;
+
+        // ---- gather the lane's 32 weights from their levels' arrays: the walk of the product kernel's scatter ----
+        uint32_t o[16];
+        {
+            const uint32_t wc_half = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)wc >> 1;
+            const uint32_t low1 = (uint32_t)__popc(w1 & 0xffffu);
+            const uint32_t low_a1 = min(n_here, 16u) - low1;
+            const uint32_t low2 = (uint32_t)__popc(bits2 & d5_low_mask(low_a1)), low_a2 = low_a1 - low2;
+            const uint32_t low3 = (uint32_t)__popc(bits3 & d5_low_mask(low_a2)), low_a3 = low_a2 - low3;
+            const uint32_t low4 = (uint32_t)__popc(bits4 & d5_low_mask(low_a3)), low5 = low_a3 - low4;
+            const uint32_t a1 = wc_half + base[0] + first1, a2 = wc_half + base[1] + first2, a3 = wc_half + base[2] + first3;
+            const uint32_t a4 = wc_half + base[3] + first4, a5 = wc_half + base[4] + first5;
+            e_u16x2 s1 = __builtin_bit_cast(e_u16x2, a1 | ((a1 + low1) << 16));
+            e_u16x2 s2 = __builtin_bit_cast(e_u16x2, a2 | ((a2 + low2) << 16));
+            e_u16x2 s3 = __builtin_bit_cast(e_u16x2, a3 | ((a3 + low3) << 16));
+            e_u16x2 s4 = __builtin_bit_cast(e_u16x2, a4 | ((a4 + low4) << 16));
+            e_u16x2 s5 = __builtin_bit_cast(e_u16x2, a5 | ((a5 + low5) << 16));
+            const e_u16x2 f2 = __builtin_bit_cast(e_u16x2, (bits2 & 0xffffu) | ((uint32_t)((uint64_t)bits2 >> low_a1) << 16));
+            const e_u16x2 f3 = __builtin_bit_cast(e_u16x2, (bits3 & 0xffffu) | ((uint32_t)((uint64_t)bits3 >> low_a2) << 16));
+            const e_u16x2 f4 = __builtin_bit_cast(e_u16x2, (bits4 & 0xffffu) | ((uint32_t)((uint64_t)bits4 >> low_a3) << 16));
+            e_u16x2 ja = {0, 0}, jb = {0, 0}, jc = {0, 0};
+            const e_u16x2 one = {1, 1};
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const e_u16x2 in1 = __builtin_bit_cast(e_u16x2, (w1 >> t) & 0x00010001u);
+                const e_u16x2 out1 = in1 ^ one;
+                const e_u16x2 in2 = (f2 >> ja) & out1;
+                const e_u16x2 out2 = out1 ^ in2;
+                const e_u16x2 in3 = (f3 >> jb) & out2;
+                const e_u16x2 out3 = out2 ^ in3;
+                const e_u16x2 in4 = (f4 >> jc) & out3;
+                const e_u16x2 in5 = out3 ^ in4;
+                const e_u16x2 at = in1 * (s1 - s5) + (in2 * (s2 - s5) + (in3 * (s3 - s5) + (in4 * (s4 - s5) + s5)));
+                const uint32_t at32 = __builtin_bit_cast(uint32_t, at);
+                // positions past the end of the tensor walk on through the last array; what they read is not stored
+                const uint32_t va = *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>((uintptr_t)((at32 & 0xffffu) << 1));
+                const uint32_t vb = *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>((uintptr_t)((at32 >> 16) << 1));
+                if (t & 1) {
+                    o[t >> 1] |= va << 16;
+                    o[8 + (t >> 1)] |= vb << 16;
+                } else {
+                    o[t >> 1] = va;
+                    o[8 + (t >> 1)] = vb;
+                }
+                s1 += in1; s2 += in2; s3 += in3; s4 += in4; s5 += in5;
+                ja += out1; jb += out2; jc += out3;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+
+        // ---- the lane's 64 bytes to their place in the output ----
+        uint16_t *dst = out + (size_t)p0 + 32 * lane;
+        if (n_el == kD5Span) {
+            e_u32x4 *const rows = reinterpret_cast<e_u32x4 *>(wc);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) rows[lane * 5 + j] = e_u32x4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            e_u32x4 *const line = reinterpret_cast<e_u32x4 *>(out + (size_t)p0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) line[64 * j + lane] = rows[(16 * j + (lane >> 2)) * 5 + (lane & 3u)];
+        } else if (n_here == 32) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                reinterpret_cast<e_u32x4 *>(dst)[j] = e_u32x4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
+        } else {
+            for (uint32_t t = 0; t < n_here; ++t) {
+                uint32_t v = 0;
+#pragma unroll
+                for (int j = 0; j < 16; ++j) v = (t >> 1) == (uint32_t)j ? o[j] : v;  // o[j]: positions 2j and 2j + 1
+                dst[t] = (uint16_t)((t & 1u) ? v >> 16 : v);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+bool decode_dense34568_supports(const Dev &P, uint32_t chunk, const int8_t *o8, const uint16_t *o16) {
+    return P.n_levels == 5 && P.bits[0] == 3 && P.bits[1] == 4 && P.bits[2] == 5 && P.bits[3] == 6 && P.bits[4] == 8 &&
+           chunk == kFastChunk && !o8 && o16 && ((uintptr_t)o16 & 15u) == 0 && ((uintptr_t)P.last & 3u) == 0 && P.n != 0;
+}
+
+int launch_decode_dense34568(const Dev &P, const int32_t *prefix, uint16_t *o16, hipStream_t s) {
+    const uint32_t n_units = (P.n + kFastChunk - 1) / kFastChunk;
+    const uint32_t n_spans = (n_units + 3) / 4;
+    static const uint32_t resident = [] {
+        int dev = 0, n_cu = 256, per_cu = 0;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_decode34568_dense, kWave * kD5Waves, 0) != hipSuccess || per_cu < 1)
+            per_cu = 3;
+        return (uint32_t)n_cu * (uint32_t)per_cu;
+    }();
+    const uint32_t blocks = min(resident, (n_spans + kD5Waves - 1) / kD5Waves);
+    hipLaunchKernelGGL(k_decode34568_dense, dim3(blocks), dim3(kWave * kD5Waves), 0, s, P, prefix, n_units, n_spans, o16);
+    return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
+}
+
 bool gemv_dense34568_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x) {
     return P.n_levels == 5 && P.bits[0] == 3 && P.bits[1] == 4 && P.bits[2] == 5 && P.bits[3] == 6 && P.bits[4] == 8 &&
            chunk == kFastChunk && m == 1 && P.in_f % kFastChunk == 0 && P.in_f != 0 && ((uintptr_t)x & 15u) == 0 &&

@@ -32,7 +32,9 @@ MAX_FUSED_ROWS = 16  # activation rows served by the fused decode+GEMV kernel
 # level 1, MI355X: the pair takes 72-75 us on 17408 x 5120 and 5120 x 17408 at any M up to 32 and 34-50 us on
 # 5120 x 5120; the fused kernels take 31 / 35 / 41 us (17408 x 5120), 39 / 46 / 60 us (5120 x 17408) and 38 / 51 / 63 us
 # (5120 x 5120) at M = 8 / 12 / 16: up to 8 rows everywhere, up to 16 on the large layers.  Dense mixes (55 / 40 / 5 %):
-# the pair takes 92 us, the fused kernels 75 / 93 / 131 us at M = 2 / 4 / 8.
+# the pair takes 84-90 us, the fused kernels 55-62 / 69-72 / 85-88 / 116-119 us at M = 1 / 2 / 4 / 8.  Dense mixes in
+# other schemes have a level-by-level kernel for one row only (five levels: 95-104 us; the pair 127 us, the any-scheme
+# kernel 209-260 us at M = 2 .. 8).
 MAX_FUSED_ROWS_WITH_BUFFER = 8
 MAX_FUSED_ROWS_WITH_BUFFER_LARGE = 16
 LARGE_LAYER_ELEMENTS = 64 * 1024 * 1024
@@ -139,8 +141,10 @@ class StreamingLinear(nn.Module):
         elif self.counts[0] * 100 >= self.N * 97:
             large = self.N >= LARGE_LAYER_ELEMENTS and self.level_bits == (3, 5, 8)
             fused_rows = MAX_FUSED_ROWS_WITH_BUFFER_LARGE if large else MAX_FUSED_ROWS_WITH_BUFFER
-        else:
+        elif self.level_bits == (3, 5, 8):
             fused_rows = MAX_FUSED_ROWS_WITH_BUFFER_DENSE
+        else:
+            fused_rows = 1
         if (self._use_fused and x.dtype == torch.bfloat16 and x.is_cuda and 1 <= rows <= fused_rows
                 and x.shape[-1] == self.in_features):
             x2 = x.reshape(rows, self.in_features)

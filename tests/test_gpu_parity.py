@@ -171,6 +171,26 @@ def test_decode_358_each_decoder(oracle, dev, force_decoder, kind, shape, decode
     assert torch.all(o16[p["N"]:] == 7.0)  # nothing written past the end
 
 
+@pytest.mark.parametrize("decoder", ["auto", "dense"])
+@pytest.mark.parametrize("kind", KINDS + ["five_dense", "zeros"])
+@pytest.mark.parametrize("shape", [(1, 1), (1, 31), (1, 512), (3, 171), (5, 413), (33, 1000), (64, 1536), (300, 1031),
+                                   (256, 4608), (17, 2048), (1, 2049), (52, 512), (1000, 2048)])
+def test_decode_34568_level_by_level(oracle, dev, force_decoder, kind, shape, decoder):
+    """(3,4,5,6,8) to bf16 at unit 512 through the five-level level-by-level decoder: what the library picks for dense
+    mixes, forced for the others (partial last lane, partial last span, tensors smaller than a lane)."""
+    force_decoder(decoder)
+    if kind == "zeros":
+        p = quantize(torch.zeros(shape, dtype=torch.bfloat16), (3, 4, 5, 6, 8))
+    else:
+        p = make_packed(kind, *shape, (3, 4, 5, 6, 8))
+    dp = device_packed(p, dev)
+    table = dp.prefix_build(512)
+    o16 = torch.full((p["N"] + 64,), 7.0, dtype=torch.bfloat16, device=dev)
+    dp.decode(table, 512, out_bf16=o16[: p["N"]])
+    assert np.array_equal(bf16_bits(o16[: p["N"]]).reshape(shape), oracle.decode_packed_bf16(p)), (kind, shape, decoder)
+    assert torch.all(o16[p["N"]:] == 7.0)  # nothing written past the end
+
+
 @pytest.mark.parametrize("level_bits", [(3, 4, 5, 6, 8), (3, 8), (3, 3, 8), (3, 4, 8), (3, 5, 6, 7, 8), (3, 4, 5, 6, 7, 8)])
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("shape", [(8, 512), (64, 1536), (1000, 2048)])
