@@ -43,10 +43,10 @@ MEASURED_TRAFFIC_BYTES = {
     "down_proj_5120x17408_m1_student_t": (23020.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "bdc69284735fd9fa"),
     "attn_proj_5120x5120_m1_student_t": (7110.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "bdc69284735fd9fa"),
     "down_proj_5120x17408_m1_calibrated": (33832.0 * 2.0 * 1024 + 40.0 * 1024, _DENSE, "4c194d30b116b40a"),
-    "down_proj_5120x17408_m1_five_level_calibrated": (49711.0 * 2.0 * 1024 + 1338.0 * 1024, _DENSE5, "25b0f9e2ddc3a686"),
+    "down_proj_5120x17408_m1_five_level_calibrated": (49711.0 * 2.0 * 1024 + 1337.0 * 1024, _DENSE5, "af662fec32ed7b32"),
     "gate_up_17408x5120_m4_student_t": (28079.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "3ceb514690dd072e"),
     "gate_up_17408x5120_m16_student_t": (26457.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "3ceb514690dd072e"),
-    "decode_5120x17408_five_level_calibrated": (48964.0 * 2.0 * 1024 + 174080.0 * 1024, _DENSE5, "25b0f9e2ddc3a686"),
+    "decode_5120x17408_five_level_calibrated": (49723.0 * 2.0 * 1024 + 174080.0 * 1024, _DENSE5, "af662fec32ed7b32"),
     "prefill_5120x5120_m512_five_level": (50297.9 * 2.0 * 1024 + 30720.0 * 1024,) + _OLD,
     "decode_5120x17408_student_t": (23268.0 * 2.0 * 1024 + 179524.0 * 1024,) + _OLD,
     "decode_5120x17408_calibrated": (36308.0 * 2.0 * 1024 + 174080.0 * 1024,) + _OLD,

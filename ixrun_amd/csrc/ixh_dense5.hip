@@ -62,12 +62,11 @@ __device__ __forceinline__ float d5_dot2(uint32_t w, uint32_t x, float acc) {
 // the low `n` bits set (n = 0 .. 32)
 __device__ __forceinline__ uint32_t d5_low_mask(uint32_t n) { return (uint32_t)(0xFFFFFFFFull >> (32u - n)); }
 
-// A lane's window of a code stream: B + 1 dwords from the dword that holds code `first` on, shifted so that the code
-// starts at bit 0 of w[0].  A dword past the stream's end reads as zero.
+// A lane's window of a code stream: B + 1 dwords from the dword that holds the bit `first_bit` on (d5_fetch), shifted
+// so that the bit lands at bit 0 of w[0] (d5_align).  A dword past the stream's end reads as zero.
 template <int B>
-__device__ __forceinline__ void d5_window(__amdgpu_buffer_rsrc_t rsrc, uint64_t first_bit, uint32_t (&w)[B]) {
-    const uint32_t at = (uint32_t)(first_bit >> 5) * 4u, sh = (uint32_t)first_bit & 31u;
-    uint32_t d[B + 1];
+__device__ __forceinline__ void d5_fetch(__amdgpu_buffer_rsrc_t rsrc, uint64_t first_bit, uint32_t (&d)[B + 1]) {
+    const uint32_t at = (uint32_t)(first_bit >> 5) * 4u;
 #pragma unroll
     for (int j = 0; j + 4 <= B + 1; j += 4) {
         const e_u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(at + 4u * j), 0, 0);
@@ -83,8 +82,20 @@ __device__ __forceinline__ void d5_window(__amdgpu_buffer_rsrc_t rsrc, uint64_t 
         const e_u32x3 v = __builtin_amdgcn_raw_buffer_load_b96(rsrc, (int)(at + 4u * done), 0, 0);
         d[done] = v[0]; d[done + 1] = v[1]; d[done + 2] = v[2];
     }
+}
+
+template <int B>
+__device__ __forceinline__ void d5_align(const uint32_t (&d)[B + 1], uint64_t first_bit, uint32_t (&w)[B]) {
+    const uint32_t sh = (uint32_t)first_bit & 31u;
 #pragma unroll
     for (int j = 0; j < B; ++j) w[j] = __builtin_amdgcn_alignbit(d[j + 1], d[j], sh);
+}
+
+template <int B>
+__device__ __forceinline__ void d5_window(__amdgpu_buffer_rsrc_t rsrc, uint64_t first_bit, uint32_t (&w)[B]) {
+    uint32_t d[B + 1];
+    d5_fetch<B>(rsrc, first_bit, d);
+    d5_align<B>(d, first_bit, w);
 }
 
 // code t (a compile-time index) of a window of B-bit codes
@@ -417,58 +428,99 @@ k_decode34568_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units,
         __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[2], 0, (int)(P.bm_words[2] * 4u), 0x00020000),
         __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[3], 0, (int)(P.bm_words[3] * 4u), 0x00020000)};
 
+    // What a span needs from memory before any arithmetic: its table entries (scalars), the lane's word of the first
+    // bitmap, the span's part of the nested bitmaps and the lane's window of every code stream.  They are asked for one
+    // span ahead (the table entries two), so that a wave's chain table -> windows -> arithmetic waits for memory once.
+    struct Ranks { uint32_t qa[4], qb[4]; };
+    struct Shape { uint32_t p0, n_el, e[5], base[5], g1, g2, g3, at_last; };
+    struct Loads { uint32_t w1, bm[3], bmx[3], d1[4], d2[5], d3[6], d4[7], d5[9]; };
+    auto table_of = [&](uint32_t sp) {
+        Ranks q;
+        const uint32_t u0 = 4 * sp, u1 = min(u0 + 4, n_units);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            q.qa[i] = (uint32_t)prefix[(size_t)i * entries + u0];
+            q.qb[i] = (uint32_t)prefix[(size_t)i * entries + u1];
+        }
+        return q;
+    };
+    auto shape_of = [&](uint32_t sp, const Ranks &q) {
+        Shape g;
+        g.p0 = 4 * sp * kFastChunk;
+        g.n_el = min(kD5Span, P.n - g.p0);
+        uint32_t rest = g.n_el, at = 0;
+#pragma unroll
+        for (int i = 0; i < 5; ++i) {
+            const uint32_t cnt = i < 4 ? q.qb[i < 4 ? i : 0] - q.qa[i < 4 ? i : 0] : rest;
+            rest -= i < 4 ? cnt : 0u;
+            g.e[i] = 4 * ((cnt + 255) / 256);
+            g.base[i] = at;
+            at += 64 * g.e[i];
+        }
+        g.g1 = g.p0 - q.qa[0]; g.g2 = g.g1 - q.qa[1]; g.g3 = g.g2 - q.qa[2]; g.at_last = g.g3 - q.qa[3];
+        return g;
+    };
+    auto fetch = [&](const Shape &g, const Ranks &q) {
+        Loads r;
+        const uint32_t n_here = 32 * lane < g.n_el ? min(32u, g.n_el - 32 * lane) : 0u;
+        r.w1 = n_here ? b1[(g.p0 >> 5) + lane] & d5_low_mask(n_here) : 0u;
+        const uint32_t gs[3] = {g.g1, g.g2, g.g3};
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const uint32_t w0 = gs[j] >> 5;
+            r.bm[j] = __builtin_amdgcn_raw_buffer_load_b32(bm_rsrc[j], (int)((w0 + lane) * 4u), 0, 0);
+            r.bmx[j] = lane < 4 ? __builtin_amdgcn_raw_buffer_load_b32(bm_rsrc[j], (int)((w0 + 64u + lane) * 4u), 0, 0) : 0u;
+        }
+        d5_fetch<3>(st_rsrc[0], (uint64_t)(q.qa[0] + lane * g.e[0]) * 3u, r.d1);
+        d5_fetch<4>(st_rsrc[1], (uint64_t)(q.qa[1] + lane * g.e[1]) * 4u, r.d2);
+        d5_fetch<5>(st_rsrc[2], (uint64_t)(q.qa[2] + lane * g.e[2]) * 5u, r.d3);
+        d5_fetch<6>(st_rsrc[3], (uint64_t)(q.qa[3] + lane * g.e[3]) * 6u, r.d4);
+        d5_fetch<8>(last_rsrc, (uint64_t)(g.at_last + lane * g.e[4]) * 8u, r.d5);
+        return r;
+    };
+
     const uint32_t stride = gridDim.x * kD5Waves;
-    uint32_t turn = wave;
-    for (uint32_t sp = blockIdx.x * kD5Waves + wave; sp < n_spans; sp += stride, ++turn) {
+    uint32_t sp = blockIdx.x * kD5Waves + wave;
+    if (sp >= n_spans) return;
+    // past the end the last span is fetched once more: loads that nobody uses
+    auto next_of = [&](uint32_t s) { return s + stride < n_spans ? s + stride : s; };
+    Ranks q_now = table_of(sp);
+    Shape g_now = shape_of(sp, q_now);
+    Loads in_now = fetch(g_now, q_now);
+    uint32_t sp_next = next_of(sp);
+    Ranks q_next = table_of(sp_next);
+    for (uint32_t turn = wave;; ++turn) {
         {   // the waves that share a SIMD take turns at the issue priority, one span each
             const uint32_t pr = turn % 3u;  // s_setprio takes an immediate
             if (pr == 0) __builtin_amdgcn_s_setprio(0);
             else if (pr == 1) __builtin_amdgcn_s_setprio(1);
             else __builtin_amdgcn_s_setprio(2);
         }
-        const uint32_t u0 = 4 * sp, u1 = min(u0 + 4, n_units);
-        const uint32_t p0 = u0 * kFastChunk, n_el = min(kD5Span, P.n - p0);
-        uint32_t qa[4], cnt[5];
-        {
-            uint32_t rest = n_el;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                qa[i] = (uint32_t)prefix[(size_t)i * entries + u0];
-                cnt[i] = (uint32_t)prefix[(size_t)i * entries + u1] - qa[i];
-                rest -= cnt[i];
-            }
-            cnt[4] = rest;
-        }
-        uint32_t e[5], base[5];
-        {
-            uint32_t at = 0;
-#pragma unroll
-            for (int i = 0; i < 5; ++i) {
-                e[i] = 4 * ((cnt[i] + 255) / 256);
-                base[i] = at;
-                at += 64 * e[i];
-            }
-        }
-        const uint32_t g1 = p0 - qa[0], g2 = g1 - qa[1], g3 = g2 - qa[2], at_last = g3 - qa[3];
+        const Shape g_next = shape_of(sp_next, q_next);
+        const Loads in_next = fetch(g_next, q_next);
+        const uint32_t sp_after = next_of(sp_next);
+        const Ranks q_after = table_of(sp_after);
+
+        const uint32_t p0 = g_now.p0, n_el = g_now.n_el;
+        const uint32_t(&qa)[4] = q_now.qa;
+        const uint32_t(&e)[5] = g_now.e;
+        const uint32_t(&base)[5] = g_now.base;
+        const uint32_t g1 = g_now.g1, g2 = g_now.g2, g3 = g_now.g3, at_last = g_now.at_last;
 
         // positions of this lane inside the span, and its bitmap word
         const uint32_t n_here = 32 * lane < n_el ? min(32u, n_el - 32 * lane) : 0u;
-        const uint32_t w1 = n_here ? b1[(p0 >> 5) + lane] & d5_low_mask(n_here) : 0u;
-        {
-            const uint32_t gs[3] = {g1, g2, g3};
+        const uint32_t w1 = in_now.w1;
 #pragma unroll
-            for (int j = 0; j < 3; ++j) {
-                const uint32_t w0 = gs[j] >> 5;
-                bmw[j][lane] = __builtin_amdgcn_raw_buffer_load_b32(bm_rsrc[j], (int)((w0 + lane) * 4u), 0, 0);
-                if (lane < 4) bmw[j][64 + lane] = __builtin_amdgcn_raw_buffer_load_b32(bm_rsrc[j], (int)((w0 + 64u + lane) * 4u), 0, 0);
-            }
+        for (int j = 0; j < 3; ++j) {
+            bmw[j][lane] = in_now.bm[j];
+            if (lane < 4) bmw[j][64 + lane] = in_now.bmx[j];
         }
         uint32_t c1w[3], c2w[4], c3w[5], c4w[6], c5w[8];
-        d5_window<3>(st_rsrc[0], (uint64_t)(qa[0] + lane * e[0]) * 3u, c1w);
-        d5_window<4>(st_rsrc[1], (uint64_t)(qa[1] + lane * e[1]) * 4u, c2w);
-        d5_window<5>(st_rsrc[2], (uint64_t)(qa[2] + lane * e[2]) * 5u, c3w);
-        d5_window<6>(st_rsrc[3], (uint64_t)(qa[3] + lane * e[3]) * 6u, c4w);
-        d5_window<8>(last_rsrc, (uint64_t)(at_last + lane * e[4]) * 8u, c5w);
+        d5_align<3>(in_now.d1, (uint64_t)(qa[0] + lane * e[0]) * 3u, c1w);
+        d5_align<4>(in_now.d2, (uint64_t)(qa[1] + lane * e[1]) * 4u, c2w);
+        d5_align<5>(in_now.d3, (uint64_t)(qa[2] + lane * e[2]) * 5u, c3w);
+        d5_align<6>(in_now.d4, (uint64_t)(qa[3] + lane * e[3]) * 6u, c4w);
+        d5_align<8>(in_now.d5, (uint64_t)(at_last + lane * e[4]) * 8u, c5w);
 
         // ---- dequantise every level where its codes lie ----
         {
@@ -596,6 +648,13 @@ k_decode34568_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units,
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
+        if (sp + stride >= n_spans) break;
+        sp = sp_next;
+        q_now = q_next;
+        g_now = g_next;
+        in_now = in_next;
+        sp_next = sp_after;
+        q_next = q_after;
     }
 }
 
