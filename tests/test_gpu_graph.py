@@ -10,15 +10,22 @@ from helpers import activations, bf16_bits, outlier_weight, student_t_weight
 pytestmark = pytest.mark.gpu
 
 
-def build_chain(n_layers, width, dev, maker):
+def build_chain(n_layers, width, dev, maker, level_bits=(3, 5, 8)):
     from ixrun_amd.engine import StreamingLinear
     from ixrun_amd.quantize import int8x_quantize
 
     layers = []
     for k in range(n_layers):
-        sl = StreamingLinear(int8x_quantize(maker(width, width, seed=k)))
+        sl = StreamingLinear(int8x_quantize(maker(width, width, seed=k), level_bits))
         layers.append(sl)
     return layers
+
+
+def dense_weight(out_f, in_f, seed=0):
+    """Weights whose every level is well populated, in (3,5,8) and in (3,4,5,6,8)."""
+    from helpers import calibrated_weight
+
+    return calibrated_weight(out_f, in_f, seed=seed, scale=0.0123046875)[0]
 
 
 def run_chain(layers, x):
@@ -28,10 +35,12 @@ def run_chain(layers, x):
     return h
 
 
-@pytest.mark.parametrize("maker,m", [(student_t_weight, 1), (outlier_weight, 1), (student_t_weight, 4), (outlier_weight, 16)])
-def test_graph_replay_matches_eager(maker, m):
+@pytest.mark.parametrize("maker,m,level_bits", [
+    (student_t_weight, 1, (3, 5, 8)), (outlier_weight, 1, (3, 5, 8)), (student_t_weight, 4, (3, 5, 8)),
+    (outlier_weight, 16, (3, 5, 8)), (dense_weight, 1, (3, 4, 5, 6, 8)), (student_t_weight, 16, (3, 4, 5, 6, 8))])
+def test_graph_replay_matches_eager(maker, m, level_bits):
     dev = torch.device("cuda:0")
-    layers = build_chain(6, 1024, dev, maker)
+    layers = build_chain(6, 1024, dev, maker, level_bits)
     x = activations(m, 1024, seed=3).to(dev)
     eager = run_chain(layers, x).clone()
     torch.cuda.synchronize()
