@@ -44,6 +44,8 @@
 
 namespace ixh {
 
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
 
 // a wave's region: ring, record queue, row sums, task list, and a copy of the activations of its own column
 // blocks (c blocks x mt rows x 512 bf16) for the elements above level 1
@@ -529,9 +531,8 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     const float scale = bf16_bits_to_f32(*P.scale);
     for (uint32_t i = tid; i < 64 * 32; i += blockDim.x) {
         const int c0 = (i >> 5) & 7, c1 = i >> 8;
-        const uint32_t w0 = c0 < 7 ? f32_to_bf16_bits((float)(c0 - 3) * scale) : 0u;
-        const uint32_t w1 = c1 < 7 ? f32_to_bf16_bits((float)(c1 - 3) * scale) : 0u;
-        lut[i] = w0 | (w1 << 16);
+        const f32x2 w = {c0 < 7 ? (float)(c0 - 3) * scale : 0.0f, c1 < 7 ? (float)(c1 - 3) * scale : 0.0f};
+        lut[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(w, bf16x2));  // round to nearest even
     }
     if (tid <= 32) {
         const uint32_t pos = 3 * tid;
