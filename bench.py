@@ -40,12 +40,13 @@ _DENSE = ("ixh_dense358.hip", "ixh_dev.h")
 _DENSE5 = ("ixh_dense5.hip", "ixh_dev.h")
 _OLD = ((), "measured-on-earlier-sources")  # figures kept for the record; reported as null
 MEASURED_TRAFFIC_BYTES = {
-    "down_proj_5120x17408_m1_student_t": (23024.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "f6a8e7cf437e671a"),
-    "attn_proj_5120x5120_m1_student_t": (7104.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "f6a8e7cf437e671a"),
+    "down_proj_5120x17408_m1_student_t": (23024.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "f61463e8fdfda96e"),
+    "attn_proj_5120x5120_m1_student_t": (7104.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "f61463e8fdfda96e"),
     "down_proj_5120x17408_m1_calibrated": (33832.0 * 2.0 * 1024 + 40.0 * 1024, _DENSE, "4c194d30b116b40a"),
     "down_proj_5120x17408_m1_five_level_calibrated": (49711.0 * 2.0 * 1024 + 1337.0 * 1024, _DENSE5, "af662fec32ed7b32"),
-    "gate_up_17408x5120_m4_student_t": (28079.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "3ceb514690dd072e"),
-    "gate_up_17408x5120_m16_student_t": (26457.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "3ceb514690dd072e"),
+    "gate_up_17408x5120_m4_student_t": (28114.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "5f7084e4014eec5e"),
+    "gate_up_17408x5120_m16_student_t": (24827.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "5f7084e4014eec5e"),
+    "attn_proj_5120x5120_m16_student_t": (7787.0 * 2.0 * 1024 + 256.0 * 1024, _TILES, "5f7084e4014eec5e"),
     "decode_5120x17408_five_level_calibrated": (49723.0 * 2.0 * 1024 + 174080.0 * 1024, _DENSE5, "af662fec32ed7b32"),
     "prefill_5120x5120_m512_five_level": (50297.9 * 2.0 * 1024 + 30720.0 * 1024,) + _OLD,
     "decode_5120x17408_student_t": (23268.0 * 2.0 * 1024 + 179524.0 * 1024,) + _OLD,
@@ -70,6 +71,12 @@ WORKLOADS = {
     "attn_proj_5120x5120_m1_calibrated": (5120, 5120, 1, "calibrated"),
     "graph64_5120x5120_m1_calibrated": (5120, 5120, 1, "calibrated"),
     "attn_proj_5120x5120_m1_student_t": (5120, 5120, 1, "student_t"),
+    "down_proj_5120x17408_m4_student_t": (5120, 17408, 4, "student_t"),
+    "down_proj_5120x17408_m8_student_t": (5120, 17408, 8, "student_t"),
+    "down_proj_5120x17408_m16_student_t": (5120, 17408, 16, "student_t"),
+    "attn_proj_5120x5120_m4_student_t": (5120, 5120, 4, "student_t"),
+    "attn_proj_5120x5120_m8_student_t": (5120, 5120, 8, "student_t"),
+    "attn_proj_5120x5120_m16_student_t": (5120, 5120, 16, "student_t"),
     "gate_up_17408x5120_m2_student_t": (17408, 5120, 2, "student_t"),
     "gate_up_17408x5120_m4_student_t": (17408, 5120, 4, "student_t"),
     "gate_up_17408x5120_m8_student_t": (17408, 5120, 8, "student_t"),
@@ -443,8 +450,10 @@ def also_block(dev, args):
         ("down_proj_5120x17408_m1_reference_recipe", [("down_proj_5120x17408_m1_reference_recipe", 1, "fused")]),
         ("down_proj_5120x17408_m1_five_level_calibrated", [("down_proj_5120x17408_m1_five_level_calibrated", 1, "fused")]),
         ("down_proj_5120x17408_m1_student_t", [("down_proj_5120x17408_m1_student_t_split_k_call", 1, "split_k"),
-                                               ("down_proj_5120x17408_m1_student_t_split_k_kernel_alone", 1, "split_k_bare")]),
-        ("attn_proj_5120x5120_m1_student_t", [("attn_proj_5120x5120_m1_student_t", 1, "fused")]),
+                                               ("down_proj_5120x17408_m1_student_t_split_k_kernel_alone", 1, "split_k_bare")]
+                                              + [(f"down_proj_5120x17408_m{m}_student_t", m, "fused") for m in (4, 8, 16)]),
+        ("attn_proj_5120x5120_m1_student_t", [("attn_proj_5120x5120_m1_student_t", 1, "fused")]
+                                             + [(f"attn_proj_5120x5120_m{m}_student_t", m, "fused") for m in (4, 8, 16)]),
         ("gate_up_17408x5120_m2_student_t", [(f"gate_up_17408x5120_m{m}_student_t", m, "fused") for m in (2, 4, 8, 16)]),
         ("graph64_5120x5120_m1_student_t", [("graph64_5120x5120_m1_student_t", 1, "fused")]),
         ("prefill_5120x17408_m512_five_level", [("prefill_5120x17408_m512_five_level", 512, "fused"),

@@ -84,9 +84,13 @@ const char *ixh_last_error(void);
  *                    call is skipped for that call
  *   "gemv_shared_x"  most activation rows (0..8, default 8) that ixh_gemv gives to the row-block kernel that
  *                    shares the activations through on-chip memory; 0 = never
- *   "gemv_tiles"     the tile kernel (16 weight rows x up to 16 activation rows per matrix instruction): -1 = never,
- *                    0 = where it pays (three activation rows or more, tiles at least half full; default),
- *                    1 = wherever it fits
+ *   "gemv_tiles"     the tile kernel (16, 8 or 4 weight rows x up to 16, 8 or 4 activation rows per matrix
+ *                    instruction): -1 = never, 0 = where it pays (three activation rows or more, tiles at least half
+ *                    full; default), 1 = wherever it fits
+ *   "gemv_tile_rows" the tile kernel's tile shape: 0 = the planner's choice (default), 2 / 3 / 4 = tiles of 4 / 8 / 16
+ *                    weight rows only (a shape that cannot serve the call's activation rows hands the call on)
+ *   "gemv_tile_cus"  the number of CUs over which the tile kernel's planner spreads the rows: 0 = the device's
+ *                    (default), 1..4096 = that many (small tensors then get workgroups with several tiles)
  *   "gemv_strips"    the strip kernel (up to eight activation rows a pass): -1 = never, 0 = for three rows or more
  *                    where the tile kernel does not run and the shape fits (default), 1..6 = wherever it fits
  * Returns IXH_EINVAL for an unknown name or a value out of range.  Calls already running are not affected.

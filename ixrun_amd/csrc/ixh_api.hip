@@ -18,6 +18,8 @@ std::atomic<int> g_opt_decode_kernel{kDecodeAuto};
 std::atomic<int> g_opt_gemv_shared_x{8};
 std::atomic<int> g_opt_gemv_strips{0};
 std::atomic<int> g_opt_gemv_tiles{0};
+std::atomic<int> g_opt_gemv_tile_rows{0};
+std::atomic<int> g_opt_gemv_tile_cus{0};
 
 void set_error(const char *fmt, ...) {
     va_list ap;
@@ -105,6 +107,16 @@ int ixh_set_option(const char *name, int64_t value) {
     if (strcmp(name, "gemv_tiles") == 0) {
         if (value < -1 || value > 1) { set_error("gemv_tiles %lld not in -1..1", (long long)value); return IXH_EINVAL; }
         g_opt_gemv_tiles.store((int)value, std::memory_order_relaxed);
+        return IXH_OK;
+    }
+    if (strcmp(name, "gemv_tile_rows") == 0) {
+        if (value != 0 && value != 2 && value != 3 && value != 4) { set_error("gemv_tile_rows %lld not 0, 2, 3 or 4", (long long)value); return IXH_EINVAL; }
+        g_opt_gemv_tile_rows.store((int)value, std::memory_order_relaxed);
+        return IXH_OK;
+    }
+    if (strcmp(name, "gemv_tile_cus") == 0) {
+        if (value < 0 || value > 4096) { set_error("gemv_tile_cus %lld not in 0..4096", (long long)value); return IXH_EINVAL; }
+        g_opt_gemv_tile_cus.store((int)value, std::memory_order_relaxed);
         return IXH_OK;
     }
     if (strcmp(name, "gemv_strips") == 0) {

@@ -124,14 +124,24 @@ struct TaskPool {
     uint32_t addr, total, first_round, round_stride, queues_addr, queue_stride;
 };
 
-template <int MT, bool STAGED, bool ANY = false, int XL = 0, bool POOL = false, uint32_t STRIP = kStripBytes>
-__device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, uint32_t tq1_addr, uint32_t tq2_addr,
+// SINK: where a resolved element goes when it is not added to the row sums here (XL == 2 only): put() takes the
+// weight's bf16 bits, the record's row field and the LDS address of the element's column in the first activation
+// row, idle() is called by the lanes that have no element in a round, and flush() by the whole wave after every
+// round of at most 64 elements (its argument: the lanes below that number may have taken part).
+struct NoSink {
+    static constexpr bool active = false;
+    __device__ __forceinline__ void put(uint32_t, uint32_t, uint32_t) {}
+    __device__ __forceinline__ void idle() {}
+    __device__ __forceinline__ void flush(uint32_t) {}
+};
+
+template <int MT, bool STAGED, bool ANY, int XL, bool POOL, uint32_t STRIP, class SINK>
+__device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const SideView &sv, uint32_t tq1_addr, uint32_t tq2_addr,
                                              uint32_t unit0, const uint4 *__restrict__ queue, uint32_t count,
                                              uint32_t rowacc_addr, uint16_t *__restrict__ tasks,
                                              uint32_t xs_addr, uint32_t xs_row, uint32_t k_first,
                                              int m, float scale, uint32_t lane,
-                                             const int32_t *__restrict__ prefix = nullptr, uint32_t entries = 0,
-                                             TaskPool pool = TaskPool{0, 0, 0, 1, 0, 0}) {
+                                             const int32_t *__restrict__ prefix, uint32_t entries, TaskPool pool) {
     const uint32_t *__restrict__ b2 = P.bm[1];
     const uint32_t b2_words = P.bm_words[1];
     // value of the element at rank r of bitmap 1's domain, unit `unit`, any scheme
@@ -180,6 +190,10 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
         // XL == 2 (up to 16 activation rows): the activations are read in a loop at the end, one register at a time
         auto add_all = [&](float w) {
             const uint32_t xa = xs_addr + ((k0 - k_first) >> 7) * STRIP + ((k0 & 127u) + e) * 2u;
+            if (SINK::active) {
+                sink.put(__float_as_uint(w) >> 16, slot, xa);
+                return;
+            }
             const uint32_t ra = rowacc_addr + slot * (uint32_t)m * 4u;
 #pragma unroll 1
             for (int j = 0; j < m; ++j)
@@ -282,7 +296,22 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
                 if (tb + lane < n_tasks) {
                     const uint32_t task = tasks[tb + lane];
                     one(queue[base + (task >> 10)], (task >> 5) & 31u, task & 31u);
+                } else if (SINK::active) {
+                    sink.idle();
                 }
+                if (SINK::active) sink.flush(n_tasks - tb);
+            }
+        } else if (SINK::active) {
+            uint32_t nth = 0;
+            for (uint64_t left = __ballot(zeros != 0); left != 0; left = __ballot(zeros != 0)) {
+                if (zeros != 0) {
+                    const uint32_t e = (uint32_t)__builtin_ctz(zeros);
+                    zeros &= zeros - 1;
+                    one(rec, nth++, e);
+                } else {
+                    sink.idle();
+                }
+                sink.flush(64u - (uint32_t)__builtin_clzll(left));
             }
         } else {
             uint32_t nth = 0;
@@ -294,6 +323,19 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
         }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the row sums have taken the additions
+}
+
+template <int MT, bool STAGED, bool ANY = false, int XL = 0, bool POOL = false, uint32_t STRIP = kStripBytes>
+__device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, uint32_t tq1_addr, uint32_t tq2_addr,
+                                             uint32_t unit0, const uint4 *__restrict__ queue, uint32_t count,
+                                             uint32_t rowacc_addr, uint16_t *__restrict__ tasks,
+                                             uint32_t xs_addr, uint32_t xs_row, uint32_t k_first,
+                                             int m, float scale, uint32_t lane,
+                                             const int32_t *__restrict__ prefix = nullptr, uint32_t entries = 0,
+                                             TaskPool pool = TaskPool{0, 0, 0, 1, 0, 0}) {
+    NoSink none;
+    resolve_rows_to<MT, STAGED, ANY, XL, POOL, STRIP>(none, P, sv, tq1_addr, tq2_addr, unit0, queue, count, rowacc_addr, tasks,
+                                                      xs_addr, xs_row, k_first, m, scale, lane, prefix, entries, pool);
 }
 
 // s_setprio takes an immediate

@@ -1,10 +1,14 @@
 // (3,5,8) fused decode + skinny GEMM for gfx950, tile variant: 16 weight rows x 16 activation rows per matrix
 // instruction, so that up to 16 activation rows cost what one costs.
 //
-// Work split.  A workgroup owns whole rows.  Its rows are cut into tiles of 16; a wave belongs to one tile and to one
-// share of the column blocks for its whole life, so its 16 x 16 accumulator never leaves its registers: wave =
-// tile * n_sub + sub, and the column blocks (512 wide) of a part are dealt in runs to the n_sub waves of a tile.
-// Lane (n, kg), n = lane % 16, kg = lane / 16, decodes strip kg (128 columns) of row n of the tile, word by word, exactly
+// Work split.  A workgroup owns whole rows.  Its rows are cut into tiles of 16, 8 or 4 (one size per launch); a tile of
+// 16 / s rows takes s column blocks side by side in a step (slots), so that the 16 columns of the matrix instruction
+// are always 16 different (row, block) pairs, and serves up to 16 / s activation rows: row a of the other operand is
+// activation row a % (16 / s) at the columns of slot a / (16 / s), and the products whose slots agree are the sums.
+// Short tiles fill the lanes where a workgroup's rows are not a multiple of 16 (5120 rows on 256 CUs: 20 each).  A
+// wave belongs to one tile and to one share of the steps for its whole life, so its 16 x 16 accumulator never leaves
+// its registers: wave = tile * n_sub + sub, and the steps of a part are dealt in runs to the n_sub waves of a tile.
+// Lane (n, kg), n = lane % 16, kg = lane / 16, decodes strip kg (128 columns) of (row, block) pair n, word by word, exactly
 // as in ixh_strips358.hip: bitmap words and table entry into registers, ranks from popcounts (the strips of a unit are
 // 16 lanes apart: their counts travel through ds_bpermute), 16 stream bytes per word, v_alignbit, splice, pair table.
 //
@@ -17,18 +21,25 @@
 // fit beside the tables they are held one part of the columns at a time, and the workgroup walks the parts in turn
 // (a barrier, the next part's copy, a barrier).
 //
-// Elements above level 1 go to the wave's record queue and are resolved by the wave itself (it owns its tile) into a
-// 16-row array of its own.  At the end every wave stores its accumulators; after one barrier the outputs are summed
-// over the sub-ranges in order.  Every addition has a fixed place, apart from the order in which the LDS adds the lanes
-// of one instruction that hit the same sum.
+// Elements above level 1 go to the wave's record queue and are resolved by the wave itself (it owns its tile): 64 at a
+// time their weights are looked up lane by lane, then they go through the matrix pipe like the others (TileSink), into
+// the same accumulators.  At the end every wave stores its accumulators; after one barrier the outputs are summed over
+// the sub-ranges in order.  Every addition has a fixed place: a call gives the same bits every time.
 #include <math.h>
 
 #include "ixh_rows_common.h"
 
 namespace ixh {
 
+// ixh_set_option("gemv_tile_rows"): 0 = the planner's choice, 2 / 3 / 4 = tiles of 4 / 8 / 16 rows only
+extern std::atomic<int> g_opt_gemv_tile_rows;
+// ixh_set_option("gemv_tile_cus"): the number of CUs the planner spreads the rows over; 0 = the device's
+extern std::atomic<int> g_opt_gemv_tile_cus;
+
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kTMaxWaves = 16;
 constexpr uint32_t kTMaxRows = 128;  // rows per workgroup at most (8 tiles)
@@ -39,7 +50,7 @@ constexpr size_t kTLdsLimit = 160 * 1024;
 constexpr uint32_t kTStripBytes = 272;
 
 struct TilesLds {
-    uint32_t tq1, tq2, side, xs, xs_row, zero, partial, waves, wave_bytes, rare_off, tasks_off, total;
+    uint32_t tq1, tq2, side, xs, xs_row, zero, partial, waves, wave_bytes, tasks_off, total;
 };
 
 // x_blocks: column blocks of the activation rows that LDS holds at a time
@@ -54,22 +65,70 @@ __host__ __device__ inline TilesLds tiles_layout(uint32_t rows_cap, uint32_t n_c
     // bytes between activation rows: the padded strips, then 16 bytes so that the 16 rows a b128 read takes
     // start four banks apart
     L.xs_row = ((x_blocks * 4u * kTStripBytes + 127u) & ~127u) + 16u;
-    L.zero = L.xs + (uint32_t)m * L.xs_row;  // a strip of zeros: what the lanes of absent activation rows read
-    // [n_sub][rows_cap][m] fp32, the waves' accumulators at the end: over the activations, which nobody reads any more
-    // then (n_sub * rows_cap <= 256, so a row of them is shorter than a row of activations)
+    // [n_sub][rows_cap][m] fp32, the waves' accumulators at the end (n_sub: waves per tile x slots per wave): over the
+    // activations, which nobody reads any more then
     L.partial = L.xs;
+    const uint32_t partial_bytes = (n_sub * rows_cap * (uint32_t)m * 4u + 15u) & ~15u;
+    // a strip of zeros: what the lanes of absent activation rows read
+    L.zero = L.xs + max((uint32_t)m * L.xs_row, partial_bytes);
     L.waves = (L.zero + kTStripBytes + 15u) & ~15u;
-    L.rare_off = qcap * 16u;  // behind the queue: [16 rows][m] fp32 for the elements above level 1
-    L.tasks_off = L.rare_off + 16u * (uint32_t)m * 4u;
+    L.tasks_off = qcap * 16u;  // behind the queue
     L.wave_bytes = (L.tasks_off + kRTasks * 2u + 15u) & ~15u;
     L.total = L.waves + n_waves * L.wave_bytes;
     return L;
 }
 
+// The resolved elements above level 1 of a round go through the matrix pipe like the others, into the same
+// accumulators: every lane keeps its element's weight, the column n of the product it belongs to and the LDS address of
+// its activation in row 0; then, sixteen elements per instruction, lane (n, kg) fetches elements 4 kg .. 4 kg + 3 from
+// the lanes that hold them and gathers the activations of its row as one operand and, as the other, the weights of the
+// elements that belong to column n (zero for the rest).  Few registers are free where this runs: one pair at a time.
+struct TileSink {
+    static constexpr bool active = true;
+    f32x4 acc;           // the wave's accumulators: taken over for the time of the resolver, handed back after it
+    uint32_t n, kg;
+    uint32_t x_off;      // bytes from activation row 0 to the lane's activation row
+    bool x_on;           // that row exists
+    uint32_t idle_addr;  // an address that can be read
+    uint32_t wn, xa;     // the lane's element of the round: weight bits | column << 16, address
+    __device__ __forceinline__ void put(uint32_t w_bits, uint32_t row_field, uint32_t addr) {
+        wn = w_bits | ((row_field >> 12) << 16);
+        xa = addr;
+    }
+    __device__ __forceinline__ void idle() {
+        wn = 0u;
+        xa = idle_addr;
+    }
+    // lanes: the lanes below this number may hold an element
+    __device__ __forceinline__ void flush(uint32_t lanes) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            if ((uint32_t)g * 16u >= lanes) break;
+            uint32_t ap[2], bp[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int src = (int)(((uint32_t)g * 16u + kg * 4u + 2u * (uint32_t)h) * 4u);
+                const uint32_t e0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)wn);
+                const uint32_t e1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src + 4, (int)wn);
+                const uint32_t a0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)xa);
+                const uint32_t a1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src + 4, (int)xa);
+                const uint32_t x0 = lds_u16(a0 + x_off), x1 = lds_u16(a1 + x_off);
+                const uint32_t w0 = (e0 >> 16) == n ? (e0 & 0xFFFFu) : 0u, w1 = (e1 >> 16) == n ? e1 << 16 : 0u;
+                ap[h] = x_on ? (x0 | (x1 << 16)) : 0u;
+                bp[h] = w0 | w1;
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, u32x2{ap[0], ap[1]}),
+                                                           __builtin_bit_cast(s16x4, u32x2{bp[0], bp[1]}), acc, 0, 0, 0);
+        }
+    }
+};
+
 template <bool ANY>
 __global__ void __launch_bounds__(kTMaxWaves * kWave)
 k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t rows_per_wg, uint32_t n_sub,
-                uint32_t x_blocks, uint32_t qcap, uint32_t flags, const uint16_t *__restrict__ x, int m, int64_t ldx,
+                uint32_t x_blocks, uint32_t lg_rows, uint32_t qcap, uint32_t flags, const uint16_t *__restrict__ x,
+                int m, int64_t ldx,
                 uint16_t *__restrict__ y, int64_t ldy, float *__restrict__ y32) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
@@ -77,10 +136,14 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t n_waves = blockDim.x >> 6;
     const uint32_t n = lane & 15u, kg = lane >> 4;
+    // a tile is tile_rows = 4, 8 or 16 weight rows by 16 / tile_rows column blocks side by side: column n of the matrix
+    // instruction is weight row n % tile_rows in column block n / tile_rows of the step (its slot)
+    const uint32_t tile_rows = 1u << lg_rows, slots = 16u >> lg_rows;
+    const uint32_t r = n & (tile_rows - 1u), slot = n >> lg_rows;
 
     const uint32_t row0 = blockIdx.x * rows_per_wg;
     const uint32_t rows_here = min(rows_per_wg, P.out_f - row0), rows_cap = rows_per_wg;
-    const TilesLds L = tiles_layout(rows_cap, n_chunks, x_blocks, n_sub, n_waves, m, qcap);
+    const TilesLds L = tiles_layout(rows_cap, n_chunks, x_blocks, n_sub * slots, n_waves, m, qcap);
 
     // the pair table is addressed with (index bits | lane bits): it must sit at LDS address 0
     if ((uint32_t)(uintptr_t)(lds_ptr_t)smem != 0) {
@@ -96,7 +159,6 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     uint32_t *const tq2 = reinterpret_cast<uint32_t *>(smem + L.tq2);
     uint8_t *const wave_base = smem + L.waves + wave * L.wave_bytes;
     uint4 *const queue = reinterpret_cast<uint4 *>(wave_base);
-    float *const rare = reinterpret_cast<float *>(wave_base + L.rare_off);
     uint16_t *const tasks = reinterpret_cast<uint16_t *>(wave_base + L.tasks_off);
 
     const uint32_t unit0 = row0 * n_chunks;
@@ -112,32 +174,35 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
     // ---- this wave's tile and its share of the column blocks of a part ----
     const uint32_t tile = wave / n_sub, sub = wave - tile * n_sub;
-    const uint32_t trow0 = tile * 16u;
+    const uint32_t trow0 = tile << lg_rows;
     const bool tile_live = trow0 < rows_here;                      // a wave beyond the workgroup's rows has nothing to do
-    const bool live = trow0 + n < rows_here;                       // this lane's row exists
-    const uint32_t lrow = min(trow0 + n, rows_here - 1);           // clamped: a lane without a row decodes and is dropped
+    const bool row_live = trow0 + r < rows_here;                   // this lane's row exists
+    const uint32_t lrow = min(trow0 + r, rows_here - 1);           // clamped: a lane without a row decodes zeros
     const uint32_t n_parts = (n_chunks + x_blocks - 1) / x_blocks;
     uint32_t part_first = 0, part_count = min(x_blocks, n_chunks);  // the part's column blocks
     uint32_t c_begin = 0, c_end = 0;                                // this wave's run of them
-    auto take_share = [&]() {
-        const uint32_t base = part_count / n_sub, rem = part_count - base * n_sub;
-        c_begin = part_first + sub * base + min(sub, rem);
-        c_end = tile_live ? c_begin + base + (sub < rem ? 1u : 0u) : c_begin;
+    auto take_share = [&]() {  // in steps of `slots` column blocks
+        const uint32_t steps = (part_count + slots - 1u) >> (4u - lg_rows);
+        const uint32_t base = steps / n_sub, rem = steps - base * n_sub;
+        c_begin = min(part_first + part_count, part_first + ((sub * base + min(sub, rem)) << (4u - lg_rows)));
+        c_end = min(part_first + part_count, c_begin + ((base + (sub < rem ? 1u : 0u)) << (4u - lg_rows)));
+        if (!tile_live) c_end = c_begin;
     };
     take_share();
 
     // what a lane needs for one task (its tile x one column block): requested first, so that it travels early
     struct TaskIn {
-        uint32_t col;    // first column of the lane's strip
-        uint32_t strip;  // strip index in the part of the activation rows in LDS
+        uint32_t col;    // first column of the lane's strip; bit 31: the lane has no task (its row does not exist, or
+                         // its slot's column block lies past the wave's run)
         uint32_t q1u;    // rank table entry of the row's unit
         u32x4 bm;        // the four bitmap words of the lane's strip
     };
-    auto request = [&](uint32_t c, TaskIn &T) {
+    auto request = [&](uint32_t c0, TaskIn &T) {
+        const uint32_t c = min(c0 + slot, c_end - 1u);  // clamped: a lane without a block reads what exists
         T.col = c * kFastChunk + kg * 128u;
-        T.strip = (c - part_first) * 4u + kg;
         T.q1u = __builtin_amdgcn_raw_buffer_load_b32(tb_rsrc, (int)((unit0 + lrow * n_chunks + c) * 4u), 0, 0);
         T.bm = __builtin_amdgcn_raw_buffer_load_b128(b1_rsrc, (int)((((row0 + lrow) * P.in_f + T.col) >> 5) * 4u), 0, 0);
+        if (!row_live || c0 + slot >= c_end) T.col |= 0x80000000u;
     };
     TaskIn T;
     if (c_begin < c_end) request(c_begin, T);
@@ -146,7 +211,9 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     // activation rows of the part's columns into padded strips: 16-byte piece p of row i holds columns 8p .. 8p+7
     auto load_activations = [&]() {
         const uint32_t pieces = part_count * (kFastChunk / 8), first_piece = part_first * (kFastChunk / 8);
-        for (uint32_t t = tid; t < (uint32_t)m * pieces; t += blockDim.x) {
+        uint32_t t0 = threadIdx.x;
+        asm volatile("" : "+v"(t0));  // worked out anew at every call: no register is held for it across the loop
+        for (uint32_t t = t0; t < (uint32_t)m * pieces; t += blockDim.x) {
             const uint32_t i = t / pieces, p = t - i * pieces;
             const uint4 v = *reinterpret_cast<const uint4 *>(x + (int64_t)i * ldx + (first_piece + p) * 8u);
             *reinterpret_cast<uint4 *>(smem + L.xs + i * L.xs_row + (p >> 4) * kTStripBytes + (p & 15u) * 16u) = v;
@@ -217,29 +284,36 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         splice[2 * tid] = make_uint4(lm[0], lm[1], lm[2], 0u);
         splice[2 * tid + 1] = make_uint4(f[0], f[1], f[2], 0u);
     }
-    for (uint32_t t = lane; t < 16u * (uint32_t)m; t += kWave) rare[t] = 0.0f;
 
     const uint32_t lut_lane = (lane & 31u) << 2;
     const uint32_t splice_addr = kRLutBytes;
     const uint32_t tq1_addr = L.tq1, tq2_addr = L.tq2;
-    // the resolver adds into rowacc + (local row * m + activation row) * 4: the wave's 16-row array, shifted by its tile
-    const uint32_t rare_addr = (uint32_t)(uintptr_t)(lds_ptr_t)rare - trow0 * (uint32_t)m * 4u;
     const uint32_t xs_addr = L.xs;
-    // lane n of each k group feeds activation row n (absent rows read zeros)
-    const bool x_real = n < (uint32_t)m;
-    const uint32_t x_lane = x_real ? L.xs + n * L.xs_row : L.zero;
+    // as row n of the other operand, lane n of each k group feeds activation row n % tile_rows at the columns of its
+    // own slot's block (absent activation rows read zeros): the product of row a and column n of the operands means
+    // something where their slots agree
+    const uint32_t x_lane = r < (uint32_t)m ? L.xs + r * L.xs_row : L.zero;
+    const uint32_t x_step = r < (uint32_t)m ? kTStripBytes : 0u;  // bytes from strip to strip
+
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};  // D[4 kg + i][n]: activation rows 4 kg .. 4 kg + 3 x this lane's weight row
 
     uint32_t qcount = 0;  // wave-uniform
     auto resolve = [&]() {
+        TileSink sink{acc, n, kg, r * L.xs_row, r < (uint32_t)m, xs_addr, 0u, xs_addr};
+        const TaskPool none{0, 0, 0, 1, 0, 0};
         if (ANY)
-            resolve_rows<kTMaxM, false, true, 2, false, kTStripBytes>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rare_addr, tasks, xs_addr,
-                                                L.xs_row, part_first * kFastChunk, m, scale, lane, prefix, entries);
+            resolve_rows_to<kTMaxM, false, true, 2, false, kTStripBytes>(
+                sink, P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, 0u, tasks, xs_addr, L.xs_row,
+                part_first * kFastChunk, m, scale, lane, prefix, entries, none);
         else if (sv.staged)
-            resolve_rows<kTMaxM, true, false, 2, false, kTStripBytes>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rare_addr, tasks, xs_addr,
-                                                L.xs_row, part_first * kFastChunk, m, scale, lane);
+            resolve_rows_to<kTMaxM, true, false, 2, false, kTStripBytes>(
+                sink, P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, 0u, tasks, xs_addr, L.xs_row,
+                part_first * kFastChunk, m, scale, lane, nullptr, 0, none);
         else
-            resolve_rows<kTMaxM, false, false, 2, false, kTStripBytes>(P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, rare_addr, tasks,
-                                                 xs_addr, L.xs_row, part_first * kFastChunk, m, scale, lane);
+            resolve_rows_to<kTMaxM, false, false, 2, false, kTStripBytes>(
+                sink, P, sv, tq1_addr, tq2_addr, unit0, queue, qcount, 0u, tasks, xs_addr, L.xs_row,
+                part_first * kFastChunk, m, scale, lane, nullptr, 0, none);
+        acc = sink.acc;
         qcount = 0;
     };
 
@@ -263,17 +337,19 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     // A task in flight: the ranks at which its words start and the stream bytes asked for with them.
     struct Stage {
         uint32_t word[4];  // bitmap words
-        uint32_t rank[4];  // level-1 elements before each word (global rank)
+        uint32_t first;    // level-1 elements before the strip's first word (global rank)
         u32x4 code[4];     // the 16 stream bytes that hold each word's codes (address = 3 x rank)
-        uint32_t col, x_strip;
+        uint32_t col;      // as in TaskIn
+        uint32_t records;  // wave-uniform: lanes x words with elements above level 1, the records the task will queue
     };
     // second step of a task: from table entry and bitmap words to the ranks, and the requests for the codes
     auto launch_codes = [&](const TaskIn &T, Stage &S) {
         S.col = T.col;
-        S.x_strip = x_lane + (x_real ? T.strip * kTStripBytes : 0u);
         u32x4 b = T.bm;
-        if (!live) b = u32x4{~0u, ~0u, ~0u, ~0u};  // a lane without a row decodes what it finds and is dropped
+        if ((int)T.col < 0) b = u32x4{~0u, ~0u, ~0u, ~0u};  // a lane without a task: no records, and zero codes below
         S.word[0] = b.x; S.word[1] = b.y; S.word[2] = b.z; S.word[3] = b.w;
+        S.records = (uint32_t)(__popcll(__ballot(b.x != ~0u)) + __popcll(__ballot(b.y != ~0u)) +
+                               __popcll(__ballot(b.z != ~0u)) + __popcll(__ballot(b.w != ~0u)));
         const uint32_t p1 = __popc(b.x), p2 = p1 + __popc(b.y), p3 = p2 + __popc(b.z), p4 = p3 + __popc(b.w);
         // level-1 elements of the unit's strips before this one: they are 16, 32 and 48 lanes down
         const uint32_t d1 = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((lane - 16u) * 4u), (int)p4);
@@ -281,20 +357,23 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         const uint32_t d3 = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((lane - 48u) * 4u), (int)p4);
         const uint32_t before = (kg >= 1 ? d1 : 0u) + (kg >= 2 ? d2 : 0u) + (kg >= 3 ? d3 : 0u);
         const uint32_t first = T.q1u + before;
-        S.rank[0] = first; S.rank[1] = first + p1; S.rank[2] = first + p2; S.rank[3] = first + p3;
+        S.first = first;
+        const uint32_t rank[4] = {first, first + p1, first + p2, first + p3};
 #pragma unroll
         for (int k = 0; k < 4; ++k)
-            S.code[k] = __builtin_amdgcn_raw_buffer_load_b128(l1_rsrc, (int)(((S.rank[k] * 3u) >> 5) * 4u), 0, 0);
+            S.code[k] = __builtin_amdgcn_raw_buffer_load_b128(l1_rsrc, (int)(((rank[k] * 3u) >> 5) * 4u), 0, 0);
     };
-
-    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};  // D[4 kg + i][n]: activation rows 4 kg .. 4 kg + 3 x this lane's weight row
 
     // third step: decode and multiply the task's words
     auto compute = [&](Stage &S) {
+        // the lane's strip of its activation row in LDS
+        const uint32_t x_strip = x_lane + (((S.col & 0x7FFFFFFFu) >> 7) - part_first * 4u) * x_step;
+        // a lane without a task looks up pair (7, 7) whatever it decodes: the table's zero
+        const uint32_t lut_x = lut_lane | ((uint32_t)((int)S.col >> 31) & 0x1F80u);
+        uint32_t rk = S.first;  // level-1 elements before the word
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const u32x4 dq = S.code[k];
-            const uint32_t rk = S.rank[k];
             const uint32_t off = rk * 3u;  // v_alignbit takes the low five bits
             uint32_t w0 = __builtin_amdgcn_alignbit(dq.y, dq.x, off);
             uint32_t w1 = __builtin_amdgcn_alignbit(dq.z, dq.y, off);
@@ -302,40 +381,45 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
             uint32_t zrem = ~S.word[k];
             const uint64_t any = __ballot(zrem != 0);
             if (any != 0) {  // lanes with elements above level 1 leave a record
-                if (qcount > qcap - kWave) resolve();
                 if (zrem != 0) {
                     const uint32_t kcol = S.col + 32u * (uint32_t)k;
                     const uint32_t unit = unit0 + lrow * n_chunks + (S.col >> 9);
                     const uint32_t r0 = (row0 + lrow) * P.in_f + kcol - rk;
-                    push_record(queue, qcount + lanes_below(any), make_uint4(zrem, r0, unit, (lrow << 16) | kcol));
+                    push_record(queue, qcount + lanes_below(any), make_uint4(zrem, r0, unit, (n << 28) | (lrow << 16) | kcol));
                 }
                 qcount += (uint32_t)__popcll(any);
                 do splice_once(w0, w1, w2, zrem);
                 while (__ballot(zrem != 0) != 0);
             }
-            // the word's activations: four steps of eight columns
-            u32x4 xa[4];
+            // sixteen code pairs through the pair table and the word's activations, eight columns per matrix
+            // instruction; in two halves, so that a half's operands are all that is in registers at a time
 #pragma unroll
-            for (int s = 0; s < 4; ++s) xa[s] = lds_u128(S.x_strip + (uint32_t)k * 64u + (uint32_t)s * 16u);
-            // sixteen code pairs through the pair table, eight weights per matrix instruction
-            uint32_t wp[16];
+            for (int half = 0; half < 2; ++half) {
+                u32x4 xa[2];
 #pragma unroll
-            for (int t = 0; t < 16; ++t) {
-                const int bit = 6 * t, ob = bit & 31, dd = bit >> 5;
-                const uint32_t lo = dd == 0 ? w0 : (dd == 1 ? w1 : w2);
-                const uint32_t hi = dd == 0 ? w1 : w2;
-                uint32_t a;  // pair index at bits 12..7
-                if (ob > 26) a = __builtin_amdgcn_alignbit(hi, lo, ob - 7);
-                else if (ob >= 7) a = lo >> (ob - 7);
-                else a = lo << (7 - ob);
-                wp[t] = lds_u32((a & 0x1F80u) | lut_lane);
+                for (int s = 0; s < 2; ++s)
+                    xa[s] = lds_u128(x_strip + (uint32_t)k * 64u + (uint32_t)(2 * half + s) * 16u);
+                uint32_t wp[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int bit = 6 * (8 * half + u), ob = bit & 31, dd = bit >> 5;
+                    const uint32_t lo = dd == 0 ? w0 : (dd == 1 ? w1 : w2);
+                    const uint32_t hi = dd == 0 ? w1 : w2;
+                    uint32_t a;  // pair index at bits 12..7
+                    if (ob > 26) a = __builtin_amdgcn_alignbit(hi, lo, ob - 7);
+                    else if (ob >= 7) a = lo >> (ob - 7);
+                    else a = lo << (7 - ob);
+                    wp[u] = lds_u32((a & 0x1F80u) | lut_x);
+                }
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const u32x4 b4 = u32x4{wp[4 * s], wp[4 * s + 1], wp[4 * s + 2], wp[4 * s + 3]};
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[s]),
+                                                                 __builtin_bit_cast(bf16x8, b4), acc, 0, 0, 0);
+                }
+                if (half == 0) __builtin_amdgcn_sched_barrier(0);
             }
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const u32x4 b4 = u32x4{wp[4 * s], wp[4 * s + 1], wp[4 * s + 2], wp[4 * s + 3]};
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[s]),
-                                                             __builtin_bit_cast(bf16x8, b4), acc, 0, 0, 0);
-            }
+            rk += (uint32_t)__popc(S.word[k]);
         }
     };
 
@@ -345,17 +429,21 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         if (c_begin < c_end) {
             Stage A, B;
             launch_codes(T, A);
-            if (c_begin + 1 < c_end) request(c_begin + 1, T);
-            for (uint32_t c = c_begin; c < c_end; c += 2) {
-                if (c + 1 < c_end) {
+            if (c_begin + slots < c_end) request(c_begin + slots, T);
+            // The queue is emptied between tasks, where one stage is dead and registers are free: before a task whose
+            // records (at most 4 x 64 = the queue's capacity) would not fit behind those that wait.
+            for (uint32_t c = c_begin; c < c_end; c += 2 * slots) {
+                if (qcount + A.records > qcap) resolve();
+                if (c + slots < c_end) {
                     launch_codes(T, B);
-                    if (c + 2 < c_end) request(c + 2, T);
+                    if (c + 2 * slots < c_end) request(c + 2 * slots, T);
                 }
                 compute(A);
-                if (c + 1 < c_end) {
-                    if (c + 2 < c_end) {
+                if (c + slots < c_end) {
+                    if (qcount + B.records > qcap) resolve();
+                    if (c + 2 * slots < c_end) {
                         launch_codes(T, A);
-                        if (c + 3 < c_end) request(c + 3, T);
+                        if (c + 3 * slots < c_end) request(c + 3 * slots, T);
                     }
                     compute(B);
                 }
@@ -364,7 +452,7 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         if (++part == n_parts) break;
         // the next part of the columns: this part's elements above level 1 meet its activations while they are there
         resolve();
-        part_first = part * x_blocks;
+        part_first = (uint32_t)__builtin_amdgcn_readfirstlane((int)(part * x_blocks));
         part_count = min(x_blocks, n_chunks - part_first);
         take_share();
         if (c_begin < c_end) request(c_begin, T);
@@ -377,24 +465,33 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     // ---- the wave's accumulators into the sub-range's slot; after the barrier the outputs are summed over the
     // sub-ranges, each with what its wave added for the elements above level 1 ----
     __syncthreads();  // the accumulators go where the activations were
-    if (live) {
-        float *const partial = reinterpret_cast<float *>(smem + L.partial) + (sub * rows_cap + trow0 + n) * (uint32_t)m;
+    {
+        // the lane holds rows 4 kg .. 4 kg + 3 of the product's column n: those of its own slot are the sums of
+        // activation rows (4 kg + i) % tile_rows.  The lane's place is worked out anew (from a lane number the
+        // compiler cannot connect with the one above), so that no register carries it through the kernel.
+        uint32_t l2 = threadIdx.x & 63u;
+        asm volatile("" : "+v"(l2));
+        const uint32_t n2 = l2 & 15u, kg2 = l2 >> 4, r2 = n2 & (tile_rows - 1u), slot2 = n2 >> lg_rows;
+        if (trow0 + r2 < rows_here) {
+            float *const partial = reinterpret_cast<float *>(smem + L.partial) +
+                                   ((sub * slots + slot2) * rows_cap + trow0 + r2) * (uint32_t)m;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (4u * kg + i < (uint32_t)m) partial[4u * kg + i] = acc[i];
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t a = 4u * kg2 + i, j = a & (tile_rows - 1u);
+                if ((a >> lg_rows) == slot2 && j < (uint32_t)m) partial[j] = acc[i];
+            }
+        }
     }
     __syncthreads();
     for (uint32_t t = tid; t < rows_here * (uint32_t)m; t += blockDim.x) {
-        const uint32_t slot = t / (uint32_t)m, i = t - slot * (uint32_t)m;
-        const uint32_t tl = slot >> 4;
+        const uint32_t row = t / (uint32_t)m, i = t - row * (uint32_t)m;
         float sum = 0.0f;
         for (uint32_t s = 0; s < n_sub; ++s) {
-            sum += reinterpret_cast<const float *>(smem + L.partial)[(s * rows_cap + slot) * (uint32_t)m + i];
-            sum += reinterpret_cast<const float *>(smem + L.waves + (tl * n_sub + s) * L.wave_bytes + L.rare_off)
-                       [(slot & 15u) * (uint32_t)m + i];
+            for (uint32_t q = 0; q < slots; ++q)
+                sum += reinterpret_cast<const float *>(smem + L.partial)[((s * slots + q) * rows_cap + row) * (uint32_t)m + i];
         }
-        if (y32) atomicAdd(&y32[(size_t)i * P.out_f + row0 + slot], sum);
-        else y[(int64_t)i * ldy + row0 + slot] = (uint16_t)f32_to_bf16_bits(sum);
+        if (y32) atomicAdd(&y32[(size_t)i * P.out_f + row0 + row], sum);
+        else y[(int64_t)i * ldy + row0 + row] = (uint16_t)f32_to_bf16_bits(sum);
     }
 }
 
@@ -402,35 +499,54 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 // host side
 // ---------------------------------------------------------------------------
 struct TilesPlan {
-    uint32_t rows, n_sub, x_blocks, qcap, waves;
+    uint32_t rows, n_sub, x_blocks, qcap, waves, lg_rows;
+    float cost;
 };
 
-// Rows per workgroup (whole rounds of one workgroup per CU, a multiple of four), waves per tile and the part of the
-// activation rows LDS holds at a time.  Every part costs the workgroup two barriers and a copy, every missing wave
-// costs latency that nobody covers: the plan with the fewest parts among those with ten waves or more, else the one
-// with the most waves.
-static TilesPlan plan_tiles(uint32_t out_f, uint32_t n_chunks, uint32_t n_cu, int m) {
+// Rows per workgroup (whole rounds of one workgroup per CU, a multiple of four), the tile shape, waves per tile and the
+// part of the activation rows that LDS holds at a time.  A tile of 16 >> k rows takes 1 << k column blocks per step and
+// serves 16 >> k activation rows, so short tiles suit workgroups whose rows are not a multiple of 16 when the rows of
+// activations are few.  A wave's time goes with the steps it decodes, and every further part costs two barriers and a
+// copy whose latency nobody covers: the plan with the fewest steps per wave, a part counted as a third of a step
+// (costs that also count the steps of all waves of a CU, or of a SIMD, chose slower plans on the shapes measured).
+static TilesPlan plan_tiles(uint32_t out_f, uint32_t n_chunks, uint32_t n_cu, int m, int lg_only) {
     const uint32_t n_quads = (out_f + 3) / 4, max_quads = kTMaxRows / 4;
     const uint32_t rounds = (n_quads + n_cu * max_quads - 1) / (n_cu * max_quads);
     const uint32_t rows = 4u * max(1u, min(max_quads, (n_quads + rounds * n_cu - 1) / (rounds * n_cu)));
-    const uint32_t tiles = (rows + 15) / 16;
-    TilesPlan best{0, 0, 0, 0, 0};
-    for (uint32_t parts = 1; parts <= n_chunks; ++parts) {
-        const uint32_t x_blocks = (n_chunks + parts - 1) / parts;
-        if ((n_chunks + x_blocks - 1) / x_blocks != parts) continue;  // the same parts with fewer blocks each: seen
-        TilesPlan here{0, 0, 0, 0, 0};
-        for (uint32_t n_sub = min((uint32_t)kTMaxWaves / tiles, x_blocks); n_sub >= 1 && here.waves == 0; --n_sub) {
-            for (uint32_t qcap : {256u, 128u}) {
-                if (tiles_layout(rows, n_chunks, x_blocks, n_sub, tiles * n_sub, m, qcap).total > kTLdsLimit) continue;
-                // no more waves than shorten the longest run of blocks
-                const uint32_t run = (x_blocks + n_sub - 1) / n_sub;
-                const uint32_t subs = (x_blocks + run - 1) / run;
-                here = TilesPlan{rows, subs, x_blocks, qcap, tiles * subs};
-                break;
+    TilesPlan best{0, 0, 0, 0, 0, 4, 0.0f};
+    for (uint32_t lg = 4; lg >= 2; --lg) {
+        if (lg_only >= 2 && (uint32_t)lg_only != lg) continue;
+        const uint32_t tile_rows = 1u << lg, slots = 16u >> lg;
+        if ((uint32_t)m > tile_rows) break;
+        const uint32_t tiles = (rows + tile_rows - 1) / tile_rows;
+        if (tiles > (uint32_t)kTMaxWaves) continue;
+        for (uint32_t parts = 1; parts <= n_chunks; ++parts) {
+            const uint32_t x_blocks = (n_chunks + parts - 1) / parts;
+            if ((n_chunks + x_blocks - 1) / x_blocks != parts) continue;  // the same parts with fewer blocks each: seen
+            const uint32_t steps = (x_blocks + slots - 1) / slots;  // of the longest part
+            TilesPlan here{0, 0, 0, 0, 0, lg, 0.0f};
+            for (uint32_t n_sub = min((uint32_t)kTMaxWaves / tiles, steps); n_sub >= 1 && here.waves == 0; --n_sub) {
+                for (uint32_t qcap : {256u}) {  // a task's records must fit: 4 words x 64 lanes
+                    if (tiles_layout(rows, n_chunks, x_blocks, n_sub * slots, tiles * n_sub, m, qcap).total > kTLdsLimit)
+                        continue;
+                    // no more waves than shorten the longest run of steps
+                    const uint32_t run = (steps + n_sub - 1) / n_sub;
+                    const uint32_t subs = (steps + run - 1) / run;
+                    uint32_t per_wave = 0;
+                    for (uint32_t first = 0; first < n_chunks; first += x_blocks) {
+                        const uint32_t st = (min(x_blocks, n_chunks - first) + slots - 1) / slots;
+                        per_wave += (st + subs - 1) / subs;
+                    }
+                    here = TilesPlan{rows, subs, x_blocks, qcap, tiles * subs, lg,
+                                     (float)per_wave + (float)(parts - 1) / 3.0f};
+                    break;
+                }
             }
+            if (here.waves != 0 && (best.waves == 0 || here.cost < best.cost)) best = here;
+            if (here.waves != 0 && here.waves >= tiles * min((uint32_t)kTMaxWaves / tiles, steps) && parts > 1 &&
+                here.cost > best.cost)
+                break;  // more parts only add to the cost from here on
         }
-        if (here.waves > best.waves) best = here;
-        if (best.waves >= 10u || best.waves >= tiles * min((uint32_t)kTMaxWaves / tiles, n_chunks)) break;
     }
     return best;
 }
@@ -443,12 +559,13 @@ static int launch_tiles(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTLdsLimit) == hipSuccess;
     if (!raised) return IXH_EUNSUPPORTED;
     const uint32_t groups = (P.out_f + plan.rows - 1) / plan.rows;
-    const size_t lds = tiles_layout(plan.rows, n_chunks, plan.x_blocks, plan.n_sub, plan.waves, m, plan.qcap).total;
+    const size_t lds =
+        tiles_layout(plan.rows, n_chunks, plan.x_blocks, plan.n_sub * (16u >> plan.lg_rows), plan.waves, m, plan.qcap).total;
     if (lds > kTLdsLimit) return IXH_EUNSUPPORTED;
     uint32_t flags = 0;
     if (((uintptr_t)P.last & 3u) == 0) flags |= kFlagStageSide;
     hipLaunchKernelGGL((k_gemv358_tiles<ANY>), dim3(groups), dim3(plan.waves * kWave), lds, s, P, prefix, n_chunks,
-                       plan.rows, plan.n_sub, plan.x_blocks, plan.qcap, flags, x, m, ldx, y, ldy, y32);
+                       plan.rows, plan.n_sub, plan.x_blocks, plan.lg_rows, plan.qcap, flags, x, m, ldx, y, ldy, y32);
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }
 
@@ -467,11 +584,15 @@ int launch_gemv_358_tiles(const Dev &P, const int32_t *prefix, const uint16_t *x
         return v;
     }();
     const uint32_t n_chunks = P.in_f / kFastChunk;
-    const TilesPlan plan = plan_tiles(P.out_f, n_chunks, (uint32_t)n_cu, m);
+    const int cus_opt = g_opt_gemv_tile_cus.load(std::memory_order_relaxed);
+    const TilesPlan plan = plan_tiles(P.out_f, n_chunks, (uint32_t)(cus_opt > 0 ? cus_opt : n_cu), m,
+                                      g_opt_gemv_tile_rows.load(std::memory_order_relaxed));
     if (plan.waves == 0) return IXH_EUNSUPPORTED;
     // by itself from three activation rows on (one or two: the kernels that multiply lane by lane are as fast or faster)
     // and where a workgroup's rows fill its tiles of 16 at least half; forced (option 1) wherever it fits
-    if (opt == 0 && (m <= 2 || plan.rows * 2u < ((plan.rows + 15u) / 16u) * 16u)) return IXH_EUNSUPPORTED;
+    const uint32_t tile_rows = 1u << plan.lg_rows;
+    if (opt == 0 && (m <= 2 || plan.rows * 2u < ((plan.rows + tile_rows - 1u) / tile_rows) * tile_rows))
+        return IXH_EUNSUPPORTED;
     return any ? launch_tiles<true>(P, prefix, n_chunks, plan, x, m, ldx, y, ldy, y32, s)
                : launch_tiles<false>(P, prefix, n_chunks, plan, x, m, ldx, y, ldy, y32, s);
 }

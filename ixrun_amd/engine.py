@@ -30,14 +30,13 @@ __all__ = ["Int8XEngine", "StreamingLinear", "GraphLinear", "ResourceScheduler"]
 MAX_FUSED_ROWS = 16  # activation rows served by the fused decode+GEMV kernel
 # With a decode buffer at hand, more rows than this go through decode + library GEMM.  Tensors that are almost all
 # level 1, MI355X: the pair takes 72-75 us on 17408 x 5120 and 5120 x 17408 at any M up to 32 and 34-50 us on
-# 5120 x 5120; the fused kernels take 31 / 35 / 41 us (17408 x 5120), 39 / 46 / 60 us (5120 x 17408) and 38 / 51 / 63 us
-# (5120 x 5120) at M = 8 / 12 / 16: up to 8 rows everywhere, up to 16 on the large layers.  Dense mixes (55 / 40 / 5 %):
-# the pair takes 84-90 us, the fused kernels 55-62 / 69-72 / 85-88 / 116-119 us at M = 1 / 2 / 4 / 8.  Dense mixes in
-# other schemes have a level-by-level kernel for one row only (five levels: 95-104 us; the pair 127 us, the any-scheme
-# kernel 209-260 us at M = 2 .. 8).
-MAX_FUSED_ROWS_WITH_BUFFER = 8
-MAX_FUSED_ROWS_WITH_BUFFER_LARGE = 16
-LARGE_LAYER_ELEMENTS = 64 * 1024 * 1024
+# 5120 x 5120 (five levels: 73-74 and 38-39 us); the fused kernels take 30 / 31 / 34 us (17408 x 5120), 40 / 44 / 54 us
+# (5120 x 17408) and 24 / 24 / 25 us (5120 x 5120) at M = 8 / 12 / 16 (five levels: 33 / 33 / 37, 45 / 50 / 59 and
+# 30 / 31 / 32 us): every row count the fused kernels take.  Dense mixes (55 / 40 / 5 %): the pair takes 84-90 us, the
+# fused kernels 55-62 / 69-72 / 85-88 / 116-119 us at M = 1 / 2 / 4 / 8.  Dense mixes in other schemes have a
+# level-by-level kernel for one row only (five levels: 95-104 us; the pair 127 us, the any-scheme kernel 209-260 us at
+# M = 2 .. 8).
+MAX_FUSED_ROWS_WITH_BUFFER = 16
 MAX_FUSED_ROWS_WITH_BUFFER_DENSE = 4
 # More rows than that: with a shared decode buffer the layer decodes into it and calls the library GEMM
 # (5120 x 5120 five-level on MI355X: 60 us at 32 rows, 84 us at 512); without one it runs the fused
@@ -139,8 +138,7 @@ class StreamingLinear(nn.Module):
         if self._w_buf is None:
             fused_rows = MAX_FUSED_ROWS
         elif self.counts[0] * 100 >= self.N * 97:
-            large = self.N >= LARGE_LAYER_ELEMENTS and self.level_bits == (3, 5, 8)
-            fused_rows = MAX_FUSED_ROWS_WITH_BUFFER_LARGE if large else MAX_FUSED_ROWS_WITH_BUFFER
+            fused_rows = MAX_FUSED_ROWS_WITH_BUFFER
         elif self.level_bits == (3, 5, 8):
             fused_rows = MAX_FUSED_ROWS_WITH_BUFFER_DENSE
         else:

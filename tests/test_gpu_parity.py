@@ -337,6 +337,34 @@ def test_gemv_strip_and_tile_kernels(oracle, dev, gemv_option, kind, shape, leve
 
 
 @pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("shape", [(20, 512), (36, 1024), (68, 5120), (132, 1536), (100, 8704), (48, 17408)])
+@pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8)])
+@pytest.mark.parametrize("tile_rows", [4, 8, 16])
+@pytest.mark.parametrize("cus", [1, 3])
+def test_gemv_tile_shapes(oracle, dev, gemv_option, kind, shape, level_bits, tile_rows, cus):
+    """The tile kernel with each of its tile shapes forced (4, 8 or 16 weight rows by 4, 2 or 1 column blocks side by
+    side; a shape that cannot serve that many activation rows hands the call on to the next kernel), the rows spread
+    over one and over three CUs so that a workgroup holds several tiles, a last tile with rows missing, steps whose last
+    slots have no column block, activations held in LDS one part of the columns at a time, queues that are emptied
+    between tasks (dense mixes), every element above level 1 through the matrix pipe."""
+    from ixrun_amd import _lib
+
+    out_f, in_f = shape
+    p = make_packed(kind, out_f, in_f, level_bits)
+    dp = device_packed(p, dev)
+    w_bits = oracle.decode_packed_bf16(p)
+    gemv_option("gemv_tiles", 1)
+    gemv_option("gemv_tile_rows", {4: 2, 8: 3, 16: 4}[tile_rows])
+    gemv_option("gemv_tile_cus", cus)
+    for m in (1, 2, 3, 4, 5, 8, 11, 16):
+        x = activations(m, in_f, seed=m)
+        y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
+        for atomic in (False, True):
+            y = run_gemv(dp, 512, x, m, dev, flags=_lib.IXH_GEMV_FORCE_358, atomic=atomic)
+            check_outputs(y, y64, f"tiles of {tile_rows} on {cus} CUs {kind} {shape} {level_bits} m={m} atomic={atomic}")
+
+
+@pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("shape", [(64, 512), (37, 1024), (130, 2048), (24, 8704), (5, 25600)])
 @pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8), (5, 8)])
 def test_gemv_staged(oracle, dev, kind, shape, level_bits):
@@ -420,17 +448,23 @@ def test_gemv_one_hot_is_exact(oracle, dev, kind):
 
 
 @pytest.mark.parametrize("kind", ["student_t", "rare_other"])
-@pytest.mark.parametrize("kernel", ["strips", "tiles"])
+@pytest.mark.parametrize("kernel", ["strips", "tiles", "tiles of 8", "tiles of 4"])
 def test_gemv_matrix_pipe_kernels_one_hot_is_exact(oracle, dev, gemv_option, kind, kernel):
     """One-hot activation rows through the strip and the tile kernel: every output equals a decoded weight, exactly
-    (the matrix pipe multiplies by 1.0 and adds zeros)."""
+    (the matrix pipe multiplies by 1.0 and adds zeros; the elements above level 1 take the same way)."""
     out_f, in_f = 96, 1024
     p = make_packed(kind, out_f, in_f)
     dp = device_packed(p, dev)
     w_want = oracle.decode_packed_bf16(p)
     gemv_option("gemv_strips", 1)
-    gemv_option("gemv_tiles", 1 if kernel == "tiles" else -1)
+    gemv_option("gemv_tiles", 1 if kernel.startswith("tiles") else -1)
+    gemv_option("gemv_tile_rows", {"tiles of 8": 3, "tiles of 4": 2}.get(kernel, 0))
+    gemv_option("gemv_tile_cus", 2 if kernel.startswith("tiles of") else 0)
     cols = (0, 3, 4, 7, 8, 31, 32, 127, 128, 511, 512, 1023)
+    if kernel == "tiles of 8":
+        cols = cols[:8]
+    if kernel == "tiles of 4":
+        cols = cols[8:]
     x = torch.zeros(len(cols), in_f, dtype=torch.bfloat16)
     for i, k in enumerate(cols):
         x[i, k] = 1.0
