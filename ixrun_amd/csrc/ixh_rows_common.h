@@ -78,6 +78,16 @@ struct SideView {
 // what keeps the compiler from putting "wait for every LDS-DMA copy in flight" (s_waitcnt vmcnt(0)) in front
 // of an LDS access that has nothing to do with the ring the copies land in.
 __device__ __forceinline__ void push_record(uint4 *__restrict__ q, uint32_t idx, uint4 v) { q[idx] = v; }
+// the 8-byte records of a kernel with a sink (resolve_rows_to), in the same queue
+__device__ __forceinline__ void push_record8(uint4 *__restrict__ q, uint32_t idx, uint32_t word, uint32_t packed) {
+    reinterpret_cast<uint2 *>(q)[idx] = make_uint2(word, packed);
+}
+template <bool COMPACT>
+__device__ __forceinline__ uint4 read_record(const uint4 *__restrict__ q, uint32_t idx) {
+    if (!COMPACT) return q[idx];
+    const uint2 v = reinterpret_cast<const uint2 *>(q)[idx];
+    return make_uint4(v.x, v.y, 0u, 0u);
+}
 
 // Two LDS operations issued outside the compiler's memory model, for the code that runs while the wave has
 // LDS-DMA copies in flight: in front of a merged two-word LDS read and of an LDS atomic the compiler puts
@@ -128,8 +138,11 @@ struct TaskPool {
 // weight's bf16 bits, the record's row field and the LDS address of the element's column in the first activation
 // row, idle() is called by the lanes that have no element in a round, and flush() by the whole wave after every
 // round of at most 64 elements (its argument: the lanes below that number may have taken part).
+// A sink also brings its own record format: 8 bytes, the bitmap word and a word that unpack() turns into the
+// fields of the 16-byte record (rank of the word's first element in bitmap 1's domain, unit, column, row field).
 struct NoSink {
     static constexpr bool active = false;
+    __device__ __forceinline__ void unpack(uint32_t, uint32_t, uint32_t, uint32_t &, uint32_t &, uint32_t &, uint32_t &) {}
     __device__ __forceinline__ void put(uint32_t, uint32_t, uint32_t) {}
     __device__ __forceinline__ void idle() {}
     __device__ __forceinline__ void flush(uint32_t) {}
@@ -179,7 +192,8 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
     // element `e` (bit of the record's word), the nth element above level 1 of its record
     auto one = [&](const uint4 rec, uint32_t nth, uint32_t e) {
         uint32_t r0_lane = rec.y, unit = rec.z, k0 = rec.w & 0xFFFFu;
-        const uint32_t slot = rec.w >> 16;
+        uint32_t slot = rec.w >> 16;
+        if (SINK::active) sink.unpack(rec.y, unit0, tq1_addr, r0_lane, unit, k0, slot);
         if (XL == 1) {  // the shared-x kernel's records: rank offset in the unit, LDS address of the unit's table
                     // entry, column block << 4 | lane
             const uint32_t in_unit = (rec.w & 15u) * 32u;
@@ -281,7 +295,7 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
         const uint32_t idx = base + lane;
         const bool has = idx < count;
         uint4 rec = make_uint4(0, 0, 0, 0);
-        if (has) rec = queue[idx];
+        if (has) rec = read_record<SINK::active>(queue, idx);
         uint32_t zeros = rec.x;
         const uint32_t mine = (uint32_t)__popc(zeros);
         const uint32_t incl = wave_scan(mine);
@@ -295,7 +309,7 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
             for (uint32_t tb = 0; tb < n_tasks; tb += kWave) {
                 if (tb + lane < n_tasks) {
                     const uint32_t task = tasks[tb + lane];
-                    one(queue[base + (task >> 10)], (task >> 5) & 31u, task & 31u);
+                    one(read_record<SINK::active>(queue, base + (task >> 10)), (task >> 5) & 31u, task & 31u);
                 } else if (SINK::active) {
                     sink.idle();
                 }

@@ -72,7 +72,7 @@ __host__ __device__ inline TilesLds tiles_layout(uint32_t rows_cap, uint32_t n_c
     // a strip of zeros: what the lanes of absent activation rows read
     L.zero = L.xs + max((uint32_t)m * L.xs_row, partial_bytes);
     L.waves = (L.zero + kTStripBytes + 15u) & ~15u;
-    L.tasks_off = qcap * 16u;  // behind the queue
+    L.tasks_off = qcap * 8u;  // behind the queue of 8-byte records
     L.wave_bytes = (L.tasks_off + kRTasks * 2u + 15u) & ~15u;
     L.total = L.waves + n_waves * L.wave_bytes;
     return L;
@@ -91,6 +91,17 @@ struct TileSink {
     bool x_on;           // that row exists
     uint32_t idle_addr;  // an address that can be read
     uint32_t wn, xa;     // the lane's element of the round: weight bits | column << 16, address
+    uint32_t n_chunks;
+    // a record's second word: column n of the product << 27 | row in the workgroup << 20 | column / 32 << 9 | level-1
+    // elements between the unit's start and the word
+    __device__ __forceinline__ void unpack(uint32_t packed, uint32_t unit0, uint32_t tq1_addr, uint32_t &r0, uint32_t &unit,
+                                           uint32_t &k0, uint32_t &row_field) {
+        const uint32_t lrow = (packed >> 20) & 127u, kw = (packed >> 9) & 2047u;
+        unit = unit0 + lrow * n_chunks + (kw >> 4);
+        r0 = unit * kFastChunk + ((kw & 15u) << 5) - lds_u32(tq1_addr + (unit - unit0) * 4u) - (packed & 511u);
+        k0 = kw << 5;
+        row_field = ((packed >> 27) << 12) | lrow;
+    }
     __device__ __forceinline__ void put(uint32_t w_bits, uint32_t row_field, uint32_t addr) {
         wn = w_bits | ((row_field >> 12) << 16);
         xa = addr;
@@ -139,7 +150,7 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     // a tile is tile_rows = 4, 8 or 16 weight rows by 16 / tile_rows column blocks side by side: column n of the matrix
     // instruction is weight row n % tile_rows in column block n / tile_rows of the step (its slot)
     const uint32_t tile_rows = 1u << lg_rows, slots = 16u >> lg_rows;
-    const uint32_t r = n & (tile_rows - 1u), slot = n >> lg_rows;
+    const uint32_t r = n & (tile_rows - 1u);
 
     const uint32_t row0 = blockIdx.x * rows_per_wg;
     const uint32_t rows_here = min(rows_per_wg, P.out_f - row0), rows_cap = rows_per_wg;
@@ -178,6 +189,10 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     const bool tile_live = trow0 < rows_here;                      // a wave beyond the workgroup's rows has nothing to do
     const bool row_live = trow0 + r < rows_here;                   // this lane's row exists
     const uint32_t lrow = min(trow0 + r, rows_here - 1);           // clamped: a lane without a row decodes zeros
+    // the two things the loop needs of the lane's row: the index of its first unit (table entries, and bitmap words at
+    // 16 a unit) and the row's part of a record
+    const uint32_t base_u = row0 * n_chunks + lrow * n_chunks;
+    const uint32_t rec_hi = (n << 27) | (lrow << 20);
     const uint32_t n_parts = (n_chunks + x_blocks - 1) / x_blocks;
     uint32_t part_first = 0, part_count = min(x_blocks, n_chunks);  // the part's column blocks
     uint32_t c_begin = 0, c_end = 0;                                // this wave's run of them
@@ -198,11 +213,16 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         u32x4 bm;        // the four bitmap words of the lane's strip
     };
     auto request = [&](uint32_t c0, TaskIn &T) {
-        const uint32_t c = min(c0 + slot, c_end - 1u);  // clamped: a lane without a block reads what exists
-        T.col = c * kFastChunk + kg * 128u;
-        T.q1u = __builtin_amdgcn_raw_buffer_load_b32(tb_rsrc, (int)((unit0 + lrow * n_chunks + c) * 4u), 0, 0);
-        T.bm = __builtin_amdgcn_raw_buffer_load_b128(b1_rsrc, (int)((((row0 + lrow) * P.in_f + T.col) >> 5) * 4u), 0, 0);
-        if (!row_live || c0 + slot >= c_end) T.col |= 0x80000000u;
+        // the lane's k group and slot, worked out from a lane number the compiler cannot connect with the one
+        // above: two instructions here instead of two registers held through the loop
+        uint32_t l2 = threadIdx.x;
+        asm volatile("" : "+v"(l2));
+        const uint32_t kg2 = (l2 >> 4) & 3u, slot2 = (l2 & 15u) >> lg_rows;
+        const uint32_t c = min(c0 + slot2, c_end - 1u);  // clamped: a lane without a block reads what exists
+        T.col = c * kFastChunk + kg2 * 128u;
+        T.q1u = __builtin_amdgcn_raw_buffer_load_b32(tb_rsrc, (int)((base_u + c) * 4u), 0, 0);
+        T.bm = __builtin_amdgcn_raw_buffer_load_b128(b1_rsrc, (int)((((base_u + c) << 4) + kg2 * 4u) * 4u), 0, 0);
+        if (!row_live || c0 + slot2 >= c_end) T.col |= 0x80000000u;
     };
     TaskIn T;
     if (c_begin < c_end) request(c_begin, T);
@@ -299,7 +319,7 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
     uint32_t qcount = 0;  // wave-uniform
     auto resolve = [&]() {
-        TileSink sink{acc, n, kg, r * L.xs_row, r < (uint32_t)m, xs_addr, 0u, xs_addr};
+        TileSink sink{acc, n, kg, r * L.xs_row, r < (uint32_t)m, xs_addr, 0u, xs_addr, n_chunks};
         const TaskPool none{0, 0, 0, 1, 0, 0};
         if (ANY)
             resolve_rows_to<kTMaxM, false, true, 2, false, kTStripBytes>(
@@ -382,10 +402,9 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
             const uint64_t any = __ballot(zrem != 0);
             if (any != 0) {  // lanes with elements above level 1 leave a record
                 if (zrem != 0) {
-                    const uint32_t kcol = S.col + 32u * (uint32_t)k;
-                    const uint32_t unit = unit0 + lrow * n_chunks + (S.col >> 9);
-                    const uint32_t r0 = (row0 + lrow) * P.in_f + kcol - rk;
-                    push_record(queue, qcount + lanes_below(any), make_uint4(zrem, r0, unit, (n << 28) | (lrow << 16) | kcol));
+                    const uint32_t kw = (S.col >> 5) + (uint32_t)k;  // column / 32
+                    const uint32_t rel = rk - lds_u32(tq1_addr + (base_u - unit0 + (S.col >> 9)) * 4u);
+                    push_record8(queue, qcount + lanes_below(any), zrem, rec_hi | (kw << 9) | rel);
                 }
                 qcount += (uint32_t)__popcll(any);
                 do splice_once(w0, w1, w2, zrem);
