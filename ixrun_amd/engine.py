@@ -30,9 +30,9 @@ __all__ = ["Int8XEngine", "StreamingLinear", "GraphLinear", "ResourceScheduler"]
 MAX_FUSED_ROWS = 16  # activation rows served by the fused decode+GEMV kernel
 # With a decode buffer at hand, more rows than this go through decode + library GEMM.  Tensors that are almost all
 # level 1, MI355X: the pair takes 72-75 us on 17408 x 5120 and 5120 x 17408 at any M up to 32 and 34-50 us on
-# 5120 x 5120 (five levels: 73-74 and 38-39 us); the fused kernels take 27 / 29 / 31 us (17408 x 5120), 34 / 40 / 47 us
-# (5120 x 17408) and 18 / 24 / 26 us (5120 x 5120) at M = 8 / 12 / 16 (five levels: 27 / 29 / 32, 38 / 45 / 51 and
-# 20 / 31 / 32 us): every row count the fused kernels take.  Dense mixes (55 / 40 / 5 %): the pair takes 84-90 us, the
+# 5120 x 5120 (five levels: 73-74 and 38-39 us); the fused kernels take 27 / 31 / 31 us (17408 x 5120), 35 / 45 / 48 us
+# (5120 x 17408) and 20 / 24 / 26 us (5120 x 5120) at M = 8 / 12 / 16 (five levels: 29 / 31 / 32, 39 / 45 / 51 and
+# 23 / 31 / 31 us): every row count the fused kernels take.  Dense mixes (55 / 40 / 5 %): the pair takes 84-90 us, the
 # fused kernels 55-62 / 69-72 / 85-88 / 116-119 us at M = 1 / 2 / 4 / 8.  Dense mixes in other schemes have a
 # level-by-level kernel for one row only (five levels: 95-104 us; the pair 127 us, the any-scheme kernel 209-260 us at
 # M = 2 .. 8).
