@@ -74,6 +74,8 @@ WORKLOADS = {
     "down_proj_5120x17408_m4_student_t": (5120, 17408, 4, "student_t"),
     "down_proj_5120x17408_m8_student_t": (5120, 17408, 8, "student_t"),
     "down_proj_5120x17408_m16_student_t": (5120, 17408, 16, "student_t"),
+    "down_proj_5120x17408_m2_student_t": (5120, 17408, 2, "student_t"),
+    "attn_proj_5120x5120_m2_student_t": (5120, 5120, 2, "student_t"),
     "attn_proj_5120x5120_m4_student_t": (5120, 5120, 4, "student_t"),
     "attn_proj_5120x5120_m8_student_t": (5120, 5120, 8, "student_t"),
     "attn_proj_5120x5120_m16_student_t": (5120, 5120, 16, "student_t"),

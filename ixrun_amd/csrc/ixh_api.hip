@@ -20,6 +20,7 @@ std::atomic<int> g_opt_gemv_strips{0};
 std::atomic<int> g_opt_gemv_tiles{0};
 std::atomic<int> g_opt_gemv_tile_rows{0};
 std::atomic<int> g_opt_gemv_tile_cus{0};
+std::atomic<int> g_opt_gemv_dense_tiles{0};
 
 void set_error(const char *fmt, ...) {
     va_list ap;
@@ -117,6 +118,11 @@ int ixh_set_option(const char *name, int64_t value) {
     if (strcmp(name, "gemv_tile_cus") == 0) {
         if (value < 0 || value > 4096) { set_error("gemv_tile_cus %lld not in 0..4096", (long long)value); return IXH_EINVAL; }
         g_opt_gemv_tile_cus.store((int)value, std::memory_order_relaxed);
+        return IXH_OK;
+    }
+    if (strcmp(name, "gemv_dense_tiles") == 0) {
+        if (value < -1 || value > 1) { set_error("gemv_dense_tiles %lld not in -1..1", (long long)value); return IXH_EINVAL; }
+        g_opt_gemv_dense_tiles.store((int)value, std::memory_order_relaxed);
         return IXH_OK;
     }
     if (strcmp(name, "gemv_strips") == 0) {
@@ -289,6 +295,12 @@ static int gemv_any(const IxhPacked *packed, const int32_t *prefix, int64_t chun
         (!mostly_l1 || (flags & IXH_GEMV_DENSE)) && gemv_dense34568_supports(d, (uint32_t)chunk, m, x))
         // the same for the five-level scheme (3,4,5,6,8)
         rc = launch_gemv_dense34568(d, prefix, x, y, y32, (float *)workspace, atomic, (hipStream_t)stream);
+    if (rc == IXH_EUNSUPPORTED && !atomic && !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED)) &&
+        (!mostly_l1 || (flags & IXH_GEMV_DENSE)) && g_opt_gemv_dense_tiles.load(std::memory_order_relaxed) >= 0 &&
+        gemv_dense358_tiles_supports(d, (uint32_t)chunk, m, x, ldx))
+        // (3,5,8), 2..16 activation rows, many elements above level 1: 16 rows' spans gathered to position order in
+        // LDS, products on the matrix pipe
+        rc = launch_gemv_dense358_tiles(d, prefix, x, m, ldx, y, ldy, (float *)workspace, (hipStream_t)stream);
     if (rc == IXH_EUNSUPPORTED && !atomic && !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED)) &&
         (!mostly_l1 || (flags & IXH_GEMV_DENSE)) && gemv_dense358_rows_supports(d, (uint32_t)chunk, m, x, ldx))
         // (3,5,8), 2..8 activation rows, many elements above level 1: weights gathered to position order per span
