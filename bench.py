@@ -42,7 +42,7 @@ _OLD = ((), "measured-on-earlier-sources")  # figures kept for the record; repor
 MEASURED_TRAFFIC_BYTES = {
     "down_proj_5120x17408_m1_student_t": (23024.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "3ff9786c3dd127e5"),
     "attn_proj_5120x5120_m1_student_t": (7104.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "3ff9786c3dd127e5"),
-    "down_proj_5120x17408_m1_calibrated": (33832.0 * 2.0 * 1024 + 40.0 * 1024, _DENSE, "4c194d30b116b40a"),
+    "down_proj_5120x17408_m1_calibrated": (33824.0 * 2.0 * 1024 + 40.0 * 1024, _DENSE, "f1be9ebc0922dff2"),
     "down_proj_5120x17408_m1_five_level_calibrated": (49711.0 * 2.0 * 1024 + 1337.0 * 1024, _DENSE5, "af662fec32ed7b32"),
     "gate_up_17408x5120_m4_student_t": (28106.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "e0872c2b358575ff"),
     "gate_up_17408x5120_m16_student_t": (26683.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "e0872c2b358575ff"),
@@ -86,6 +86,9 @@ WORKLOADS = {
     "gate_up_17408x5120_m2_calibrated": (17408, 5120, 2, "calibrated"),
     "gate_up_17408x5120_m4_calibrated": (17408, 5120, 4, "calibrated"),
     "gate_up_17408x5120_m8_calibrated": (17408, 5120, 8, "calibrated"),
+    "gate_up_17408x5120_m16_calibrated": (17408, 5120, 16, "calibrated"),
+    "down_proj_5120x17408_m8_calibrated": (5120, 17408, 8, "calibrated"),
+    "attn_proj_5120x5120_m8_calibrated": (5120, 5120, 8, "calibrated"),
     # 64 distinct 5120x5120 layers chained (each output feeds the next layer), one hipGraph: us per layer
     "graph64_5120x5120_m1_student_t": (5120, 5120, 1, "student_t"),
     # many activation rows: decode into LDS tiles + bf16 MFMA, five-level scheme
@@ -448,7 +451,8 @@ def also_block(dev, args):
 
     # (workload that names the layer, [(reported name, activation rows, variant)])
     plan = [
-        ("down_proj_5120x17408_m1_calibrated", [("down_proj_5120x17408_m1_calibrated", 1, "fused")]),
+        ("down_proj_5120x17408_m1_calibrated", [("down_proj_5120x17408_m1_calibrated", 1, "fused"),
+                                                ("down_proj_5120x17408_m8_calibrated", 8, "fused")]),
         ("down_proj_5120x17408_m1_reference_recipe", [("down_proj_5120x17408_m1_reference_recipe", 1, "fused")]),
         ("down_proj_5120x17408_m1_five_level_calibrated", [("down_proj_5120x17408_m1_five_level_calibrated", 1, "fused")]),
         ("down_proj_5120x17408_m1_student_t", [("down_proj_5120x17408_m1_student_t_split_k_call", 1, "split_k"),

@@ -296,10 +296,12 @@ static int gemv_any(const IxhPacked *packed, const int32_t *prefix, int64_t chun
         // the same for the five-level scheme (3,4,5,6,8)
         rc = launch_gemv_dense34568(d, prefix, x, y, y32, (float *)workspace, atomic, (hipStream_t)stream);
     if (rc == IXH_EUNSUPPORTED && !atomic && !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED)) &&
-        (!mostly_l1 || (flags & IXH_GEMV_DENSE)) && g_opt_gemv_dense_tiles.load(std::memory_order_relaxed) >= 0 &&
+        (!mostly_l1 || (flags & IXH_GEMV_DENSE)) &&
+        (g_opt_gemv_dense_tiles.load(std::memory_order_relaxed) > 0 ||
+         (g_opt_gemv_dense_tiles.load(std::memory_order_relaxed) == 0 && m >= 4)) &&
         gemv_dense358_tiles_supports(d, (uint32_t)chunk, m, x, ldx))
-        // (3,5,8), 2..16 activation rows, many elements above level 1: 16 rows' spans gathered to position order in
-        // LDS, products on the matrix pipe
+        // (3,5,8), 4..16 activation rows (2..16 when the option says so), many elements above level 1: 16 rows' spans
+        // gathered to position order in LDS, products on the matrix pipe; its time does not grow with the rows
         rc = launch_gemv_dense358_tiles(d, prefix, x, m, ldx, y, ldy, (float *)workspace, (hipStream_t)stream);
     if (rc == IXH_EUNSUPPORTED && !atomic && !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED)) &&
         (!mostly_l1 || (flags & IXH_GEMV_DENSE)) && gemv_dense358_rows_supports(d, (uint32_t)chunk, m, x, ldx))

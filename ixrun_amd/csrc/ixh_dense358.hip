@@ -354,7 +354,7 @@ struct DnFlatSpans {
     }
 };
 
-template <bool GS, class Spans, class Sink>
+template <bool GS, class Spans, class Sink, bool TAKE_TURNS = true>
 __device__ __forceinline__ void dn_walk_spans(const Dev &P, const int32_t *__restrict__ prefix, uint32_t entries,
                                               const uint16_t *__restrict__ group_scales, uint32_t group_shift,
                                               const uint32_t *lut, uint16_t *wc, float scale, uint32_t lane,
@@ -429,7 +429,7 @@ __device__ __forceinline__ void dn_walk_spans(const Dev &P, const int32_t *__res
     for (uint32_t turn = wave_turn;; ++turn) {
         // the waves that share a SIMD take turns at the issue priority, one span each, so that they do not meet at the
         // same phase (dequantise, gather, store or multiply) span after span
-        {
+        if (TAKE_TURNS) {  // (not where the waves meet at a barrier every span: there they should keep pace)
             const uint32_t pr = turn % 3u;  // s_setprio takes an immediate
             if (pr == 0) __builtin_amdgcn_s_setprio(0);
             else if (pr == 1) __builtin_amdgcn_s_setprio(1);
@@ -930,7 +930,8 @@ k_gemv358_dense_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chun
     sink.tile_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)(dt_smem + kDnLutBytes);
     sink.red = reinterpret_cast<float *>(dt_smem + kDnLutBytes + (size_t)kDtWaves * kDtRegion);
     sink.acc = d_f32x4{0.f, 0.f, 0.f, 0.f};
-    dn_walk_spans<false>(P, prefix, P.out_f * n_chunks + 1, nullptr, 0u, lut, wc, scale, lane, spans, sink, wave);
+    dn_walk_spans<false, DnTileSpans, DnMfmaSink, false>(P, prefix, P.out_f * n_chunks + 1, nullptr, 0u, lut, wc, scale, lane,
+                                                         spans, sink, wave);
 }
 
 bool gemv_dense358_tiles_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x, int64_t ldx) {

@@ -32,12 +32,13 @@ MAX_FUSED_ROWS = 16  # activation rows served by the fused decode+GEMV kernel
 # level 1, MI355X: the pair takes 72-75 us on 17408 x 5120 and 5120 x 17408 at any M up to 32 and 34-50 us on
 # 5120 x 5120 (five levels: 73-74 and 38-39 us); the fused kernels take 27 / 31 / 31 us (17408 x 5120), 35 / 45 / 48 us
 # (5120 x 17408) and 20 / 24 / 26 us (5120 x 5120) at M = 8 / 12 / 16 (five levels: 29 / 31 / 32, 39 / 45 / 51 and
-# 23 / 31 / 31 us): every row count the fused kernels take.  Dense mixes (55 / 40 / 5 %): the pair takes 84-90 us, the
-# fused kernels 55-62 / 69-72 / 85-88 / 116-119 us at M = 1 / 2 / 4 / 8.  Dense mixes in other schemes have a
-# level-by-level kernel for one row only (five levels: 95-104 us; the pair 127 us, the any-scheme kernel 209-260 us at
-# M = 2 .. 8).
+# 23 / 31 / 31 us): every row count the fused kernels take.  Dense mixes (55 / 40 / 5 %): the pair takes
+# 91-93 us on the large layers and 34-52 us on 5120 x 5120, the fused kernels 54-62 / 69-73 / 79-85 / 80-85 / 83-88 us
+# (large layers) and 21 / 26 / 29 / 29 / 31 us (5120 x 5120) at M = 1 / 2 / 4 / 8 / 16: every row count as well.  Dense
+# mixes in other schemes have a level-by-level kernel for one row only (five levels: 95-104 us; the pair 127 us, the
+# any-scheme kernel 209-260 us at M = 2 .. 8).
 MAX_FUSED_ROWS_WITH_BUFFER = 16
-MAX_FUSED_ROWS_WITH_BUFFER_DENSE = 4
+MAX_FUSED_ROWS_WITH_BUFFER_DENSE = 16
 # More rows than that: with a shared decode buffer the layer decodes into it and calls the library GEMM
 # (5120 x 5120 five-level on MI355X: 60 us at 32 rows, 84 us at 512); without one it runs the fused
 # decode+GEMM, which keeps the bf16 weight out of HBM altogether but is slower (84 us and 194 us): its

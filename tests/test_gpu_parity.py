@@ -291,7 +291,7 @@ def test_gemv_dense_rows_on_the_matrix_pipe(oracle, dev, gemv_option, kind, shap
     for m in (2, 3, 8, 9, 16):
         x = activations(m, in_f, seed=m)
         y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
-        for dense_tiles in (0, -1) if (m <= 8 and cus == 0) else (0,):
+        for dense_tiles in (1, 0, -1) if (m <= 8 and cus == 0) else (1,):
             gemv_option("gemv_dense_tiles", dense_tiles)
             y = run_gemv(dp, 512, x, m, dev, flags=_lib.IXH_GEMV_DENSE)
             check_outputs(y, y64, f"{kind} {shape} m={m} on {cus} CUs, gemv_dense_tiles={dense_tiles}")
