@@ -681,7 +681,10 @@ def test_full_size_calibrated_layer(oracle, dev):
     sl._set_shared_buf(shared)
     w_bits = oracle.decode_packed_bf16(p)
     assert np.array_equal(bf16_bits(sl._decode()), w_bits)
-    x = activations(2, in_f, seed=1)
-    y = sl(x.to(dev))
-    y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
-    check_outputs(bf16_bits(y), y64, "full-size calibrated m=2")
+    # two rows: weights gathered per wave; eight and sixteen: the matrix-pipe kernel (a row block's spans lie in two
+    # workgroups here: 320 blocks of 16 rows x 9 spans dealt to one workgroup per CU)
+    for m in (2, 8, 16):
+        x = activations(m, in_f, seed=m)
+        y = sl(x.to(dev))
+        y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
+        check_outputs(bf16_bits(y), y64, f"full-size calibrated m={m}")
