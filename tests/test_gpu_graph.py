@@ -37,7 +37,8 @@ def run_chain(layers, x):
 
 @pytest.mark.parametrize("maker,m,level_bits", [
     (student_t_weight, 1, (3, 5, 8)), (outlier_weight, 1, (3, 5, 8)), (student_t_weight, 4, (3, 5, 8)),
-    (outlier_weight, 16, (3, 5, 8)), (dense_weight, 1, (3, 4, 5, 6, 8)), (student_t_weight, 16, (3, 4, 5, 6, 8))])
+    (outlier_weight, 16, (3, 5, 8)), (dense_weight, 1, (3, 4, 5, 6, 8)), (student_t_weight, 16, (3, 4, 5, 6, 8)),
+    (dense_weight, 2, (3, 5, 8)), (dense_weight, 8, (3, 5, 8)), (dense_weight, 16, (3, 5, 8)), (student_t_weight, 8, (3, 5, 8))])
 def test_graph_replay_matches_eager(maker, m, level_bits):
     dev = torch.device("cuda:0")
     layers = build_chain(6, 1024, dev, maker, level_bits)
