@@ -92,8 +92,9 @@ const char *ixh_last_error(void);
  *   "gemv_tile_cus"  the number of CUs over which the tile kernel's planner spreads the rows: 0 = the device's
  *                    (default), 1..4096 = that many (small tensors then get workgroups with several tiles); also the
  *                    number of workgroups of the dense-mix matrix-pipe kernel
- *   "gemv_dense_tiles" the level-by-level kernel for dense (3,5,8) mixes that multiplies on the matrix pipe (2..16
- *                    activation rows): -1 = never, 0 = from four rows on (default), 1 = from two rows on
+ *   "gemv_dense_tiles" the level-by-level kernels for dense mixes that multiply on the matrix pipe (2..16
+ *                    activation rows): -1 = never, 0 = (3,5,8) from four rows on, (3,4,5,6,8) from two (default),
+ *                    1 = both from two rows on
  *   "gemv_strips"    the strip kernel (up to eight activation rows a pass): -1 = never, 0 = for three rows or more
  *                    where the tile kernel does not run and the shape fits (default), 1..6 = wherever it fits
  * Returns IXH_EINVAL for an unknown name or a value out of range.  Calls already running are not affected.

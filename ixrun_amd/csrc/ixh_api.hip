@@ -304,6 +304,11 @@ static int gemv_any(const IxhPacked *packed, const int32_t *prefix, int64_t chun
         // gathered to position order in LDS, products on the matrix pipe; its time does not grow with the rows
         rc = launch_gemv_dense358_tiles(d, prefix, x, m, ldx, y, ldy, (float *)workspace, (hipStream_t)stream);
     if (rc == IXH_EUNSUPPORTED && !atomic && !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED)) &&
+        (!mostly_l1 || (flags & IXH_GEMV_DENSE)) && g_opt_gemv_dense_tiles.load(std::memory_order_relaxed) >= 0 &&
+        gemv_dense34568_tiles_supports(d, (uint32_t)chunk, m, x, ldx))
+        // the same for the five-level scheme (3,4,5,6,8), from two rows on (it has no kernel of its own for two and three)
+        rc = launch_gemv_dense34568_tiles(d, prefix, x, m, ldx, y, ldy, (float *)workspace, (hipStream_t)stream);
+    if (rc == IXH_EUNSUPPORTED && !atomic && !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED)) &&
         (!mostly_l1 || (flags & IXH_GEMV_DENSE)) && gemv_dense358_rows_supports(d, (uint32_t)chunk, m, x, ldx))
         // (3,5,8), 2..8 activation rows, many elements above level 1: weights gathered to position order per span
         rc = launch_gemv_dense358_rows(d, prefix, x, m, ldx, y, ldy, (float *)workspace, (hipStream_t)stream);

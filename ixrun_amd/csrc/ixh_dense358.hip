@@ -23,6 +23,7 @@
 // per 2048 weights), five waves per SIMD cover the load latency.  A wave sums whole rows when rows spread evenly over
 // the launch; otherwise partial sums of the spans of a row are combined through the workspace in span order (or
 // added to y32 with atomics).
+#include "ixh_dense_tiles.h"
 #include "ixh_fast358.h"
 
 namespace ixh {
@@ -784,25 +785,12 @@ k_gemv358_dense_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunk
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// Product with 2..16 activation rows for dense mixes on the matrix pipe.  A workgroup of 16 waves takes 16 neighbouring
-// weight rows, one per wave, span by span: every wave brings its row's span to position order with the walker above
-// and leaves it in its own LDS array (64 lane rows of 80 bytes, as the full decode does before it stores); after a
-// barrier the 16 arrays are a tile of 16 rows x 2048 columns, and wave w multiplies columns 128 w .. 128 w + 127 of it
-// with the activations: four v_mfma_f32_16x16x32_bf16 (the weights of row n, eight at a time, from wave n's array as
-// one operand, eight activations of row a at the same columns, loaded from global memory while the span was decoded,
-// as the other).  The accumulators stay in registers from span to span; when the row block ends (or the workgroup's
-// share of the work does) the 16 waves' accumulators are added in wave order and written as one piece of the block's
-// partial sums, which a second kernel adds in piece order: the steps (row block, span) are dealt to the workgroups
-// in equal contiguous shares, so a row block's spans may lie in two or more workgroups.  The decode costs what it
-// costs the full decoder, whatever the number of activation rows.
+// Product with 2..16 activation rows for dense mixes on the matrix pipe: the walker above, 16 waves to a workgroup,
+// with the sink of ixh_dense_tiles.h (the 16 waves' spans as a tile in LDS, v_mfma_f32_16x16x32_bf16, pieces of partial
+// sums for k_reduce_chunks).  The decode costs what it costs the full decoder, whatever the number of activation rows.
 // ---------------------------------------------------------------------------------------------------------------
-typedef __bf16 d_bf16x8 __attribute__((ext_vector_type(8)));
-typedef float d_f32x4 __attribute__((ext_vector_type(4)));
-
-constexpr int kDtWaves = 16;
-extern std::atomic<int> g_opt_gemv_tile_cus;
-constexpr uint32_t kDtRegion = kDnSlots * 2 + 16;  // bytes between the waves' arrays: the tile's rows four banks apart
-constexpr size_t kDtLdsBytes = kDnLutBytes + (size_t)kDtWaves * kDtRegion + (size_t)kDtWaves * 256 * 4;
+constexpr uint32_t kDtRegion = kDnSlots * 2 + 16;  // bytes between the waves' arrays
+constexpr size_t kDtLdsBytes = kDnLutBytes + (size_t)kDtWaves * kDtRegion + kDtSumsBytes;
 
 // the workgroup's steps [step_begin, step_end) of the sequence (row block, span); this wave's row of every block
 struct DnTileSpans {
@@ -832,74 +820,9 @@ struct DnTileSpans {
 };
 
 struct DnMfmaSink {
-    const uint16_t *__restrict__ x;
-    int64_t ldx;
-    int m;
-    float *__restrict__ ws;
-    uint32_t out_f, in_f, spans_per_row, n_pieces, total_steps, step_end;
-    uint32_t wave, lane;
-    uint16_t *wc;        // this wave's array
-    uint32_t tile_addr;  // LDS address of wave 0's array
-    float *red;          // [16 waves][16 activation rows][16 weight rows]
-    d_u32x4 xa[4];
-    d_f32x4 acc;
-
-    // the workgroup that holds step t when `total_steps` steps are dealt to gridDim.x workgroups in contiguous shares
-    __device__ __forceinline__ uint32_t group_of(uint32_t t) const {
-        return (uint32_t)((((uint64_t)t + 1u) * gridDim.x + total_steps - 1u) / total_steps) - 1u;
-    }
-    // the activations this wave multiplies with: rows lane % 16, eight columns per k group of each of its four steps
-    __device__ __forceinline__ void begin(const DnSpan &sp) {
-        const uint32_t a = lane & 15u, kg = lane >> 4;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t col = sp.b * kDnSpan + (wave * 4u + (uint32_t)j) * 32u + kg * 8u;
-            xa[j] = d_u32x4{0u, 0u, 0u, 0u};
-            if (a < (uint32_t)m && col < in_f) {
-                const uint4 v = *reinterpret_cast<const uint4 *>(x + (int64_t)a * ldx + col);
-                xa[j] = d_u32x4{v.x, v.y, v.z, v.w};
-            }
-        }
-    }
-    __device__ __forceinline__ void end(const DnSpan &sp, const uint32_t (&o)[16], uint32_t) {
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        d_u32x4 *const rows = reinterpret_cast<d_u32x4 *>(wc);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) rows[lane * 5 + j] = d_u32x4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
-        __syncthreads();  // the tile is whole
-        const uint32_t n = lane & 15u, kg = lane >> 4;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            // weight row n, columns 32 (4 wave + j) + 8 kg ..: lane row 4 wave + j of wave n's array, 16 bytes in
-            const d_u32x4 b = *reinterpret_cast<const __attribute__((address_space(3))) d_u32x4 *>(
-                (uintptr_t)(tile_addr + n * kDtRegion + (wave * 4u + (uint32_t)j) * 80u + kg * 16u));
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(d_bf16x8, xa[j]), __builtin_bit_cast(d_bf16x8, b),
-                                                         acc, 0, 0, 0);
-        }
-        __syncthreads();  // before any wave's next span overwrites its array
-        const bool block_ends = sp.b + 1 == spans_per_row;
-        if (!block_ends && sp.c + 1 != step_end) return;
-        // ---- the block's sums so far leave: added over the waves in order, one piece per workgroup ----
-#pragma unroll
-        for (int i = 0; i < 4; ++i) red[wave * 256u + (4u * kg + (uint32_t)i) * 16u + n] = acc[i];
-        acc = d_f32x4{0.f, 0.f, 0.f, 0.f};
-        __syncthreads();
-        const uint32_t tid = wave * kWave + lane;
-        if (tid < 256) {
-            const uint32_t a = tid >> 4, row = sp.a * (uint32_t)kDtWaves + (tid & 15u);
-            if (a < (uint32_t)m && row < out_f) {
-                float sum = 0.0f;
-#pragma unroll
-                for (int w = 0; w < kDtWaves; ++w) sum += red[(uint32_t)w * 256u + tid];
-                const uint32_t piece = blockIdx.x - group_of(sp.a * spans_per_row);
-                ws[((size_t)piece * m + a) * out_f + row] = sum;
-                if (block_ends)  // the pieces nobody writes
-                    for (uint32_t q = piece + 1; q < n_pieces; ++q) ws[((size_t)q * m + a) * out_f + row] = 0.0f;
-            }
-        }
-        __syncthreads();  // the sums are read before the next block's arrive
-    }
+    DtMfmaSink<kDtRegion> t;
+    __device__ __forceinline__ void begin(const DnSpan &sp) { t.begin(DtStep{sp.a, sp.b, sp.c}); }
+    __device__ __forceinline__ void end(const DnSpan &sp, const uint32_t (&o)[16], uint32_t) { t.end(DtStep{sp.a, sp.b, sp.c}, o); }
 };
 
 __global__ void __launch_bounds__(kWave *kDtWaves)
@@ -923,13 +846,13 @@ k_gemv358_dense_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chun
     const uint32_t step_end = (uint32_t)(((uint64_t)blockIdx.x + 1u) * total_steps / gridDim.x);
     const DnTileSpans spans{n_chunks, spans_per_row, P.out_f, wave, step_begin, step_end};
     DnMfmaSink sink;
-    sink.x = x; sink.ldx = ldx; sink.m = m; sink.ws = ws;
-    sink.out_f = P.out_f; sink.in_f = P.in_f; sink.spans_per_row = spans_per_row; sink.n_pieces = n_pieces;
-    sink.total_steps = total_steps; sink.step_end = step_end;
-    sink.wave = wave; sink.lane = lane; sink.wc = wc;
-    sink.tile_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)(dt_smem + kDnLutBytes);
-    sink.red = reinterpret_cast<float *>(dt_smem + kDnLutBytes + (size_t)kDtWaves * kDtRegion);
-    sink.acc = d_f32x4{0.f, 0.f, 0.f, 0.f};
+    sink.t.x = x; sink.t.ldx = ldx; sink.t.m = m; sink.t.ws = ws;
+    sink.t.out_f = P.out_f; sink.t.in_f = P.in_f; sink.t.spans_per_row = spans_per_row; sink.t.n_pieces = n_pieces;
+    sink.t.total_steps = total_steps; sink.t.step_end = step_end;
+    sink.t.wave = wave; sink.t.lane = lane; sink.t.wc = wc;
+    sink.t.tile_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)(dt_smem + kDnLutBytes);
+    sink.t.red = reinterpret_cast<float *>(dt_smem + kDnLutBytes + (size_t)kDtWaves * kDtRegion);
+    sink.t.acc = dt_f32x4{0.f, 0.f, 0.f, 0.f};
     dn_walk_spans<false, DnTileSpans, DnMfmaSink, false>(P, prefix, P.out_f * n_chunks + 1, nullptr, 0u, lut, wc, scale, lane,
                                                          spans, sink, wave);
 }
@@ -940,33 +863,27 @@ bool gemv_dense358_tiles_supports(const Dev &P, uint32_t chunk, int m, const uin
            ((uintptr_t)P.last & 3u) == 0 && P.out_f != 0;
 }
 
+static uint32_t dt_cu_count() {
+    static const uint32_t n_cu = [] {
+        int dev = 0, v = 256;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
+        return (uint32_t)v;
+    }();
+    return n_cu;
+}
+
 // The workspace holds n_pieces x m x out_f partial sums (n_pieces <= in_f / 512, what ixh_gemv_workspace_bytes asks for).
 int launch_gemv_dense358_tiles(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
                                int64_t ldy, float *ws, hipStream_t s) {
     static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_dense_tiles),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDtLdsBytes) == hipSuccess;
     if (!raised) return IXH_EUNSUPPORTED;
-    static const uint32_t n_cu = [] {
-        int dev = 0, v = 256;
-        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
-        return (uint32_t)v;
-    }();
-    const uint32_t n_chunks = P.in_f / kFastChunk;
-    const uint32_t spans_per_row = (n_chunks + 3) / 4;
-    const uint32_t n_blocks = (P.out_f + kDtWaves - 1) / kDtWaves;
-    const uint64_t total = (uint64_t)n_blocks * spans_per_row;
-    if (total >= (1ull << 31)) return IXH_EUNSUPPORTED;
-    // one workgroup per CU; fewer where the pieces of a row block would not fit the workspace (a block's spans lie in
-    // at most ceil(groups / blocks) + 1 workgroups)
-    const int cus_opt = g_opt_gemv_tile_cus.load(std::memory_order_relaxed);  // ixh_set_option("gemv_tile_cus")
-    uint32_t groups = (uint32_t)min((uint64_t)(cus_opt > 0 ? (uint32_t)cus_opt : n_cu), total);
-    groups = (uint32_t)min((uint64_t)groups, (uint64_t)(n_chunks - 1u) * n_blocks);
-    const uint32_t n_pieces = (groups + n_blocks - 1) / n_blocks + 1;
-    if (n_pieces > n_chunks) return IXH_EUNSUPPORTED;
-    hipLaunchKernelGGL(k_gemv358_dense_tiles, dim3(groups), dim3(kWave * kDtWaves), kDtLdsBytes, s, P, prefix, n_chunks,
-                       spans_per_row, (uint32_t)total, x, m, ldx, ws, n_pieces);
+    const DtPlan plan = dt_plan(P.out_f, P.in_f, dt_cu_count());
+    if (plan.groups == 0) return IXH_EUNSUPPORTED;
+    hipLaunchKernelGGL(k_gemv358_dense_tiles, dim3(plan.groups), dim3(kWave * kDtWaves), kDtLdsBytes, s, P, prefix,
+                       plan.n_chunks, plan.spans_per_row, plan.total_steps, x, m, ldx, ws, plan.n_pieces);
     if (hipGetLastError() != hipSuccess) return IXH_ELAUNCH;
-    return launch_reduce_chunks(ws, n_pieces, m, P.out_f, y, ldy, s);
+    return launch_reduce_chunks(ws, plan.n_pieces, m, P.out_f, y, ldy, s);
 }
 
 bool gemv_dense358_rows_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x, int64_t ldx) {

@@ -17,6 +17,7 @@
 // meet the compacted x pairs in v_dot2_f32_bf16: level 1 through the table of dequantised pairs, the others as
 // fma(code, scale, -T * scale), exact in fp32, rounded to bf16 as the reference's decoder does
 // (ixrun/triton_kernels.py:168-177).  Every array is padded with zeros up to 64 x codes-per-lane.
+#include "ixh_dense_tiles.h"
 #include "ixh_fast358.h"
 
 namespace ixh {
@@ -391,28 +392,47 @@ __device__ __forceinline__ void d5_dequant(const uint32_t (&w)[B], uint32_t *dst
     }
 }
 
-__global__ void __launch_bounds__(kWave *kD5Waves)
-k_decode34568_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, uint32_t n_spans, uint16_t *__restrict__ out) {
-    __shared__ __attribute__((aligned(16))) uint32_t lut[kD5LutBytes / 4];
-    __shared__ __attribute__((aligned(16))) uint16_t wc_all[kD5Waves][kD5Slots];
-    __shared__ uint32_t bm_all[kD5Waves][3][kD5BmWords];
+// TILE: the product with 2..16 activation rows on the matrix pipe instead of the store (ixh_dense_tiles.h): 16 waves
+// to a workgroup, wave w on row 16 rb + w of every step (row block rb, span k of the row) of the workgroup's share.
+struct D5TileArgs {
+    uint32_t n_chunks, spans_per_row, total_steps, n_pieces;
+    const uint16_t *x;
+    int m;
+    int64_t ldx;
+    float *ws;
+};
+constexpr uint32_t kD5Region = kD5Slots * 2 + 16;  // bytes between the waves' arrays in the tile kernel
+constexpr size_t kD5TileLds = kD5LutBytes + (size_t)kDtWaves * kD5Region + (size_t)kDtWaves * 3 * kD5BmWords * 4 + kDtSumsBytes;
+
+template <bool TILE>
+__global__ void __launch_bounds__(kWave *(TILE ? kDtWaves : kD5Waves))
+k_decode34568_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units, uint32_t n_spans, uint16_t *__restrict__ out,
+                    D5TileArgs ta) {
+    constexpr int kWaves = TILE ? kDtWaves : kD5Waves;
+    extern __shared__ __attribute__((aligned(16))) uint8_t d5_smem[];  // the tile kernel's (more than a static array may hold)
+    __shared__ __attribute__((aligned(16))) uint32_t lut_s[TILE ? 4 : kD5LutBytes / 4];
+    __shared__ __attribute__((aligned(16))) uint16_t wc_s[TILE ? 1 : kD5Waves][TILE ? 8 : kD5Slots];
+    __shared__ uint32_t bm_s[TILE ? 1 : kD5Waves][3][TILE ? 1 : kD5BmWords];
     static_assert(kD5Slots * 2 >= 64 * 80 && (kD5Slots * 2) % 16 == 0, "a wave's slots are re-used as 64 rows of 80 bytes");
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    uint32_t *const lut = TILE ? reinterpret_cast<uint32_t *>(d5_smem) : lut_s;
+    uint16_t *const wc = TILE ? reinterpret_cast<uint16_t *>(d5_smem + kD5LutBytes + wave * kD5Region) : wc_s[TILE ? 0 : wave];
+    uint32_t(*const bmw)[kD5BmWords] =
+        TILE ? reinterpret_cast<uint32_t(*)[kD5BmWords]>(d5_smem + kD5LutBytes + (size_t)kDtWaves * kD5Region) + wave * 3
+             : reinterpret_cast<uint32_t(*)[kD5BmWords]>(&bm_s[TILE ? 0 : wave][0][0]);
     const float scale = bf16_bits_to_f32(*P.scale);
     const float m7 = -7.0f * scale, m15 = -15.0f * scale, m31 = -31.0f * scale, m127 = -127.0f * scale;  // exact
-    for (uint32_t e = tid; e < 64 * 32; e += kWave * kD5Waves) {
+    for (uint32_t e = tid; e < 64 * 32; e += kWave * kWaves) {
         const uint32_t idx = e >> 5;
         lut[e] = d5_pack(dequant((int)(idx & 7u) - 3, scale), dequant((int)(idx >> 3) - 3, scale));
     }
-    // Positions past the tensor's end walk on through the arrays; what they read is not stored but must be there to
-    // read: start from zeros.
-    for (uint32_t j = lane; j < kD5Slots / 8; j += kWave) reinterpret_cast<e_u32x4 *>(wc_all[wave])[j] = e_u32x4{0, 0, 0, 0};
+    // Positions past the tensor's (or the row's) end walk on through the arrays; what they read is not stored (or meets
+    // activations that are zero) but must be there to read, and finite: start from zeros.
+    for (uint32_t j = lane; j < kD5Slots / 8; j += kWave) reinterpret_cast<e_u32x4 *>(wc)[j] = e_u32x4{0, 0, 0, 0};
     __syncthreads();
 
-    uint16_t *const wc = wc_all[wave];
     uint32_t *const wc32 = reinterpret_cast<uint32_t *>(wc);
-    uint32_t(*const bmw)[kD5BmWords] = bm_all[wave];
     const uint32_t lut_lane = (lane & 31u) << 2;
     const uint32_t entries = n_units + 1;
     const uint32_t *__restrict__ b1 = P.bm[0];
@@ -434,9 +454,22 @@ k_decode34568_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units,
     struct Ranks { uint32_t qa[4], qb[4]; };
     struct Shape { uint32_t p0, n_el, e[5], base[5], g1, g2, g3, at_last; };
     struct Loads { uint32_t w1, bm[3], bmx[3], d1[4], d2[5], d3[6], d4[7], d5[9]; };
+    // table units [u0, u1) of span (or step) sp: four of the flat tensor, or up to four of the wave's row
+    auto units_of = [&](uint32_t sp, uint32_t &u0, uint32_t &u1) {
+        if (TILE) {
+            const uint32_t rb = sp / ta.spans_per_row, k = sp - rb * ta.spans_per_row;
+            const uint32_t row = min(rb * (uint32_t)kDtWaves + wave, P.out_f - 1u);  // a wave past the last row: it again
+            u0 = row * ta.n_chunks + 4 * k;
+            u1 = u0 + min(4u, ta.n_chunks - 4 * k);
+        } else {
+            u0 = 4 * sp;
+            u1 = min(u0 + 4, n_units);
+        }
+    };
     auto table_of = [&](uint32_t sp) {
         Ranks q;
-        const uint32_t u0 = 4 * sp, u1 = min(u0 + 4, n_units);
+        uint32_t u0, u1;
+        units_of(sp, u0, u1);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             q.qa[i] = (uint32_t)prefix[(size_t)i * entries + u0];
@@ -446,8 +479,10 @@ k_decode34568_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units,
     };
     auto shape_of = [&](uint32_t sp, const Ranks &q) {
         Shape g;
-        g.p0 = 4 * sp * kFastChunk;
-        g.n_el = min(kD5Span, P.n - g.p0);
+        uint32_t u0, u1;
+        units_of(sp, u0, u1);
+        g.p0 = u0 * kFastChunk;
+        g.n_el = min((u1 - u0) * kFastChunk, P.n - g.p0);
         uint32_t rest = g.n_el, at = 0;
 #pragma unroll
         for (int i = 0; i < 5; ++i) {
@@ -479,18 +514,32 @@ k_decode34568_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units,
         return r;
     };
 
-    const uint32_t stride = gridDim.x * kD5Waves;
-    uint32_t sp = blockIdx.x * kD5Waves + wave;
-    if (sp >= n_spans) return;
+    // flat spans dealt to the waves of the launch in turn, or (TILE) the workgroup's contiguous share of the steps,
+    // every wave of it on its own row
+    const uint32_t stride = TILE ? 1u : gridDim.x * kD5Waves;
+    const uint32_t sp_end = TILE ? (uint32_t)(((uint64_t)blockIdx.x + 1u) * ta.total_steps / gridDim.x) : n_spans;
+    uint32_t sp = TILE ? (uint32_t)((uint64_t)blockIdx.x * ta.total_steps / gridDim.x) : blockIdx.x * kD5Waves + wave;
+    if (sp >= sp_end) return;
+    DtMfmaSink<kD5Region> sink;
+    if (TILE) {
+        sink.x = ta.x; sink.ldx = ta.ldx; sink.m = ta.m; sink.ws = ta.ws;
+        sink.out_f = P.out_f; sink.in_f = P.in_f; sink.spans_per_row = ta.spans_per_row; sink.n_pieces = ta.n_pieces;
+        sink.total_steps = ta.total_steps; sink.step_end = sp_end;
+        sink.wave = wave; sink.lane = lane; sink.wc = wc;
+        sink.tile_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)(d5_smem + kD5LutBytes);
+        sink.red = reinterpret_cast<float *>(d5_smem + kD5TileLds - kDtSumsBytes);
+        sink.acc = dt_f32x4{0.f, 0.f, 0.f, 0.f};
+    }
     // past the end the last span is fetched once more: loads that nobody uses
-    auto next_of = [&](uint32_t s) { return s + stride < n_spans ? s + stride : s; };
+    auto next_of = [&](uint32_t s) { return s + stride < sp_end ? s + stride : s; };
     Ranks q_now = table_of(sp);
     Shape g_now = shape_of(sp, q_now);
     Loads in_now = fetch(g_now, q_now);
     uint32_t sp_next = next_of(sp);
     Ranks q_next = table_of(sp_next);
     for (uint32_t turn = wave;; ++turn) {
-        {   // the waves that share a SIMD take turns at the issue priority, one span each
+        if (!TILE) {  // the waves that share a SIMD take turns at the issue priority, one span each (not where they
+                      // meet at a barrier every span)
             const uint32_t pr = turn % 3u;  // s_setprio takes an immediate
             if (pr == 0) __builtin_amdgcn_s_setprio(0);
             else if (pr == 1) __builtin_amdgcn_s_setprio(1);
@@ -500,6 +549,8 @@ k_decode34568_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units,
         const Loads in_next = fetch(g_next, q_next);
         const uint32_t sp_after = next_of(sp_next);
         const Ranks q_after = table_of(sp_after);
+        const DtStep step{sp / (TILE ? ta.spans_per_row : 1u), sp % (TILE ? ta.spans_per_row : 1u), sp};
+        if (TILE) sink.begin(step);
 
         const uint32_t p0 = g_now.p0, n_el = g_now.n_el;
         const uint32_t(&qa)[4] = q_now.qa;
@@ -623,9 +674,11 @@ k_decode34568_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units,
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
 
-        // ---- the lane's 64 bytes to their place in the output ----
+        // ---- the lane's 64 bytes to their place in the output (or to the tile, and the matrix pipe) ----
         uint16_t *dst = out + (size_t)p0 + 32 * lane;
-        if (n_el == kD5Span) {
+        if (TILE) {
+            sink.end(step, o);
+        } else if (n_el == kD5Span) {
             e_u32x4 *const rows = reinterpret_cast<e_u32x4 *>(wc);
 #pragma unroll
             for (int j = 0; j < 4; ++j) rows[lane * 5 + j] = e_u32x4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
@@ -648,7 +701,7 @@ k_decode34568_dense(Dev P, const int32_t *__restrict__ prefix, uint32_t n_units,
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        if (sp + stride >= n_spans) break;
+        if (sp + stride >= sp_end) break;
         sp = sp_next;
         q_now = q_next;
         g_now = g_next;
@@ -669,13 +722,42 @@ int launch_decode_dense34568(const Dev &P, const int32_t *prefix, uint16_t *o16,
     static const uint32_t resident = [] {
         int dev = 0, n_cu = 256, per_cu = 0;
         if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_decode34568_dense, kWave * kD5Waves, 0) != hipSuccess || per_cu < 1)
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_decode34568_dense<false>, kWave * kD5Waves, 0) != hipSuccess || per_cu < 1)
             per_cu = 3;
         return (uint32_t)n_cu * (uint32_t)per_cu;
     }();
     const uint32_t blocks = min(resident, (n_spans + kD5Waves - 1) / kD5Waves);
-    hipLaunchKernelGGL(k_decode34568_dense, dim3(blocks), dim3(kWave * kD5Waves), 0, s, P, prefix, n_units, n_spans, o16);
+    hipLaunchKernelGGL(k_decode34568_dense<false>, dim3(blocks), dim3(kWave * kD5Waves), 0, s, P, prefix, n_units, n_spans, o16,
+                       D5TileArgs{0, 0, 0, 0, nullptr, 0, 0, nullptr});
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
+}
+
+// 2..16 activation rows on dense five-level mixes: the decoder above in its tile mode
+bool gemv_dense34568_tiles_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x, int64_t ldx) {
+    return P.n_levels == 5 && P.bits[0] == 3 && P.bits[1] == 4 && P.bits[2] == 5 && P.bits[3] == 6 && P.bits[4] == 8 &&
+           chunk == kFastChunk && m >= 2 && m <= 16 && P.in_f % kFastChunk == 0 && P.in_f >= 2 * kFastChunk &&
+           ((uintptr_t)x & 15u) == 0 && (ldx & 7) == 0 && ((uintptr_t)P.last & 3u) == 0 && P.out_f != 0 &&
+           (uint64_t)P.out_f * P.in_f == P.n;
+}
+
+int launch_gemv_dense34568_tiles(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
+                                 int64_t ldy, float *ws, hipStream_t s) {
+    static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(k_decode34568_dense<true>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)kD5TileLds) == hipSuccess;
+    if (!raised) return IXH_EUNSUPPORTED;
+    static const uint32_t n_cu = [] {
+        int dev = 0, v = 256;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
+        return (uint32_t)v;
+    }();
+    const DtPlan plan = dt_plan(P.out_f, P.in_f, n_cu);
+    if (plan.groups == 0) return IXH_EUNSUPPORTED;
+    const uint32_t n_units = P.out_f * plan.n_chunks;
+    hipLaunchKernelGGL(k_decode34568_dense<true>, dim3(plan.groups), dim3(kWave * kDtWaves), kD5TileLds, s, P, prefix, n_units,
+                       0u, (uint16_t *)nullptr,
+                       D5TileArgs{plan.n_chunks, plan.spans_per_row, plan.total_steps, plan.n_pieces, x, m, ldx, ws});
+    if (hipGetLastError() != hipSuccess) return IXH_ELAUNCH;
+    return launch_reduce_chunks(ws, plan.n_pieces, m, P.out_f, y, ldy, s);
 }
 
 bool gemv_dense34568_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x) {

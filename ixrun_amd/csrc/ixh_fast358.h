@@ -32,6 +32,9 @@ int launch_gemv_dense34568(const Dev &P, const int32_t *prefix, const uint16_t *
                            bool atomic, hipStream_t s);
 bool decode_dense34568_supports(const Dev &P, uint32_t chunk, const int8_t *o8, const uint16_t *o16);
 int launch_decode_dense34568(const Dev &P, const int32_t *prefix, uint16_t *o16, hipStream_t s);
+bool gemv_dense34568_tiles_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x, int64_t ldx);
+int launch_gemv_dense34568_tiles(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
+                                 int64_t ldy, float *ws, hipStream_t s);
 bool gemv_dense358_tiles_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x, int64_t ldx);
 int launch_gemv_dense358_tiles(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
                                int64_t ldy, float *ws, hipStream_t s);

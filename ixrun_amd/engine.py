@@ -35,8 +35,8 @@ MAX_FUSED_ROWS = 16  # activation rows served by the fused decode+GEMV kernel
 # 23 / 31 / 31 us): every row count the fused kernels take.  Dense mixes (55 / 40 / 5 %): the pair takes
 # 91-93 us on the large layers and 34-52 us on 5120 x 5120, the fused kernels 54-62 / 69-73 / 79-85 / 80-85 / 83-88 us
 # (large layers) and 21 / 26 / 29 / 29 / 31 us (5120 x 5120) at M = 1 / 2 / 4 / 8 / 16: every row count as well.  Dense
-# mixes in other schemes have a level-by-level kernel for one row only (five levels: 95-104 us; the pair 127 us, the
-# any-scheme kernel 209-260 us at M = 2 .. 8).
+# five-level mixes: one row 97-105 us fused against 120 us for the pair; two to sixteen rows 113-126 us fused (the
+# decoder in its tile mode) against 119-123 us: the pair keeps those (the any-scheme kernel took 209-260 us).
 MAX_FUSED_ROWS_WITH_BUFFER = 16
 MAX_FUSED_ROWS_WITH_BUFFER_DENSE = 16
 # More rows than that: with a shared decode buffer the layer decodes into it and calls the library GEMM

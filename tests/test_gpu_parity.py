@@ -273,25 +273,27 @@ def test_gemv_fast_and_general(oracle, dev, kind, shape, m):
             check_outputs(y, y64, f"{kind} {shape} m={m} level-by-level kernel atomic={atomic}")
 
 
-@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("kind", KINDS + ["five_dense"])
 @pytest.mark.parametrize("shape", [(64, 1024), (37, 1024), (130, 1536), (256, 4608), (24, 8704), (21, 17408), (5, 25600), (300, 2048)])
 @pytest.mark.parametrize("cus", [0, 1, 3, 7])
-def test_gemv_dense_rows_on_the_matrix_pipe(oracle, dev, gemv_option, kind, shape, cus):
+@pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8)])
+def test_gemv_dense_rows_on_the_matrix_pipe(oracle, dev, gemv_option, kind, shape, cus, level_bits):
     """The level-by-level kernel for 2..16 activation rows that multiplies 16 rows' spans on the matrix pipe, forced
     for every mix: row counts that are not multiples of 16 (waves without a row), rows whose last span is short,
     the steps dealt to 1, 3, 7 or all workgroups, so that workgroups hold several row blocks and row blocks lie in
-    several workgroups (pieces added by the second kernel); and the kernel it replaced for 2..8 rows, still reachable."""
+    several workgroups (pieces added by the second kernel); the (3,5,8) kernel and the five-level one (the full
+    decoder in its tile mode); and the (3,5,8) kernel it replaced for 2..8 rows, still reachable."""
     from ixrun_amd import _lib
 
     out_f, in_f = shape
-    p = make_packed(kind, out_f, in_f)
+    p = make_packed(kind, out_f, in_f, level_bits)
     dp = device_packed(p, dev)
     w_bits = oracle.decode_packed_bf16(p)
     gemv_option("gemv_tile_cus", cus)
     for m in (2, 3, 8, 9, 16):
         x = activations(m, in_f, seed=m)
         y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
-        for dense_tiles in (1, 0, -1) if (m <= 8 and cus == 0) else (1,):
+        for dense_tiles in (1, 0, -1) if (m <= 8 and cus == 0 and len(level_bits) == 3) else (1,):
             gemv_option("gemv_dense_tiles", dense_tiles)
             y = run_gemv(dp, 512, x, m, dev, flags=_lib.IXH_GEMV_DENSE)
             check_outputs(y, y64, f"{kind} {shape} m={m} on {cus} CUs, gemv_dense_tiles={dense_tiles}")
