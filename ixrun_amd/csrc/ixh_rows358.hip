@@ -50,7 +50,7 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 // a wave's region: ring, record queue, row sums, task list, and a copy of the activations of its own column
 // blocks (c blocks x mt rows x 512 bf16) for the elements above level 1
 __host__ __device__ constexpr uint32_t wave_lds_bytes(int mt, int c) {
-    return kRStages * kRStageBytes + kRQueue * 16 + kRSlots * mt * 4 + kRTasks * 2 + (uint32_t)(c * mt) * kFastChunk * 2;
+    return kRStages * kRStageBytes + kRQueue * 16 + kRSlots * mt * 4 + kRTasks2 * 2 + (uint32_t)(c * mt) * kFastChunk * 2;
 }
 
 // byte offsets of the regions of a workgroup's LDS; the pair table is at 0, the splice masks follow
@@ -110,7 +110,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     uint4 *const queue = reinterpret_cast<uint4 *>(wave_base + kRStages * kRStageBytes);
     float *const rowacc = reinterpret_cast<float *>(wave_base + kRStages * kRStageBytes + kRQueue * 16);
     uint16_t *const tasks = reinterpret_cast<uint16_t *>(rowacc + kRSlots * MT);
-    uint32_t *const xs = reinterpret_cast<uint32_t *>(tasks + kRTasks);  // [MT][C * 512] bf16
+    uint32_t *const xs = reinterpret_cast<uint32_t *>(tasks + kRTasks2);  // [MT][C * 512] bf16
 
     // ---- workgroup set-up: table slices and x first (they wait on memory), then the tables built here ----
     const uint32_t unit0 = row0 * n_chunks;
@@ -443,10 +443,9 @@ constexpr int kXMaxWaves = 16;
 // by the wave that works on the neighbouring column block.
 constexpr int kXStages = 2;
 
-// a wave's region: ring, record queue (qcap records: 128, or 256 where a wave expects to fill the short one and LDS
-// holds the long one, which is resolved less often and in fuller batches), row sums (one per row of the workgroup and activation row), task list
+// a wave's region: ring, record queue (qcap records), row sums (one per row of the workgroup and activation row), task list
 __host__ __device__ constexpr uint32_t wave_lds_bytes_x(int mt, uint32_t rows_cap, uint32_t qcap) {
-    return kXStages * kRStageBytes + qcap * 16 + ((rows_cap * (uint32_t)mt * 4 + 15u) & ~15u) + kRTasks * 2;
+    return kXStages * kRStageBytes + qcap * 16 + ((rows_cap * (uint32_t)mt * 4 + 15u) & ~15u) + kRTasks2 * 2;
 }
 
 struct RowsXLds {
@@ -468,7 +467,7 @@ __host__ __device__ inline RowsXLds rowsx_layout(uint32_t rows_cap, uint32_t n_c
 
 // Five to eight activation rows (MT = 8) run with eight waves of up to 256 registers: the activations of a
 // unit-quad are 128 registers per lane.
-template <int MT, bool ANY, int QCAP>
+template <int MT, bool ANY>
 __global__ void __launch_bounds__((MT > 4 ? kXMaxWaves / 2 : kXMaxWaves) * kWave)
 k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t quads_per_wg, uint32_t flags,
                 const uint16_t *__restrict__ x, int m, int64_t ldx, uint16_t *__restrict__ y, int64_t ldy,
@@ -485,7 +484,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     const uint32_t n_steps = min(quads_per_wg, n_quads - quad0);
     const uint32_t row0 = quad0 * 4;
     const uint32_t rows_here = min(n_steps * 4, P.out_f - row0);
-    constexpr uint32_t qcap = QCAP;  // records the wave's queue holds
+    constexpr uint32_t qcap = kRQueue;  // records the wave's queue holds
     const uint32_t rows_cap = min(quads_per_wg * 4, P.out_f);
     const RowsXLds L = rowsx_layout(rows_cap, n_chunks, n_waves, MT, qcap);
 
@@ -506,7 +505,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     uint8_t *const ring = wave_base;
     uint4 *const queue = reinterpret_cast<uint4 *>(wave_base + kXStages * kRStageBytes);
     float *const rowacc = reinterpret_cast<float *>(wave_base + kXStages * kRStageBytes + qcap * 16);
-    uint16_t *const tasks = reinterpret_cast<uint16_t *>(wave_base + wave_lds_bytes_x(MT, rows_cap, qcap) - kRTasks * 2);
+    uint16_t *const tasks = reinterpret_cast<uint16_t *>(wave_base + wave_lds_bytes_x(MT, rows_cap, qcap) - kRTasks2 * 2);
 
     // ---- the activation row: needs nothing but the arguments, so it is requested first.  Lane (t, l) of the copy
     // fetches piece l * 4 + t of the block and the hardware puts it at piece t * 16 + l.
@@ -725,7 +724,10 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
             else if (turn == 2) __builtin_amdgcn_s_setprio(2);
             else if (turn == 3) __builtin_amdgcn_s_setprio(3);
 
-            if (qcount > qcap - kWave) resolve();  // keep room for a full wave of records
+            // Keep room for a full wave of records.  (A queue of 256 records emptied once, at the end, was 2 % faster
+            // where a wave collects 90 records and 20 % slower where it collects 140: what is resolved inside the loop
+            // hides behind the other waves' decoding.)
+            if (qcount > qcap - kWave) resolve();
             // refill the stage whose window was read last time (it is st_issue); make unit i+1 readable
             if (i + kXStages < n_mine) {
                 issue();
@@ -873,33 +875,31 @@ static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
         return v;
     }();
     static const bool raised =  // per instantiation
-        hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_rowsx<MT, ANY, 128>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit) == hipSuccess &&
-        hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_rowsx<MT, ANY, 256>),
+        hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_rowsx<MT, ANY>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit) == hipSuccess;
     if (!raised) return IXH_EUNSUPPORTED;
     // the answers for the last few shapes are kept (a model asks for the same handful over and over), under a
     // lock: a torn entry would launch one shape with another one's LDS layout
     struct Plan {
-        uint32_t chunks, out_f, waves, quads, qcap;
+        uint32_t chunks, out_f, waves, quads;
     };
     static Plan plans[8] = {};
     static uint32_t next_plan = 0;
     static std::mutex plans_lock;
-    uint32_t k_waves = 0, k_quads = 0, k_qcap = 0;
+    uint32_t k_waves = 0, k_quads = 0;
     {
         std::lock_guard<std::mutex> guard(plans_lock);
         const Plan *hit = nullptr;
         for (const Plan &pl : plans)
             if (pl.chunks == n_chunks && pl.out_f == P.out_f) hit = &pl;
         if (!hit) {
-            uint32_t waves = 0, quads = 0, qcap = 0;
+            uint32_t waves = 0, quads = 0;
             for (uint32_t w : {16u, 12u, 8u}) {
                 if (MT > 4 && w > (uint32_t)kXMaxWaves / 2) continue;
                 const size_t probe = rowsx_layout(min(16u, P.out_f), n_chunks, w, MT, kRQueue).total;
                 int per_cu = 0;
                 if (probe > kLdsLimit ||
-                    hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rowsx<MT, ANY, 128>, (int)(w * kWave),
+                    hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rowsx<MT, ANY>, (int)(w * kWave),
                                                                  probe) != hipSuccess || per_cu < 1)
                     continue;
                 // whole rounds of resident workgroups, each with a contiguous run of at most 16 row quads
@@ -910,36 +910,23 @@ static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
                 if (rowsx_layout(min(q * 4, P.out_f), n_chunks, w, MT, kRQueue).total > kLdsLimit) continue;
                 waves = w;
                 quads = q;
-                // A longer queue pays where a wave fills the short one before it is through (5120 x 5120 with 1.8 %
-                // of the elements above level 1: -3 %); where it never does, the larger LDS footprint costs 1 %.
-                // Records a wave expects: its unit-quads x 64 lanes x the chance of a bitmap word with a zero bit.
-                qcap = kRQueue;
-                const double l1_share = min(1.0, (double)P.st_words[0] * (32.0 / 3.0) / (double)P.n);
-                const double expected = (double)((q * n_chunks + w - 1) / w) * 64.0 * (1.0 - pow(l1_share, 32.0));
-                if (expected > 0.75 * kRQueue && rowsx_layout(min(q * 4, P.out_f), n_chunks, w, MT, 256).total <= kLdsLimit)
-                    qcap = 256;
                 break;
             }
             Plan &slot = plans[next_plan++ % 8u];
-            slot = Plan{n_chunks, P.out_f, waves, quads, qcap};
+            slot = Plan{n_chunks, P.out_f, waves, quads};
             hit = &slot;
         }
         k_waves = hit->waves;
         k_quads = hit->quads;
-        k_qcap = hit->qcap;
     }
     if (k_waves == 0) return IXH_EUNSUPPORTED;
     const uint32_t waves = k_waves, quads = k_quads;
     const uint32_t groups = (n_quads + quads - 1) / quads;
     uint32_t flags = 0;
     if (((uintptr_t)P.last & 3u) == 0) flags |= kFlagStageSide;
-    const size_t lds = rowsx_layout(min(quads * 4, P.out_f), n_chunks, waves, MT, k_qcap).total;
-    if (k_qcap == 256)
-        hipLaunchKernelGGL((k_gemv358_rowsx<MT, ANY, 256>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix,
-                           n_chunks, quads, flags, x, m, ldx, y, ldy, y32);
-    else
-        hipLaunchKernelGGL((k_gemv358_rowsx<MT, ANY, 128>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix,
-                           n_chunks, quads, flags, x, m, ldx, y, ldy, y32);
+    const size_t lds = rowsx_layout(min(quads * 4, P.out_f), n_chunks, waves, MT, kRQueue).total;
+    hipLaunchKernelGGL((k_gemv358_rowsx<MT, ANY>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks, quads,
+                       flags, x, m, ldx, y, ldy, y32);
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }
 

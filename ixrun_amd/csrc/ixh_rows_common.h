@@ -13,6 +13,7 @@ constexpr int kRStages = 3;              // unit-quads in flight per wave
 constexpr uint32_t kRStageBytes = 1280;  // 1024 stream + 256 bitmap
 constexpr uint32_t kRQueue = 128;        // records per wave
 constexpr uint32_t kRTasks = 192;        // elements above level 1 of 64 records that are spread over the lanes
+constexpr uint32_t kRTasks2 = 320;       // the same for the kernels that resolve 128 records at a time
 constexpr uint32_t kRSlots = 64;         // rows per workgroup at most
 constexpr int kRMaxWaves = 12;           // waves per workgroup at most: 3 per SIMD, up to 168 VGPRs each
 constexpr uint32_t kRLutBytes = 64 * 32 * 4;
@@ -101,6 +102,30 @@ __device__ __forceinline__ void lds_add_f32_raw(uint32_t addr, float v) {  // co
     asm volatile("ds_add_f32 %0, %1" ::"v"(addr), "v"(v) : "memory");
 }
 
+// Sums over runs of equal keys among neighbouring lanes of a 16-lane row (a segmented scan in four DPP steps):
+// v becomes the sum of the run's values up to and including this lane; returns true in the last lane of a run.
+// Used in front of LDS atomics whose lanes mostly target a handful of addresses: the elements of one weight row come
+// in runs, and lanes that add to one address are served one after the other.
+template <int MT>
+__device__ __forceinline__ bool run_sums(uint32_t key, float (&v)[MT], uint32_t lane) {
+    const uint32_t k1 = key + 1u;  // never 0, which is what a row's first lane reads from "the lane below"
+    const uint32_t head = dpp_shr(k1, 1) != k1 ? 1u : 0u;
+    uint32_t f = head;
+#pragma unroll
+    for (int d = 1; d < 16; d <<= 1) {
+        const uint32_t fs = dpp_shr(f, d);
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            const float vs = __uint_as_float(dpp_shr(__float_as_uint(v[j]), d));
+            v[j] += f ? 0.0f : vs;
+        }
+        f |= fs;
+    }
+    // the head flag of the lane above (row_shl:1; a row's last lane reads 0 and is a tail anyway)
+    const uint32_t next_head = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)head, 0x101, 0xf, 0xf, true);
+    return next_head != 0 || (lane & 15u) == 15u;
+}
+
 // inclusive sum over the lanes at or below this one
 __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
     v = row_scan(v);
@@ -140,6 +165,8 @@ struct TaskPool {
 // round of at most 64 elements (its argument: the lanes below that number may have taken part).
 // A sink also brings its own record format: 8 bytes, the bitmap word and a word that unpack() turns into the
 // fields of the 16-byte record (rank of the word's first element in bitmap 1's domain, unit, column, row field).
+struct Now { static constexpr bool value = false; };    // one(): add the element's products to the row sums
+struct Later { static constexpr bool value = true; };  // one(): leave them to the caller
 struct NoSink {
     static constexpr bool active = false;
     __device__ __forceinline__ void unpack(uint32_t, uint32_t, uint32_t, uint32_t &, uint32_t &, uint32_t &, uint32_t &) {}
@@ -189,8 +216,12 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
         }
         return r < P.last_bytes ? (int)P.last[r] - 127 : 0;
     };
-    // element `e` (bit of the record's word), the nth element above level 1 of its record
-    auto one = [&](const uint4 rec, uint32_t nth, uint32_t e) {
+    // element `e` (bit of the record's word), the nth element above level 1 of its record; with Later the products
+    // are not added to the row sums here but left in d_p / d_slot for the caller (XL != 2 only)
+    float d_p[XL == 2 ? 1 : MT];
+    uint32_t d_slot = 0;
+    auto one = [&](const uint4 rec, uint32_t nth, uint32_t e, auto when) {
+        constexpr bool kDefer = decltype(when)::value && XL != 2;
         uint32_t r0_lane = rec.y, unit = rec.z, k0 = rec.w & 0xFFFFu;
         uint32_t slot = rec.w >> 16;
         if (SINK::active) sink.unpack(rec.y, unit0, tq1_addr, r0_lane, unit, k0, slot);
@@ -226,6 +257,12 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
             const float w = dequant(value_any(unit, r0_lane + nth), scale);
             if (XL == 2) {
                 add_all(w);
+                return;
+            }
+            if (kDefer) {
+                d_slot = slot;
+#pragma unroll
+                for (int j = 0; j < (XL == 2 ? 0 : MT); ++j) d_p[j] = j < m ? bf16_bits_to_f32(xe[j]) * w : 0.0f;
                 return;
             }
 #pragma unroll
@@ -275,6 +312,12 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
             add_all(w);
             return;
         }
+        if (kDefer) {
+            d_slot = slot;
+#pragma unroll
+            for (int j = 0; j < (XL == 2 ? 0 : MT); ++j) d_p[j] = j < m ? bf16_bits_to_f32(xe[j]) * w : 0.0f;
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < MT; ++j)
             if (j < m) lds_add_f32_raw(rowacc_addr + (slot * MT + j) * 4, bf16_bits_to_f32(xe[j]) * w);
@@ -285,54 +328,85 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
             if (t < pool.total) {
                 const uint32_t task = lds_u32(pool.addr + t * 4u);
                 const u32x4 rv = lds_u128(pool.queues_addr + (task >> 18) * pool.queue_stride + ((task >> 10) & 255u) * 16u);
-                one(make_uint4(rv.x, rv.y, rv.z, rv.w), (task >> 5) & 31u, task & 31u);
+                one(make_uint4(rv.x, rv.y, rv.z, rv.w), (task >> 5) & 31u, task & 31u, Now{});
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         return;
     }
-    for (uint32_t base = 0; base < count; base += kWave) {
-        const uint32_t idx = base + lane;
-        const bool has = idx < count;
-        uint4 rec = make_uint4(0, 0, 0, 0);
-        if (has) rec = read_record<SINK::active>(queue, idx);
-        uint32_t zeros = rec.x;
-        const uint32_t mine = (uint32_t)__popc(zeros);
-        const uint32_t incl = wave_scan(mine);
-        const uint32_t n_tasks = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
-        if (n_tasks <= kRTasks) {
-            uint32_t t = incl - mine, nth = 0;
-            while (zeros != 0) {
-                tasks[t++] = (uint16_t)((lane << 10) | (nth++ << 5) | (uint32_t)__builtin_ctz(zeros));
-                zeros &= zeros - 1;
-            }
+    // Batches of up to 128 records, two per lane (A: record base + lane, B: base + 64 + lane): one scan, one task list
+    // (A's elements first, then B's, kRTasks2 at most) and full rounds for a wave that comes with 65..128 records.
+    // With a sink, whose kernel has no register to spare, and with XL == 2: 64 records, one per lane, kRTasks elements.
+    constexpr bool kTwo = !SINK::active && XL != 2;
+    constexpr uint32_t kTaskCap = kTwo ? kRTasks2 : kRTasks;
+    for (uint32_t base = 0; base < count; base += (kTwo ? 2 : 1) * kWave) {
+        const uint32_t idx_a = base + lane, idx_b = idx_a + kWave;
+        uint32_t zeros_a = 0, zeros_b = 0;
+        if (idx_a < count) zeros_a = read_record<SINK::active>(queue, idx_a).x;
+        if (kTwo && idx_b < count) zeros_b = read_record<SINK::active>(queue, idx_b).x;
+        const uint32_t mine_a = (uint32_t)__popc(zeros_a), mine_b = (uint32_t)__popc(zeros_b);
+        const uint32_t incl = wave_scan(mine_a | (mine_b << 16));  // at most 64 x 32 elements each: 12 bits
+        const uint32_t totals = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+        const uint32_t n_a = totals & 0xFFFFu, n_tasks = n_a + (totals >> 16);
+        if (n_tasks <= kTaskCap) {
+            // task = record of the batch << 5 | bit of its word
+            for (uint32_t t = (incl & 0xFFFFu) - mine_a; zeros_a != 0; zeros_a &= zeros_a - 1)
+                tasks[t++] = (uint16_t)((lane << 5) | (uint32_t)__builtin_ctz(zeros_a));
+            if (kTwo)
+                for (uint32_t t = n_a + (incl >> 16) - mine_b; zeros_b != 0; zeros_b &= zeros_b - 1)
+                    tasks[t++] = (uint16_t)(((lane + kWave) << 5) | (uint32_t)__builtin_ctz(zeros_b));
+            // Without a sink the products of a round are summed over runs of one weight row first (the tasks are in
+            // record order, so a row's elements sit in neighbouring lanes), and only the last lane of a run adds.
+            constexpr bool kRuns = !SINK::active && XL != 2;
             for (uint32_t tb = 0; tb < n_tasks; tb += kWave) {
+                if (kRuns) {
+                    d_slot = ~1u;  // lanes without an element: a key no row has
+#pragma unroll
+                    for (int j = 0; j < (XL == 2 ? 0 : MT); ++j) d_p[j] = 0.0f;
+                }
                 if (tb + lane < n_tasks) {
                     const uint32_t task = tasks[tb + lane];
-                    one(read_record<SINK::active>(queue, base + (task >> 10)), (task >> 5) & 31u, task & 31u);
+                    const uint4 rec = read_record<SINK::active>(queue, base + (task >> 5));
+                    const uint32_t e = task & 31u;
+                    one(rec, (uint32_t)__popc(rec.x & ((1u << e) - 1u)), e, Later{});
                 } else if (SINK::active) {
                     sink.idle();
                 }
                 if (SINK::active) sink.flush(n_tasks - tb);
+                if (kRuns) {
+                    const bool tail = run_sums<(XL == 2 ? 1 : MT)>(d_slot, d_p, lane);
+                    if (tail && d_slot != ~1u) {
+#pragma unroll
+                        for (int j = 0; j < (XL == 2 ? 0 : MT); ++j)
+                            if (j < m) lds_add_f32_raw(rowacc_addr + (d_slot * MT + j) * 4, d_p[j]);
+                    }
+                }
             }
-        } else if (SINK::active) {
-            uint32_t nth = 0;
-            for (uint64_t left = __ballot(zeros != 0); left != 0; left = __ballot(zeros != 0)) {
-                if (zeros != 0) {
+            continue;
+        }
+        // more elements than the task list holds: every lane walks its own records, A then B
+        for (uint32_t half = 0; half < (kTwo ? 2u : 1u); ++half) {
+            const uint32_t idx = half == 0 ? idx_a : idx_b;
+            uint4 rec = make_uint4(0, 0, 0, 0);
+            if (idx < count) rec = read_record<SINK::active>(queue, idx);
+            uint32_t zeros = rec.x, nth = 0;
+            if (SINK::active) {
+                for (uint64_t left = __ballot(zeros != 0); left != 0; left = __ballot(zeros != 0)) {
+                    if (zeros != 0) {
+                        const uint32_t e = (uint32_t)__builtin_ctz(zeros);
+                        zeros &= zeros - 1;
+                        one(rec, nth++, e, Now{});
+                    } else {
+                        sink.idle();
+                    }
+                    sink.flush(64u - (uint32_t)__builtin_clzll(left));
+                }
+            } else {
+                while (zeros != 0) {
                     const uint32_t e = (uint32_t)__builtin_ctz(zeros);
                     zeros &= zeros - 1;
-                    one(rec, nth++, e);
-                } else {
-                    sink.idle();
+                    one(rec, nth++, e, Now{});
                 }
-                sink.flush(64u - (uint32_t)__builtin_clzll(left));
-            }
-        } else {
-            uint32_t nth = 0;
-            while (zeros != 0) {
-                const uint32_t e = (uint32_t)__builtin_ctz(zeros);
-                zeros &= zeros - 1;
-                one(rec, nth++, e);
             }
         }
     }
