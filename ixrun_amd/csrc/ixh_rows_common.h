@@ -336,8 +336,8 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
     }
     // Batches of up to 128 records, two per lane (A: record base + lane, B: base + 64 + lane): one scan, one task list
     // (A's elements first, then B's, kRTasks2 at most) and full rounds for a wave that comes with 65..128 records.
-    // With a sink, whose kernel has no register to spare, and with XL == 2: 64 records, one per lane, kRTasks elements.
-    constexpr bool kTwo = !SINK::active && XL != 2;
+    // With XL == 2 and no sink: 64 records, one per lane, kRTasks elements.
+    constexpr bool kTwo = SINK::active || XL != 2;
     constexpr uint32_t kTaskCap = kTwo ? kRTasks2 : kRTasks;
     for (uint32_t base = 0; base < count; base += (kTwo ? 2 : 1) * kWave) {
         const uint32_t idx_a = base + lane, idx_b = idx_a + kWave;

@@ -50,7 +50,7 @@ constexpr size_t kTLdsLimit = 160 * 1024;
 constexpr uint32_t kTStripBytes = 272;
 
 struct TilesLds {
-    uint32_t tq1, tq2, side, xs, xs_row, zero, partial, waves, wave_bytes, tasks_off, total;
+    uint32_t tq1, tq2, side, xs, xs_row, zero, partial, waves, wave_bytes, tasks_off, round_off, total;
 };
 
 // x_blocks: column blocks of the activation rows that LDS holds at a time
@@ -73,16 +73,18 @@ __host__ __device__ inline TilesLds tiles_layout(uint32_t rows_cap, uint32_t n_c
     L.zero = L.xs + max((uint32_t)m * L.xs_row, partial_bytes);
     L.waves = (L.zero + kTStripBytes + 15u) & ~15u;
     L.tasks_off = qcap * 8u;  // behind the queue of 8-byte records
-    L.wave_bytes = (L.tasks_off + kRTasks * 2u + 15u) & ~15u;
+    L.round_off = (L.tasks_off + kRTasks2 * 2u + 15u) & ~15u;  // the elements of a round: {weight | column, address}
+    L.wave_bytes = L.round_off + kWave * 8u;
     L.total = L.waves + n_waves * L.wave_bytes;
     return L;
 }
 
 // The resolved elements above level 1 of a round go through the matrix pipe like the others, into the same
-// accumulators: every lane keeps its element's weight, the column n of the product it belongs to and the LDS address of
-// its activation in row 0; then, sixteen elements per instruction, lane (n, kg) fetches elements 4 kg .. 4 kg + 3 from
-// the lanes that hold them and gathers the activations of its row as one operand and, as the other, the weights of the
-// elements that belong to column n (zero for the rest).  Few registers are free where this runs: one pair at a time.
+// accumulators: every lane writes its element's weight, the column n of the product it belongs to and the LDS address of
+// its activation in row 0 to the wave's list of the round; then, sixteen elements per instruction, lane (n, kg) reads
+// elements 4 kg .. 4 kg + 3 (32 consecutive bytes, the same for the 16 lanes of a k group) and gathers the activations
+// of its row as one operand and, as the other, the weights of the elements that belong to column n (zero for the rest).
+// (Fetching the four elements from the lanes that hold them, eight ds_bpermute a group, took 1.6 times as long.)
 struct TileSink {
     static constexpr bool active = true;
     f32x4 acc;           // the wave's accumulators: taken over for the time of the resolver, handed back after it
@@ -92,6 +94,7 @@ struct TileSink {
     uint32_t idle_addr;  // an address that can be read
     uint32_t wn, xa;     // the lane's element of the round: weight bits | column << 16, address
     uint32_t n_chunks;
+    uint32_t round_addr;  // the wave's list of a round's elements, 8 bytes each
     // a record's second word: column n of the product << 27 | row in the workgroup << 20 | column / 32 << 9 | level-1
     // elements between the unit's start and the word
     __device__ __forceinline__ void unpack(uint32_t packed, uint32_t unit0, uint32_t tq1_addr, uint32_t &r0, uint32_t &unit,
@@ -112,25 +115,19 @@ struct TileSink {
     }
     // lanes: the lanes below this number may hold an element
     __device__ __forceinline__ void flush(uint32_t lanes) {
+        *reinterpret_cast<__attribute__((address_space(3))) u32x2 *>((uintptr_t)(round_addr + (kg * 16u + n) * 8u)) = u32x2{wn, xa};
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             if ((uint32_t)g * 16u >= lanes) break;
-            uint32_t ap[2], bp[2];
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int src = (int)(((uint32_t)g * 16u + kg * 4u + 2u * (uint32_t)h) * 4u);
-                const uint32_t e0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)wn);
-                const uint32_t e1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src + 4, (int)wn);
-                const uint32_t a0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)xa);
-                const uint32_t a1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src + 4, (int)xa);
-                const uint32_t x0 = lds_u16(a0 + x_off), x1 = lds_u16(a1 + x_off);
-                const uint32_t w0 = (e0 >> 16) == n ? (e0 & 0xFFFFu) : 0u, w1 = (e1 >> 16) == n ? e1 << 16 : 0u;
-                ap[h] = x_on ? (x0 | (x1 << 16)) : 0u;
-                bp[h] = w0 | w1;
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, u32x2{ap[0], ap[1]}),
-                                                           __builtin_bit_cast(s16x4, u32x2{bp[0], bp[1]}), acc, 0, 0, 0);
+            const uint32_t at = round_addr + ((uint32_t)g * 16u + kg * 4u) * 8u;
+            const u32x4 p = lds_u128(at), q = lds_u128(at + 16u);  // {wn, xa} of elements 4 kg, 4 kg + 1 | + 2, + 3
+            const uint32_t x0 = lds_u16(p.y + x_off), x1 = lds_u16(p.w + x_off);
+            const uint32_t x2 = lds_u16(q.y + x_off), x3 = lds_u16(q.w + x_off);
+            const uint32_t w0 = (p.x >> 16) == n ? (p.x & 0xFFFFu) : 0u, w1 = (p.z >> 16) == n ? p.z << 16 : 0u;
+            const uint32_t w2 = (q.x >> 16) == n ? (q.x & 0xFFFFu) : 0u, w3 = (q.z >> 16) == n ? q.z << 16 : 0u;
+            const u32x2 ap = {x_on ? (x0 | (x1 << 16)) : 0u, x_on ? (x2 | (x3 << 16)) : 0u};
+            const u32x2 bp = {w0 | w1, w2 | w3};
+            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, ap), __builtin_bit_cast(s16x4, bp), acc, 0, 0, 0);
         }
     }
 };
@@ -319,7 +316,8 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
     uint32_t qcount = 0;  // wave-uniform
     auto resolve = [&]() {
-        TileSink sink{acc, n, kg, r * L.xs_row, r < (uint32_t)m, xs_addr, 0u, xs_addr, n_chunks};
+        TileSink sink{acc, n, kg, r * L.xs_row, r < (uint32_t)m, xs_addr, 0u, xs_addr, n_chunks,
+                      L.waves + wave * L.wave_bytes + L.round_off};
         const TaskPool none{0, 0, 0, 1, 0, 0};
         if (ANY)
             resolve_rows_to<kTMaxM, false, true, 2, false, kTStripBytes>(
