@@ -193,13 +193,16 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
             const uint32_t qu = (uint32_t)prefix[(size_t)i * entries + unit];  // level-i elements before the unit
             const uint32_t wf = ru >> 5, wl = min(r >> 5, wf + 17u);
             const uint32_t first_mask = ~0u << (ru & 31);
-            uint32_t cnt = 0;
-            for (uint32_t w = wf; w < wl; ++w) {
-                uint32_t bits = w < words ? bm[w] : 0u;
-                if (w == wf) bits &= first_mask;
-                cnt += __popc(bits);
+            // the first two words are asked for together with the table entry: where few elements are above level 1
+            // the element's bit is in one of them, and the chain is one trip to memory long instead of three
+            const uint32_t word0 = wf < words ? bm[wf] : 0u, word1 = wf + 1 < words ? bm[wf + 1] : 0u;
+            uint32_t cnt = wl > wf ? __popc(word0 & first_mask) : 0u;
+            uint32_t bits = wl == wf ? word0 : word1;
+            if (wl > wf + 1) {
+                cnt += __popc(word1);
+                for (uint32_t w = wf + 2; w < wl; ++w) cnt += __popc(w < words ? bm[w] : 0u);
+                bits = wl < words ? bm[wl] : 0u;
             }
-            const uint32_t bits = wl < words ? bm[wl] : 0u;
             uint32_t low = (1u << (r & 31)) - 1u;
             if (wl == wf) low &= first_mask;
             cnt += __popc(bits & low);
@@ -277,14 +280,18 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
         const uint32_t r = r0_lane + nth;
         // level-2 elements among bitmap-1 bits [r0u, r) (a unit spans at most 17 words), and the bit at r
         const uint32_t wl = min(r >> 5, wf + 17u);
-        uint32_t cnt = 0;
-        for (uint32_t w = wf; w < wl; ++w) {
-            uint32_t bits = STAGED ? lds_u32(sv.base + kRSideB2 + (w - sv.b2w0) * 4) : (w < b2_words ? b2[w] : 0u);
-            if (w == wf) bits &= first_mask;
-            cnt += __popc(bits);
+        // the first two words together (see value_any); a staged word past the share's end is a word of the next region
+        auto b2_word = [&](uint32_t w) {
+            return STAGED ? lds_u32(sv.base + kRSideB2 + (w - sv.b2w0) * 4) : (w < b2_words ? b2[w] : 0u);
+        };
+        const uint32_t word0 = b2_word(wf), word1 = b2_word(wf + 1);
+        uint32_t cnt = wl > wf ? __popc(word0 & first_mask) : 0u;
+        uint32_t bits = wl == wf ? word0 : word1;
+        if (wl > wf + 1) {
+            cnt += __popc(word1);
+            for (uint32_t w = wf + 2; w < wl; ++w) cnt += __popc(b2_word(w));
+            bits = b2_word(wl);
         }
-        const uint32_t bits = STAGED ? lds_u32(sv.base + kRSideB2 + (wl - sv.b2w0) * 4)
-                                     : (wl < b2_words ? b2[wl] : 0u);
         uint32_t low = (1u << (r & 31)) - 1u;
         if (wl == wf) low &= first_mask;
         cnt += __popc(bits & low);
