@@ -79,6 +79,7 @@ WORKLOADS = {
     "attn_proj_5120x5120_m4_student_t": (5120, 5120, 4, "student_t"),
     "attn_proj_5120x5120_m8_student_t": (5120, 5120, 8, "student_t"),
     "attn_proj_5120x5120_m16_student_t": (5120, 5120, 16, "student_t"),
+    "gate_up_17408x5120_m1_student_t": (17408, 5120, 1, "student_t"),
     "gate_up_17408x5120_m2_student_t": (17408, 5120, 2, "student_t"),
     "gate_up_17408x5120_m4_student_t": (17408, 5120, 4, "student_t"),
     "gate_up_17408x5120_m8_student_t": (17408, 5120, 8, "student_t"),
@@ -460,7 +461,7 @@ def also_block(dev, args):
                                               + [(f"down_proj_5120x17408_m{m}_student_t", m, "fused") for m in (4, 8, 16)]),
         ("attn_proj_5120x5120_m1_student_t", [("attn_proj_5120x5120_m1_student_t", 1, "fused")]
                                              + [(f"attn_proj_5120x5120_m{m}_student_t", m, "fused") for m in (4, 8, 16)]),
-        ("gate_up_17408x5120_m2_student_t", [(f"gate_up_17408x5120_m{m}_student_t", m, "fused") for m in (2, 4, 8, 16)]),
+        ("gate_up_17408x5120_m2_student_t", [(f"gate_up_17408x5120_m{m}_student_t", m, "fused") for m in (1, 2, 4, 8, 16)]),
         ("graph64_5120x5120_m1_student_t", [("graph64_5120x5120_m1_student_t", 1, "fused")]),
         ("prefill_5120x17408_m512_five_level", [("prefill_5120x17408_m512_five_level", 512, "fused"),
                                                 ("prefill_5120x17408_m512_five_level", 512, "unfused")]),

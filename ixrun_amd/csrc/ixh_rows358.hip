@@ -438,6 +438,7 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
 // with k_gemv358_rows), which leaves the lanes one addition per table or bitmap address: a lane constant plus the
 // scalar index of the unit-quad.
 constexpr int kXMaxWaves = 16;
+constexpr uint32_t kXSlots = 128;  // rows per workgroup at most
 // Unit-quads in flight per wave, the one being read included.  Two: measured against three and four (with 16 waves
 // per CU), every stage more costs 2-3 %; fewer copies in flight leave more of a CU's cache lines to be found again
 // by the wave that works on the neighbouring column block.
@@ -902,12 +903,22 @@ static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
                     hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemv358_rowsx<MT, ANY>, (int)(w * kWave),
                                                                  probe) != hipSuccess || per_cu < 1)
                     continue;
-                // whole rounds of resident workgroups, each with a contiguous run of at most 16 row quads
-                const uint32_t resident = (uint32_t)n_cu * (uint32_t)per_cu;
-                const uint32_t rounds = (n_quads + resident * (kRSlots / 4) - 1) / (resident * (kRSlots / 4));
-                uint32_t q = (n_quads + rounds * resident - 1) / (rounds * resident);
-                q = max(1u, min(q, kRSlots / 4));
-                if (rowsx_layout(min(q * 4, P.out_f), n_chunks, w, MT, kRQueue).total > kLdsLimit) continue;
+                // Whole rounds of resident workgroups, as few as LDS admits (every round pays the set-up, the last
+                // resolve and the final sums again: 17408 x 5120 in two rounds of 9 row quads took 22.4 us, in one of
+                // 17 it takes 19), each workgroup with a contiguous run of at most kXSlots / 4 row quads.
+                uint32_t q = 0;
+                for (uint32_t rounds = 1; rounds <= 64 && q == 0; ++rounds) {
+                    uint32_t groups_at_once = (uint32_t)n_cu * (uint32_t)per_cu;
+                    uint32_t cand = max(1u, (n_quads + rounds * groups_at_once - 1) / (rounds * groups_at_once));
+                    size_t total = rowsx_layout(min(cand * 4, P.out_f), n_chunks, w, MT, kRQueue).total;
+                    if (per_cu > 1 && total * (size_t)per_cu > kLdsLimit) {  // fewer of these fit a CU than of the probe
+                        groups_at_once = (uint32_t)n_cu * (uint32_t)max((size_t)1, kLdsLimit / max(total, (size_t)1));
+                        cand = max(1u, (n_quads + rounds * groups_at_once - 1) / (rounds * groups_at_once));
+                        total = rowsx_layout(min(cand * 4, P.out_f), n_chunks, w, MT, kRQueue).total;
+                    }
+                    if (cand <= kXSlots / 4 && total <= kLdsLimit) q = cand;
+                }
+                if (q == 0) continue;
                 waves = w;
                 quads = q;
                 break;

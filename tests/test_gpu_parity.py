@@ -551,6 +551,24 @@ def test_reference_call_surface(oracle, dev, shape):
         assert rel_l2(got, want) < 6e-3  # bias add and output are bf16-rounded
 
 
+@pytest.mark.parametrize("kind", ["outlier", "student_t", "rare_other", "only_l3"])
+@pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8)])
+def test_gemv_many_rows_to_a_workgroup(oracle, dev, kind, level_bits):
+    """More rows than 256 workgroups hold at 64 apiece (16640 rows: 68 to a workgroup, in one round): the row-block
+    kernel with row slots above 63, for one and two activation rows, dense mixes forced onto it as well (every lane
+    with elements above level 1, the queue resolved inside the loop)."""
+    from ixrun_amd import _lib
+
+    out_f, in_f = 16640, 512
+    p = make_packed(kind, out_f, in_f, level_bits)
+    dp = device_packed(p, dev)
+    w_bits = oracle.decode_packed_bf16(p)
+    for m in (1, 2):
+        x = activations(m, in_f, seed=m)
+        y = run_gemv(dp, 512, x, m, dev, flags=_lib.IXH_GEMV_FORCE_358)
+        check_outputs(y, oracle.gemm_f64(w_bits, bf16_bits(x)), f"{kind} {level_bits} {out_f}x{in_f} m={m}")
+
+
 @pytest.fixture(scope="module")
 def gate_up_layer(oracle, dev):
     """BASELINE config 4's layer, 17408 x 5120 Student-t, packed once for its four batch sizes."""
@@ -561,11 +579,11 @@ def gate_up_layer(oracle, dev):
     return StreamingLinear(p), w_bits
 
 
-@pytest.mark.parametrize("m", [2, 4, 8, 16])
+@pytest.mark.parametrize("m", [1, 2, 4, 8, 16])
 def test_full_size_config4_every_batch(oracle, dev, gate_up_layer, m):
-    """BASELINE config 4 as stated: 17408 x 5120 with M in {2, 4, 8, 16} activation rows, each through the kernel the
-    library picks for it (2 rows: the row-block kernel; 4, 8 and 16 rows: the tile kernel, at 16 rows with the
-    activations in two column parts)."""
+    """BASELINE config 4 as stated: 17408 x 5120 with M in {2, 4, 8, 16} activation rows, and one row, each through the
+    kernel the library picks for it (1 and 2 rows: the row-block kernel, 68 rows to a workgroup; 4, 8 and 16 rows: the
+    tile kernel, at 16 rows with the activations in two column parts)."""
     sl, w_bits = gate_up_layer
     x = activations(m, 5120, seed=1)
     y = sl(x.to(dev))
