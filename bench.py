@@ -90,6 +90,9 @@ WORKLOADS = {
     "gate_up_17408x5120_m8_calibrated": (17408, 5120, 8, "calibrated"),
     "gate_up_17408x5120_m16_calibrated": (17408, 5120, 16, "calibrated"),
     "down_proj_5120x17408_m8_calibrated": (5120, 17408, 8, "calibrated"),
+    # dense five-level mixes at several rows: the five-level decoder's tile mode
+    "down_proj_5120x17408_m8_five_level_calibrated": (5120, 17408, 8, "calibrated", (3, 4, 5, 6, 8)),
+    "gate_up_17408x5120_m8_five_level_calibrated": (17408, 5120, 8, "calibrated", (3, 4, 5, 6, 8)),
     "attn_proj_5120x5120_m8_calibrated": (5120, 5120, 8, "calibrated"),
     # 64 distinct 5120x5120 layers chained (each output feeds the next layer), one hipGraph: us per layer
     "graph64_5120x5120_m1_student_t": (5120, 5120, 1, "student_t"),
