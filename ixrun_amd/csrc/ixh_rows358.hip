@@ -508,6 +508,9 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     float *const rowacc = reinterpret_cast<float *>(wave_base + kXStages * kRStageBytes + qcap * 16);
     uint16_t *const tasks = reinterpret_cast<uint16_t *>(wave_base + wave_lds_bytes_x(MT, rows_cap, qcap) - kRTasks2 * 2);
 
+    // the scale is asked for here, with the first requests: read where the pair table is built, it was a trip to memory
+    // of its own between the table slices' and the barrier
+    const uint16_t scale_bits = *P.scale;
     // ---- the activation row: needs nothing but the arguments, so it is requested first.  Lane (t, l) of the copy
     // fetches piece l * 4 + t of the block and the hardware puts it at piece t * 16 + l.
     {
@@ -528,7 +531,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         tq1[i] = (uint32_t)prefix[unit0 + i];
         if (!ANY) tq2[i] = (uint32_t)prefix[entries + unit0 + i];
     }
-    const float scale = bf16_bits_to_f32(*P.scale);
+    const float scale = bf16_bits_to_f32(scale_bits);
     for (uint32_t i = tid; i < 64 * 32; i += blockDim.x) {
         const int c0 = (i >> 5) & 7, c1 = i >> 8;
         const f32x2 w = {c0 < 7 ? (float)(c0 - 3) * scale : 0.0f, c1 < 7 ? (float)(c1 - 3) * scale : 0.0f};

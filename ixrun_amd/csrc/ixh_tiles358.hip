@@ -161,6 +161,7 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         }
         return;
     }
+    const uint16_t scale_bits = *P.scale;  // asked for with the first requests, not where the pair table is built
     uint32_t *const lut = reinterpret_cast<uint32_t *>(smem);            // [64][32]
     uint4 *const splice = reinterpret_cast<uint4 *>(smem + kRLutBytes);  // [33][2]
     uint32_t *const tq1 = reinterpret_cast<uint32_t *>(smem + L.tq1);
@@ -280,7 +281,7 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
             }
         }
     }
-    const float scale = bf16_bits_to_f32(*P.scale);
+    const float scale = bf16_bits_to_f32(scale_bits);
     for (uint32_t i = tid; i < 64 * 32; i += blockDim.x) {
         const int c0 = (i >> 5) & 7, c1 = i >> 8;
         const uint32_t w0 = c0 < 7 ? f32_to_bf16_bits((float)(c0 - 3) * scale) : 0u;
