@@ -40,14 +40,14 @@ _DENSE = ("ixh_dense358.hip", "ixh_dense_tiles.h", "ixh_dev.h")
 _DENSE5 = ("ixh_dense5.hip", "ixh_dense_tiles.h", "ixh_dev.h")
 _OLD = ((), "measured-on-earlier-sources")  # figures kept for the record; reported as null
 MEASURED_TRAFFIC_BYTES = {
-    "down_proj_5120x17408_m1_student_t": (23035.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "65573860fb392e0a"),
-    "gate_up_17408x5120_m1_student_t": (22939.0 * 2.0 * 1024 + 40.0 * 1024, _ROWS, "65573860fb392e0a"),
-    "attn_proj_5120x5120_m1_student_t": (7139.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "65573860fb392e0a"),
+    "down_proj_5120x17408_m1_student_t": (23035.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "6f04b190cb6e676f"),
+    "gate_up_17408x5120_m1_student_t": (22939.0 * 2.0 * 1024 + 40.0 * 1024, _ROWS, "6f04b190cb6e676f"),
+    "attn_proj_5120x5120_m1_student_t": (7139.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "6f04b190cb6e676f"),
     "down_proj_5120x17408_m1_calibrated": (33826.0 * 2.0 * 1024 + 40.0 * 1024, _DENSE, "687a9e669409fe32"),
     "down_proj_5120x17408_m1_five_level_calibrated": (49708.0 * 2.0 * 1024 + 1335.0 * 1024, _DENSE5, "2ca11f7c18f16b0b"),
-    "gate_up_17408x5120_m4_student_t": (28090.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "8b42a20ff4590f76"),
-    "gate_up_17408x5120_m16_student_t": (26571.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "8b42a20ff4590f76"),
-    "attn_proj_5120x5120_m16_student_t": (7798.0 * 2.0 * 1024 + 256.0 * 1024, _TILES, "8b42a20ff4590f76"),
+    "gate_up_17408x5120_m4_student_t": (28092.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "e4e86a49151e5b13"),
+    "gate_up_17408x5120_m16_student_t": (26572.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "e4e86a49151e5b13"),
+    "attn_proj_5120x5120_m16_student_t": (7797.0 * 2.0 * 1024 + 256.0 * 1024, _TILES, "e4e86a49151e5b13"),
     "decode_5120x17408_five_level_calibrated": (49757.0 * 2.0 * 1024 + 174080.0 * 1024, _DENSE5, "2ca11f7c18f16b0b"),
     "prefill_5120x5120_m512_five_level": (50297.9 * 2.0 * 1024 + 30720.0 * 1024,) + _OLD,
     "decode_5120x17408_student_t": (23268.0 * 2.0 * 1024 + 179524.0 * 1024,) + _OLD,
