@@ -227,14 +227,40 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
     // ---- workgroup set-up: activations, table slices, side streams, pair table, splice masks ----
     // activation rows of the part's columns into padded strips: 16-byte piece p of row i holds columns 8p .. 8p+7
-    auto load_activations = [&]() {
+    auto load_activations = [&]() __attribute__((always_inline)) {
         const uint32_t pieces = part_count * (kFastChunk / 8), first_piece = part_first * (kFastChunk / 8);
         uint32_t t0 = threadIdx.x;
         asm volatile("" : "+v"(t0));  // worked out anew at every call: no register is held for it across the loop
-        for (uint32_t t = t0; t < (uint32_t)m * pieces; t += blockDim.x) {
-            const uint32_t i = t / pieces, p = t - i * pieces;
-            const uint4 v = *reinterpret_cast<const uint4 *>(x + (int64_t)i * ldx + (first_piece + p) * 8u);
-            *reinterpret_cast<uint4 *>(smem + L.xs + i * L.xs_row + (p >> 4) * kTStripBytes + (p & 15u) * 16u) = v;
+        // eight loads of a thread in flight at a time, then their stores: one piece a trip to memory (a loop of load
+        // and store) made a part of five column blocks at 16 activation rows eight trips long.  Row and piece are
+        // stepped, not divided out, for every load.
+        const uint32_t total = (uint32_t)m * pieces, stride = blockDim.x;
+        const uint32_t di = stride / pieces, dp = stride - di * pieces;
+        uint32_t i = t0 / pieces, p = t0 - i * pieces;
+        for (uint32_t tb = t0, done = 0; tb < total; tb += 8u * stride, done += 8u * stride) {
+            // (named registers, not an array: the array went to scratch memory; a slot that no thread of the workgroup
+            // needs is skipped by a scalar branch)
+#define IXH_T_LOAD(u)                                                                                              \
+    const bool any##u = done + (uint32_t)(u) * stride < total;                                                      \
+    uint4 v##u = make_uint4(0, 0, 0, 0);                                                                            \
+    uint32_t at##u = ~0u;                                                                                           \
+    if (any##u) {                                                                                                   \
+        const bool live = tb + (uint32_t)(u) * stride < total;                                                      \
+        v##u = *reinterpret_cast<const uint4 *>(x + (int64_t)(live ? i : 0u) * ldx + (first_piece + (live ? p : 0u)) * 8u); \
+        if (live) at##u = L.xs + i * L.xs_row + (p >> 4) * kTStripBytes + (p & 15u) * 16u;                          \
+        i += di;                                                                                                    \
+        p += dp;                                                                                                    \
+        if (p >= pieces) {                                                                                          \
+            p -= pieces;                                                                                            \
+            ++i;                                                                                                    \
+        }                                                                                                           \
+    }
+            IXH_T_LOAD(0) IXH_T_LOAD(1) IXH_T_LOAD(2) IXH_T_LOAD(3) IXH_T_LOAD(4) IXH_T_LOAD(5) IXH_T_LOAD(6) IXH_T_LOAD(7)
+#undef IXH_T_LOAD
+#define IXH_T_STORE(u) \
+    if (at##u != ~0u) *reinterpret_cast<uint4 *>(smem + at##u) = v##u;
+            IXH_T_STORE(0) IXH_T_STORE(1) IXH_T_STORE(2) IXH_T_STORE(3) IXH_T_STORE(4) IXH_T_STORE(5) IXH_T_STORE(6) IXH_T_STORE(7)
+#undef IXH_T_STORE
         }
     };
     load_activations();
