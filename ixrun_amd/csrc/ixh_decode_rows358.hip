@@ -303,12 +303,13 @@ k_decode358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_quads, ui
         (uint32_t)(uintptr_t)(dr_lds_ptr_t)(wave_base + kDrStages * kDrStageBytes + kDrQueue * 16 + kDrTasks * 2);
 
     // ---- workgroup set-up: table slice first (it waits on memory), then the tables built here ----
+    const uint16_t scale_bits = *P.scale;  // asked for with the table slice, not in a trip to memory of its own after it
     const uint32_t entries = n_quads * 4 + 1;
     for (uint32_t i = tid; i <= units_here; i += blockDim.x) {
         tq1[i] = (uint32_t)prefix[unit0 + i];
         if (!ANY) tq2[i] = (uint32_t)prefix[entries + unit0 + i];
     }
-    const float scale = bf16_bits_to_f32(*P.scale);
+    const float scale = bf16_bits_to_f32(scale_bits);
     for (uint32_t i = tid; i < 64 * 32; i += blockDim.x) {
         const int c0 = (i >> 5) & 7, c1 = i >> 8;
         const uint32_t w0 = c0 < 7 ? f32_to_bf16_bits((float)(c0 - 3) * scale) : 0u;

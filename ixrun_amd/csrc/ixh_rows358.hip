@@ -113,13 +113,14 @@ k_gemv358_rows(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uin
     uint32_t *const xs = reinterpret_cast<uint32_t *>(tasks + kRTasks2);  // [MT][C * 512] bf16
 
     // ---- workgroup set-up: table slices and x first (they wait on memory), then the tables built here ----
+    const uint16_t scale_bits = *P.scale;  // asked for with the table slices, not in a trip to memory of its own after them
     const uint32_t unit0 = row0 * n_chunks;
     const uint32_t entries = P.out_f * n_chunks + 1;
     for (uint32_t i = tid; i <= rows_here * n_chunks; i += blockDim.x) {
             tq1[i] = (uint32_t)prefix[unit0 + i];
             if (!ANY) tq2[i] = (uint32_t)prefix[entries + unit0 + i];
         }
-    const float scale = bf16_bits_to_f32(*P.scale);
+    const float scale = bf16_bits_to_f32(scale_bits);
     for (uint32_t i = tid; i < 64 * 32; i += blockDim.x) {
             const int c0 = (i >> 5) & 7, c1 = i >> 8;
             const uint32_t w0 = c0 < 7 ? f32_to_bf16_bits((float)(c0 - 3) * scale) : 0u;
