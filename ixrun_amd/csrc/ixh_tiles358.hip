@@ -377,7 +377,7 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         w2 = (w2 & ~fm.z) | (kZeroCodes2 & fm.z);
     };
 
-    __syncthreads();
+    // (the barrier that ends the set-up comes after the first task's codes have been asked for, below)
 
     // A task in flight: the ranks at which its words start and the stream bytes asked for with them.
     struct Stage {
@@ -469,11 +469,15 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
     // Three steps per task, each one task ahead of the next: table entry + bitmap words (request), ranks and code
     // requests (launch_codes), decode (compute).  Two stages take turns, so nothing is copied between iterations.
+    // The first task's codes are asked for before the barrier that ends the set-up, and travel across it (no fence:
+    // this wave's LDS stores have completed, and the loads in flight are nobody else's business).
+    auto setup_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
     for (uint32_t part = 0;;) {
         if (c_begin < c_end) {
             Stage A, B;
             launch_codes(T, A);
             if (c_begin + slots < c_end) request(c_begin + slots, T);
+            if (part == 0) setup_barrier();
             // The queue is emptied between tasks, where one stage is dead and registers are free: before a task whose
             // records (at most 4 x 64 = the queue's capacity) would not fit behind those that wait.
             for (uint32_t c = c_begin; c < c_end; c += 2 * slots) {
@@ -493,6 +497,7 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
                 }
             }
         }
+        else if (part == 0) setup_barrier();
         if (++part == n_parts) break;
         // the next part of the columns: this part's elements above level 1 meet its activations while they are there
         resolve();
