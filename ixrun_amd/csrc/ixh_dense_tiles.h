@@ -64,13 +64,17 @@ struct DtMfmaSink {
     }
     // o: the lane's 32 weights of the span in position order, as 16 bf16 pairs (lanes past the row's end: anything
     // finite; their activations are zero)
+    // A barrier for LDS traffic only: this wave's LDS accesses have completed, nothing is said about global memory.
+    // __syncthreads() carries a fence that waits for every load in flight, and here the next span's table entries,
+    // bitmap words and code windows are in flight across both barriers of a span.
+    static __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
     __device__ __forceinline__ void end(const DtStep &st, const uint32_t (&o)[16]) {
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
         dt_u32x4 *const rows = reinterpret_cast<dt_u32x4 *>(wc);
 #pragma unroll
         for (int j = 0; j < 4; ++j) rows[lane * 5 + j] = dt_u32x4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
-        __syncthreads();  // the tile is whole
+        lds_barrier();  // the tile is whole
         const uint32_t n = lane & 15u, kg = lane >> 4;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -80,7 +84,7 @@ struct DtMfmaSink {
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(dt_bf16x8, xa[j]),
                                                          __builtin_bit_cast(dt_bf16x8, b), acc, 0, 0, 0);
         }
-        __syncthreads();  // before any wave's next span overwrites its array
+        lds_barrier();  // before any wave's next span overwrites its array
         const bool block_ends = st.k + 1 == spans_per_row;
         if (!block_ends && st.step + 1 != step_end) return;
         // ---- the block's sums so far leave: added over the waves in order, one piece per workgroup ----
