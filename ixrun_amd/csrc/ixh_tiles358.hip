@@ -471,13 +471,22 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     // requests (launch_codes), decode (compute).  Two stages take turns, so nothing is copied between iterations.
     // The first task's codes are asked for before the barrier that ends the set-up, and travel across it (no fence:
     // this wave's LDS stores have completed, and the loads in flight are nobody else's business).
-    auto setup_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
     for (uint32_t part = 0;;) {
-        if (c_begin < c_end) {
-            Stage A, B;
+        const bool mine = c_begin < c_end;
+        Stage A, B;
+        if (mine) {
             launch_codes(T, A);
             if (c_begin + slots < c_end) request(c_begin + slots, T);
-            if (part == 0) setup_barrier();
+        }
+        if (part != 0) {
+            // the next part of the columns (the last part's elements above level 1 have met its activations): the
+            // copy travels together with the first task's codes
+            lds_barrier();  // nobody reads the old part any more
+            load_activations();
+        }
+        lds_barrier();  // the set-up, or the part's activations, are in LDS
+        if (mine) {
             // The queue is emptied between tasks, where one stage is dead and registers are free: before a task whose
             // records (at most 4 x 64 = the queue's capacity) would not fit behind those that wait.
             for (uint32_t c = c_begin; c < c_end; c += 2 * slots) {
@@ -497,17 +506,13 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
                 }
             }
         }
-        else if (part == 0) setup_barrier();
         if (++part == n_parts) break;
-        // the next part of the columns: this part's elements above level 1 meet its activations while they are there
+        // this part's elements above level 1 meet its activations while they are there
         resolve();
         part_first = (uint32_t)__builtin_amdgcn_readfirstlane((int)(part * x_blocks));
         part_count = min(x_blocks, n_chunks - part_first);
         take_share();
         if (c_begin < c_end) request(c_begin, T);
-        __syncthreads();  // nobody reads the old part any more
-        load_activations();
-        __syncthreads();
     }
     resolve();
 
