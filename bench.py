@@ -40,15 +40,15 @@ _DENSE = ("ixh_dense358.hip", "ixh_dense_tiles.h", "ixh_dev.h")
 _DENSE5 = ("ixh_dense5.hip", "ixh_dense_tiles.h", "ixh_dev.h")
 _OLD = ((), "measured-on-earlier-sources")  # figures kept for the record; reported as null
 MEASURED_TRAFFIC_BYTES = {
-    "down_proj_5120x17408_m1_student_t": (23035.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "6f04b190cb6e676f"),
-    "gate_up_17408x5120_m1_student_t": (22939.0 * 2.0 * 1024 + 40.0 * 1024, _ROWS, "6f04b190cb6e676f"),
-    "attn_proj_5120x5120_m1_student_t": (7139.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "6f04b190cb6e676f"),
-    "down_proj_5120x17408_m1_calibrated": (33826.0 * 2.0 * 1024 + 40.0 * 1024, _DENSE, "687a9e669409fe32"),
-    "down_proj_5120x17408_m1_five_level_calibrated": (49708.0 * 2.0 * 1024 + 1335.0 * 1024, _DENSE5, "2ca11f7c18f16b0b"),
-    "gate_up_17408x5120_m4_student_t": (28112.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "65f9ddd2bd5b2abe"),
-    "gate_up_17408x5120_m16_student_t": (26599.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "65f9ddd2bd5b2abe"),
-    "attn_proj_5120x5120_m16_student_t": (7821.0 * 2.0 * 1024 + 256.0 * 1024, _TILES, "65f9ddd2bd5b2abe"),
-    "decode_5120x17408_five_level_calibrated": (49757.0 * 2.0 * 1024 + 174080.0 * 1024, _DENSE5, "2ca11f7c18f16b0b"),
+    "down_proj_5120x17408_m1_student_t": (23035.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "e45341197bdab021"),
+    "gate_up_17408x5120_m1_student_t": (22939.0 * 2.0 * 1024 + 40.0 * 1024, _ROWS, "e45341197bdab021"),
+    "attn_proj_5120x5120_m1_student_t": (7139.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "e45341197bdab021"),
+    "down_proj_5120x17408_m1_calibrated": (33825.0 * 2.0 * 1024 + 40.0 * 1024, _DENSE, "711eef94d053feb1"),
+    "down_proj_5120x17408_m1_five_level_calibrated": (49708.0 * 2.0 * 1024 + 1338.0 * 1024, _DENSE5, "aaca19573f1ed2a1"),
+    "gate_up_17408x5120_m4_student_t": (28602.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "261f8c8a3cdc0c74"),
+    "gate_up_17408x5120_m16_student_t": (26546.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "261f8c8a3cdc0c74"),
+    "attn_proj_5120x5120_m16_student_t": (7829.0 * 2.0 * 1024 + 256.0 * 1024, _TILES, "261f8c8a3cdc0c74"),
+    "decode_5120x17408_five_level_calibrated": (49719.0 * 2.0 * 1024 + 174080.0 * 1024, _DENSE5, "aaca19573f1ed2a1"),
     "prefill_5120x5120_m512_five_level": (50297.9 * 2.0 * 1024 + 30720.0 * 1024,) + _OLD,
     "decode_5120x17408_student_t": (23268.0 * 2.0 * 1024 + 179524.0 * 1024,) + _OLD,
     "decode_5120x17408_calibrated": (36308.0 * 2.0 * 1024 + 174080.0 * 1024,) + _OLD,
