@@ -89,6 +89,9 @@ const char *ixh_last_error(void);
  *                    full; default), 1 = wherever it fits
  *   "gemv_tile_rows" the tile kernel's tile shape: 0 = the planner's choice (default), 2 / 3 / 4 = tiles of 4 / 8 / 16
  *                    weight rows only (a shape that cannot serve the call's activation rows hands the call on)
+ *   "gemv_tile_split" the number of workgroups of the tile kernel that share a block of rows, each taking a run of its
+ *                    column blocks, their sums added by a second launch (needs the workspace of ixh_gemv): 0 = the
+ *                    planner's choice (default), 1..8 = that many where the workspace allows
  *   "gemv_tile_cus"  the number of CUs over which the tile kernel's planner spreads the rows: 0 = the device's
  *                    (default), 1..4096 = that many (small tensors then get workgroups with several tiles); also the
  *                    number of workgroups of the dense-mix matrix-pipe kernel

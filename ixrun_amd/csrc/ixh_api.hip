@@ -20,6 +20,7 @@ std::atomic<int> g_opt_gemv_strips{0};
 std::atomic<int> g_opt_gemv_tiles{0};
 std::atomic<int> g_opt_gemv_tile_rows{0};
 std::atomic<int> g_opt_gemv_tile_cus{0};
+std::atomic<int> g_opt_gemv_tile_split{0};
 std::atomic<int> g_opt_gemv_dense_tiles{0};
 
 void set_error(const char *fmt, ...) {
@@ -113,6 +114,11 @@ int ixh_set_option(const char *name, int64_t value) {
     if (strcmp(name, "gemv_tile_rows") == 0) {
         if (value != 0 && value != 2 && value != 3 && value != 4) { set_error("gemv_tile_rows %lld not 0, 2, 3 or 4", (long long)value); return IXH_EINVAL; }
         g_opt_gemv_tile_rows.store((int)value, std::memory_order_relaxed);
+        return IXH_OK;
+    }
+    if (strcmp(name, "gemv_tile_split") == 0) {
+        if (value < 0 || value > 8) { set_error("gemv_tile_split %lld not in 0..8", (long long)value); return IXH_EINVAL; }
+        g_opt_gemv_tile_split.store((int)value, std::memory_order_relaxed);
         return IXH_OK;
     }
     if (strcmp(name, "gemv_tile_cus") == 0) {
@@ -266,7 +272,9 @@ static int gemv_any(const IxhPacked *packed, const int32_t *prefix, int64_t chun
         // (atomic mode excepted: a later group that does not fit must not leave an earlier one added).
         uint16_t *const yb = atomic ? nullptr : y;
         float *const yf = atomic ? y32 : nullptr;
-        rc = launch_gemv_358_tiles(d, prefix, x, m, ldx, yb, ldy, yf, (hipStream_t)stream);
+        // (the workspace holds in_f / chunk pieces of m x out_f sums)
+        rc = launch_gemv_358_tiles(d, prefix, x, m, ldx, yb, ldy, yf, atomic ? nullptr : (float *)workspace,
+                                   workspace && !atomic ? (uint32_t)(d.in_f / (uint32_t)chunk) : 0u, (hipStream_t)stream);
         if (rc == IXH_EUNSUPPORTED) rc = launch_gemv_358_strips(d, prefix, x, m, ldx, yb, ldy, yf, (hipStream_t)stream);
         if (rc == IXH_EUNSUPPORTED && m <= 8)
             rc = launch_gemv_358_rows(d, prefix, x, m, ldx, yb, ldy, yf, (hipStream_t)stream);

@@ -19,9 +19,10 @@ int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x,
 // strip kernel (ixh_strips358.hip): up to four activation rows, products on the matrix pipe; same contract
 int launch_gemv_358_strips(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
                            int64_t ldy, float *y32, hipStream_t s);
-// tile kernel (ixh_tiles358.hip): 16 weight rows x up to 16 activation rows per matrix instruction; same contract
+// tile kernel (ixh_tiles358.hip): 16 weight rows x up to 16 activation rows per matrix instruction; same contract.
+// ws: room for ws_pieces x m x out_f fp32 sums (or none), for plans in which several workgroups share a block of rows
 int launch_gemv_358_tiles(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
-                          int64_t ldy, float *y32, hipStream_t s);
+                          int64_t ldy, float *y32, float *ws, uint32_t ws_pieces, hipStream_t s);
 // level-by-level kernel for one activation row and mixes with many elements above level 1 (ixh_dense358.hip)
 bool gemv_dense358_supports(const Dev &P, uint32_t chunk, int m, const uint16_t *x);
 int launch_gemv_dense358(const Dev &P, const int32_t *prefix, const uint16_t *x, uint16_t *y, float *y32, float *ws,

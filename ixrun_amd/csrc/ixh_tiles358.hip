@@ -35,6 +35,9 @@ namespace ixh {
 extern std::atomic<int> g_opt_gemv_tile_rows;
 // ixh_set_option("gemv_tile_cus"): the number of CUs the planner spreads the rows over; 0 = the device's
 extern std::atomic<int> g_opt_gemv_tile_cus;
+// ixh_set_option("gemv_tile_split"): the number of workgroups that share a block of rows, each taking a run of its
+// column blocks; 0 = the planner's choice
+extern std::atomic<int> g_opt_gemv_tile_split;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -44,10 +47,13 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 constexpr int kTMaxWaves = 16;
 constexpr uint32_t kTMaxRows = 128;  // rows per workgroup at most (8 tiles)
 constexpr int kTMaxM = 16;
+constexpr uint32_t kTQueue = 256;  // records in a wave's queue: a task's records must fit (4 words x 64 lanes)
 constexpr size_t kTLdsLimit = 160 * 1024;
 // bytes between the 128-column strips of an activation row: 16-byte reads need 16-byte aligned strips, and 272 = 68
 // dwords puts the four strips of a column block four banks apart, as the 16-byte shift between rows does for the rows
 constexpr uint32_t kTStripBytes = 272;
+
+constexpr uint32_t kFlagPieces = 0x100u;  // y32 is a workspace of pieces: plain stores at the workgroup's piece
 
 struct TilesLds {
     uint32_t tq1, tq2, side, xs, xs_row, zero, partial, waves, wave_bytes, tasks_off, round_off, total;
@@ -135,8 +141,8 @@ struct TileSink {
 template <bool ANY>
 __global__ void __launch_bounds__(kTMaxWaves * kWave)
 k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t rows_per_wg, uint32_t n_sub,
-                uint32_t x_blocks, uint32_t lg_rows, uint32_t qcap, uint32_t flags, const uint16_t *__restrict__ x,
-                int m, int64_t ldx,
+                uint32_t x_blocks, uint32_t lg_rows, uint32_t flags, uint32_t k_plan,
+                const uint16_t *__restrict__ x, int m, int64_t ldx,
                 uint16_t *__restrict__ y, int64_t ldy, float *__restrict__ y32) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
@@ -149,14 +155,22 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     const uint32_t tile_rows = 1u << lg_rows, slots = 16u >> lg_rows;
     const uint32_t r = n & (tile_rows - 1u);
 
-    const uint32_t row0 = blockIdx.x * rows_per_wg;
+    // k_split workgroups share a block of rows, k_blocks column blocks of every row each; with kFlagPieces their
+    // sums go to y32 as a workspace ([piece][m][row] fp32) for the kernel that adds the pieces in order
+    // (k_plan: k_split | k_blocks << 8)
+    const uint32_t k_split = k_plan & 255u, k_blocks = k_plan >> 8;
+    const uint32_t row_group = blockIdx.x / k_split;
+    const uint32_t kb_end = min(n_chunks, (blockIdx.x - row_group * k_split + 1u) * k_blocks);
+    const uint32_t row0 = row_group * rows_per_wg;
     const uint32_t rows_here = min(rows_per_wg, P.out_f - row0), rows_cap = rows_per_wg;
+    constexpr uint32_t qcap = kTQueue;
     const TilesLds L = tiles_layout(rows_cap, n_chunks, x_blocks, n_sub * slots, n_waves, m, qcap);
 
     // the pair table is addressed with (index bits | lane bits): it must sit at LDS address 0
     if ((uint32_t)(uintptr_t)(lds_ptr_t)smem != 0) {
         for (uint32_t t = tid; t < rows_here * (uint32_t)m; t += blockDim.x) {
-            if (y32) y32[(size_t)(t % m) * P.out_f + row0 + t / m] = __uint_as_float(0x7FC00000u);  // NaN
+            const uint32_t piece = (flags & kFlagPieces) ? blockIdx.x % k_split : 0u;
+            if (y32) y32[((size_t)piece * m + t % m) * P.out_f + row0 + t / m] = __uint_as_float(0x7FC00000u);  // NaN
             else y[(int64_t)(t % m) * ldy + row0 + t / m] = 0x7FC0;
         }
         return;
@@ -191,8 +205,8 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     // 16 a unit) and the row's part of a record
     const uint32_t base_u = row0 * n_chunks + lrow * n_chunks;
     const uint32_t rec_hi = (n << 27) | (lrow << 20);
-    const uint32_t n_parts = (n_chunks + x_blocks - 1) / x_blocks;
-    uint32_t part_first = 0, part_count = min(x_blocks, n_chunks);  // the part's column blocks
+    uint32_t part_first = (blockIdx.x - row_group * k_split) * k_blocks;  // the part's column blocks
+    uint32_t part_count = min(x_blocks, kb_end - part_first);
     uint32_t c_begin = 0, c_end = 0;                                // this wave's run of them
     auto take_share = [&]() {  // in steps of `slots` column blocks
         const uint32_t steps = (part_count + slots - 1u) >> (4u - lg_rows);
@@ -472,14 +486,14 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     // The first task's codes are asked for before the barrier that ends the set-up, and travel across it (no fence:
     // this wave's LDS stores have completed, and the loads in flight are nobody else's business).
     auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
-    for (uint32_t part = 0;;) {
+    for (bool later = false;; later = true) {
         const bool mine = c_begin < c_end;
         Stage A, B;
         if (mine) {
             launch_codes(T, A);
             if (c_begin + slots < c_end) request(c_begin + slots, T);
         }
-        if (part != 0) {
+        if (later) {
             // the next part of the columns (the last part's elements above level 1 have met its activations): the
             // copy travels together with the first task's codes
             lds_barrier();  // nobody reads the old part any more
@@ -506,11 +520,11 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
                 }
             }
         }
-        if (++part == n_parts) break;
+        if (part_first + part_count >= kb_end) break;
         // this part's elements above level 1 meet its activations while they are there
         resolve();
-        part_first = (uint32_t)__builtin_amdgcn_readfirstlane((int)(part * x_blocks));
-        part_count = min(x_blocks, n_chunks - part_first);
+        part_first = (uint32_t)__builtin_amdgcn_readfirstlane((int)(part_first + part_count));
+        part_count = min(x_blocks, kb_end - part_first);
         take_share();
         if (c_begin < c_end) request(c_begin, T);
     }
@@ -544,7 +558,8 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
             for (uint32_t q = 0; q < slots; ++q)
                 sum += reinterpret_cast<const float *>(smem + L.partial)[((s * slots + q) * rows_cap + row) * (uint32_t)m + i];
         }
-        if (y32) atomicAdd(&y32[(size_t)i * P.out_f + row0 + row], sum);
+        if (y32 && (flags & kFlagPieces)) y32[((size_t)(blockIdx.x % k_split) * m + i) * P.out_f + row0 + row] = sum;
+        else if (y32) atomicAdd(&y32[(size_t)i * P.out_f + row0 + row], sum);
         else y[(int64_t)i * ldy + row0 + row] = (uint16_t)f32_to_bf16_bits(sum);
     }
 }
@@ -553,53 +568,64 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 // host side
 // ---------------------------------------------------------------------------
 struct TilesPlan {
-    uint32_t rows, n_sub, x_blocks, qcap, waves, lg_rows;
+    uint32_t rows, n_sub, x_blocks, qcap, waves, lg_rows, k_split, k_blocks;
     float cost;
 };
 
-// Rows per workgroup (whole rounds of one workgroup per CU, a multiple of four), the tile shape, waves per tile and the
-// part of the activation rows that LDS holds at a time.  A tile of 16 >> k rows takes 1 << k column blocks per step and
-// serves 16 >> k activation rows, so short tiles suit workgroups whose rows are not a multiple of 16 when the rows of
-// activations are few.  A wave's time goes with the steps it decodes, and every further part costs two barriers and a
-// copy whose latency nobody covers: the plan with the fewest steps per wave, a part counted as a third of a step
-// (costs that also count the steps of all waves of a CU, or of a SIMD, chose slower plans on the shapes measured).
-static TilesPlan plan_tiles(uint32_t out_f, uint32_t n_chunks, uint32_t n_cu, int m, int lg_only) {
+// Rows per workgroup (whole rounds of one workgroup per CU, a multiple of four), the tile shape, waves per tile, the
+// part of the activation rows that LDS holds at a time, and the number of workgroups that share a block of rows, each
+// taking a run of its column blocks.  A tile of 16 >> k rows takes 1 << k column blocks per step and serves 16 >> k
+// activation rows, so short tiles suit workgroups whose rows are not a multiple of 16 when the rows of activations are
+// few.  A wave's time goes with the steps it decodes, and every further part costs two barriers and a copy: the plan
+// with the fewest steps per wave, a part counted as a third of a step (costs that also count the steps of all waves of
+// a CU, or of a SIMD, chose slower plans on the shapes measured).  Sharing the rows' columns among k workgroups makes
+// the row blocks k times as tall, which fills tiles of 16 that a short block leaves mostly empty and takes k times
+// fewer parts per workgroup; it costs the second launch that adds the pieces (kSplitCost steps).
+constexpr float kSetupCost = 2.5f, kSplitCost = 1.0f;  // in steps: a round's set-up and final sums; the second launch
+static TilesPlan plan_tiles(uint32_t out_f, uint32_t n_chunks, uint32_t n_cu, int m, int lg_only, uint32_t max_split,
+                            uint32_t split_only) {
     const uint32_t n_quads = (out_f + 3) / 4, max_quads = kTMaxRows / 4;
-    const uint32_t rounds = (n_quads + n_cu * max_quads - 1) / (n_cu * max_quads);
-    const uint32_t rows = 4u * max(1u, min(max_quads, (n_quads + rounds * n_cu - 1) / (rounds * n_cu)));
-    TilesPlan best{0, 0, 0, 0, 0, 4, 0.0f};
-    for (uint32_t lg = 4; lg >= 2; --lg) {
-        if (lg_only >= 2 && (uint32_t)lg_only != lg) continue;
-        const uint32_t tile_rows = 1u << lg, slots = 16u >> lg;
-        if ((uint32_t)m > tile_rows) break;
-        const uint32_t tiles = (rows + tile_rows - 1) / tile_rows;
-        if (tiles > (uint32_t)kTMaxWaves) continue;
-        for (uint32_t parts = 1; parts <= n_chunks; ++parts) {
-            const uint32_t x_blocks = (n_chunks + parts - 1) / parts;
-            if ((n_chunks + x_blocks - 1) / x_blocks != parts) continue;  // the same parts with fewer blocks each: seen
-            const uint32_t steps = (x_blocks + slots - 1) / slots;  // of the longest part
-            TilesPlan here{0, 0, 0, 0, 0, lg, 0.0f};
-            for (uint32_t n_sub = min((uint32_t)kTMaxWaves / tiles, steps); n_sub >= 1 && here.waves == 0; --n_sub) {
-                for (uint32_t qcap : {256u}) {  // a task's records must fit: 4 words x 64 lanes
+    TilesPlan best{0, 0, 0, 0, 0, 4, 1, 0, 0.0f};
+    for (uint32_t k_split = 1; k_split <= min(min(max_split, 8u), n_chunks); ++k_split) {
+        if (split_only != 0 && k_split != split_only) continue;
+        const uint32_t k_blocks = (n_chunks + k_split - 1) / k_split;
+        if ((n_chunks + k_blocks - 1) / k_blocks != k_split) continue;  // a piece would be empty
+        const uint32_t per_round = max(1u, n_cu / k_split);             // blocks of rows at a time
+        const uint32_t rounds = (n_quads + per_round * max_quads - 1) / (per_round * max_quads);
+        const uint32_t rows = 4u * max(1u, min(max_quads, (n_quads + rounds * per_round - 1) / (rounds * per_round)));
+        for (uint32_t lg = 4; lg >= 2; --lg) {
+            if (lg_only >= 2 && (uint32_t)lg_only != lg) continue;
+            const uint32_t tile_rows = 1u << lg, slots = 16u >> lg;
+            if ((uint32_t)m > tile_rows) break;
+            const uint32_t tiles = (rows + tile_rows - 1) / tile_rows;
+            if (tiles > (uint32_t)kTMaxWaves) continue;
+            for (uint32_t parts = 1; parts <= k_blocks; ++parts) {
+                const uint32_t x_blocks = (k_blocks + parts - 1) / parts;
+                if ((k_blocks + x_blocks - 1) / x_blocks != parts) continue;  // the same parts with fewer blocks each: seen
+                const uint32_t steps = (x_blocks + slots - 1) / slots;      // of the longest part
+                TilesPlan here{0, 0, 0, 0, 0, lg, k_split, k_blocks, 0.0f};
+                for (uint32_t n_sub = min((uint32_t)kTMaxWaves / tiles, steps); n_sub >= 1 && here.waves == 0; --n_sub) {
+                    const uint32_t qcap = kTQueue;
                     if (tiles_layout(rows, n_chunks, x_blocks, n_sub * slots, tiles * n_sub, m, qcap).total > kTLdsLimit)
                         continue;
                     // no more waves than shorten the longest run of steps
                     const uint32_t run = (steps + n_sub - 1) / n_sub;
                     const uint32_t subs = (steps + run - 1) / run;
-                    uint32_t per_wave = 0;
-                    for (uint32_t first = 0; first < n_chunks; first += x_blocks) {
-                        const uint32_t st = (min(x_blocks, n_chunks - first) + slots - 1) / slots;
+                    uint32_t per_wave = 0;  // of the longest piece, the first
+                    for (uint32_t first = 0; first < k_blocks; first += x_blocks) {
+                        const uint32_t st = (min(x_blocks, k_blocks - first) + slots - 1) / slots;
                         per_wave += (st + subs - 1) / subs;
                     }
-                    here = TilesPlan{rows, subs, x_blocks, qcap, tiles * subs, lg,
-                                     (float)per_wave + (float)(parts - 1) / 3.0f};
-                    break;
+                    here.rows = rows, here.n_sub = subs, here.x_blocks = x_blocks, here.qcap = qcap;
+                    here.waves = tiles * subs;
+                    here.cost = (float)rounds * ((float)per_wave + (float)(parts - 1) / 3.0f + kSetupCost) +
+                                (k_split > 1 ? kSplitCost : 0.0f);
                 }
+                if (here.waves != 0 && (best.waves == 0 || here.cost < best.cost)) best = here;
+                if (here.waves != 0 && here.waves >= tiles * min((uint32_t)kTMaxWaves / tiles, steps) && parts > 1 &&
+                    here.cost > best.cost)
+                    break;  // more parts only add to the cost from here on
             }
-            if (here.waves != 0 && (best.waves == 0 || here.cost < best.cost)) best = here;
-            if (here.waves != 0 && here.waves >= tiles * min((uint32_t)kTMaxWaves / tiles, steps) && parts > 1 &&
-                here.cost > best.cost)
-                break;  // more parts only add to the cost from here on
         }
     }
     return best;
@@ -607,7 +633,7 @@ static TilesPlan plan_tiles(uint32_t out_f, uint32_t n_chunks, uint32_t n_cu, in
 
 template <bool ANY>
 static int launch_tiles(const Dev &P, const int32_t *prefix, uint32_t n_chunks, const TilesPlan &plan, const uint16_t *x,
-                        int m, int64_t ldx, uint16_t *y, int64_t ldy, float *y32, hipStream_t s) {
+                        int m, int64_t ldx, uint16_t *y, int64_t ldy, float *y32, float *ws, hipStream_t s) {
     static const bool raised =  // per instantiation
         hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemv358_tiles<ANY>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTLdsLimit) == hipSuccess;
@@ -616,17 +642,27 @@ static int launch_tiles(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
     const size_t lds =
         tiles_layout(plan.rows, n_chunks, plan.x_blocks, plan.n_sub * (16u >> plan.lg_rows), plan.waves, m, plan.qcap).total;
     if (lds > kTLdsLimit) return IXH_EUNSUPPORTED;
+    // every piece has column blocks (the kernel's part loop counts on it)
+    if (plan.k_split < 1 || plan.k_blocks < 1 || (uint64_t)(plan.k_split - 1) * plan.k_blocks >= n_chunks ||
+        (uint64_t)plan.k_split * plan.k_blocks < n_chunks)
+        return IXH_EUNSUPPORTED;
+    const bool pieces = plan.k_split > 1 && !y32;
+    if (pieces && !ws) return IXH_EUNSUPPORTED;
     uint32_t flags = 0;
     if (((uintptr_t)P.last & 3u) == 0) flags |= kFlagStageSide;
-    hipLaunchKernelGGL((k_gemv358_tiles<ANY>), dim3(groups), dim3(plan.waves * kWave), lds, s, P, prefix, n_chunks,
-                       plan.rows, plan.n_sub, plan.x_blocks, plan.lg_rows, plan.qcap, flags, x, m, ldx, y, ldy, y32);
-    return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
+    if (pieces) flags |= kFlagPieces;
+    hipLaunchKernelGGL((k_gemv358_tiles<ANY>), dim3(groups * plan.k_split), dim3(plan.waves * kWave), lds, s, P, prefix,
+                       n_chunks, plan.rows, plan.n_sub, plan.x_blocks, plan.lg_rows, flags,
+                       plan.k_split | (plan.k_blocks << 8), x, m, ldx, pieces ? nullptr : y, ldy, pieces ? ws : y32);
+    if (hipGetLastError() != hipSuccess) return IXH_ELAUNCH;
+    return pieces ? launch_reduce_chunks(ws, plan.k_split, m, P.out_f, y, ldy, s) : IXH_OK;
 }
 
 // The tile kernel: up to 16 activation rows, rows of whole 512-column blocks, row counts that are multiples of four;
-// IXH_EUNSUPPORTED sends the caller on to the other row-block kernels.
+// IXH_EUNSUPPORTED sends the caller on to the other row-block kernels.  ws: room for ws_pieces x m x out_f fp32 sums
+// (none: every workgroup takes whole rows).
 int launch_gemv_358_tiles(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
-                          int64_t ldy, float *y32, hipStream_t s) {
+                          int64_t ldy, float *y32, float *ws, uint32_t ws_pieces, hipStream_t s) {
     if (m < 1 || m > kTMaxM || P.out_f % 4u != 0 || P.in_f % kFastChunk != 0 || P.in_f > 65536u) return IXH_EUNSUPPORTED;
     if (((uintptr_t)x & 15u) != 0 || (m > 1 && (ldx & 7) != 0)) return IXH_EUNSUPPORTED;
     const int opt = g_opt_gemv_tiles.load(std::memory_order_relaxed);  // ixh_set_option("gemv_tiles")
@@ -639,16 +675,20 @@ int launch_gemv_358_tiles(const Dev &P, const int32_t *prefix, const uint16_t *x
     }();
     const uint32_t n_chunks = P.in_f / kFastChunk;
     const int cus_opt = g_opt_gemv_tile_cus.load(std::memory_order_relaxed);
+    const int split_opt = g_opt_gemv_tile_split.load(std::memory_order_relaxed);
+    // pieces need the workspace, or the caller's fp32 sums, which the workgroups add to one by one anyway
+    const uint32_t max_split = y32 ? 8u : (ws ? ws_pieces : 1u);
     const TilesPlan plan = plan_tiles(P.out_f, n_chunks, (uint32_t)(cus_opt > 0 ? cus_opt : n_cu), m,
-                                      g_opt_gemv_tile_rows.load(std::memory_order_relaxed));
+                                      g_opt_gemv_tile_rows.load(std::memory_order_relaxed), max(1u, max_split),
+                                      (uint32_t)(split_opt > 0 ? split_opt : 0));
     if (plan.waves == 0) return IXH_EUNSUPPORTED;
     // by itself from three activation rows on (one or two: the kernels that multiply lane by lane are as fast or faster)
     // and where a workgroup's rows fill its tiles of 16 at least half; forced (option 1) wherever it fits
     const uint32_t tile_rows = 1u << plan.lg_rows;
     if (opt == 0 && (m <= 2 || plan.rows * 2u < ((plan.rows + tile_rows - 1u) / tile_rows) * tile_rows))
         return IXH_EUNSUPPORTED;
-    return any ? launch_tiles<true>(P, prefix, n_chunks, plan, x, m, ldx, y, ldy, y32, s)
-               : launch_tiles<false>(P, prefix, n_chunks, plan, x, m, ldx, y, ldy, y32, s);
+    return any ? launch_tiles<true>(P, prefix, n_chunks, plan, x, m, ldx, y, ldy, y32, ws, s)
+               : launch_tiles<false>(P, prefix, n_chunks, plan, x, m, ldx, y, ldy, y32, ws, s);
 }
 
 }  // namespace ixh

@@ -391,6 +391,48 @@ def test_gemv_tile_shapes(oracle, dev, gemv_option, kind, shape, level_bits, til
 
 
 @pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("shape", [(20, 1024), (68, 5120), (132, 1536), (100, 8704), (48, 17408)])
+@pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8)])
+@pytest.mark.parametrize("split", [2, 3, 4, 7])
+def test_gemv_tile_split(oracle, dev, gemv_option, kind, shape, level_bits, split):
+    """The tile kernel with several workgroups to a block of rows, each taking a run of the rows' column blocks: the
+    pieces go through the workspace (filled with NaN before the call: every piece must be written) and a second launch
+    that adds them, or one by one into the caller's fp32 sums; row blocks several times as tall, pieces of unequal
+    length, pieces held in LDS in several parts, a split that leaves a piece empty (the planner then takes another
+    plan), a workspace too small for pieces (chunk = in_f: no workspace, whole rows per workgroup); the same call
+    twice gives the same bits."""
+    from ixrun_amd import _lib
+
+    out_f, in_f = shape
+    p = make_packed(kind, out_f, in_f, level_bits)
+    dp = device_packed(p, dev)
+    w_bits = oracle.decode_packed_bf16(p)
+    gemv_option("gemv_tiles", 1)
+    gemv_option("gemv_tile_split", split)
+    for cus in (2, 8):
+        gemv_option("gemv_tile_cus", cus)
+        for m in (3, 8, 16):
+            x = activations(m, in_f, seed=m)
+            y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
+            what = f"split {split} on {cus} CUs {kind} {shape} {level_bits} m={m}"
+            y = run_gemv(dp, 512, x, m, dev, flags=_lib.IXH_GEMV_FORCE_358, atomic=True)
+            check_outputs(y, y64, what + " atomic")
+            table = dp.prefix_build(512)
+            xd = x.to(dev)
+            outs = []
+            for _ in range(2):
+                yd = torch.zeros((m, out_f), dtype=torch.bfloat16, device=dev)
+                nbytes = dp.gemv_workspace_bytes(512, m, _lib.IXH_GEMV_FORCE_358)
+                ws = torch.full((max(nbytes // 4, 1),), float("nan"), dtype=torch.float32, device=dev)
+                dp.gemv(table, 512, xd, y=yd, workspace=ws, flags=_lib.IXH_GEMV_FORCE_358)
+                outs.append(bf16_bits(yd))
+            check_outputs(outs[0], y64, what)
+            assert np.array_equal(outs[0], outs[1]), what + ": two calls differ"
+            y = run_gemv(dp, in_f, x, m, dev, flags=_lib.IXH_GEMV_FORCE_358)
+            check_outputs(y, y64, what + " chunk = in_f")
+
+
+@pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("shape", [(64, 512), (37, 1024), (130, 2048), (24, 8704), (5, 25600)])
 @pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8), (5, 8)])
 def test_gemv_staged(oracle, dev, kind, shape, level_bits):
