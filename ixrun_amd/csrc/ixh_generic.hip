@@ -249,19 +249,20 @@ k_reduce_chunks(const float *__restrict__ ws, uint32_t n_chunks, int m, uint32_t
     const uint32_t row = blockIdx.x * 256 + threadIdx.x;
     const int j = blockIdx.y;
     if (row >= out_f) return;
-    // eight loads in flight at a time; the additions stay in chunk order
+    // sixteen loads in flight at a time (the pieces come from memory, written by other workgroups: one after the other
+    // they cost a trip each), the last ones past the end clamped to the last piece and left out of the sum; the additions
+    // stay in chunk order
     const size_t stride = (size_t)m * out_f;
     const float *p = ws + (size_t)j * out_f + row;
     float sum = 0.0f;
-    uint32_t c = 0;
-    for (; c + 8 <= n_chunks; c += 8) {
-        float v[8];
+    for (uint32_t c = 0; c < n_chunks; c += 16) {
+        float v[16];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) v[k] = p[(size_t)(c + k) * stride];
+        for (uint32_t k = 0; k < 16; ++k) v[k] = p[(size_t)min(c + k, n_chunks - 1u) * stride];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) sum += v[k];
+        for (uint32_t k = 0; k < 16; ++k)
+            if (c + k < n_chunks) sum += v[k];
     }
-    for (; c < n_chunks; ++c) sum += p[(size_t)c * stride];
     y[(int64_t)j * ldy + row] = (uint16_t)f32_to_bf16_bits(sum);
 }
 

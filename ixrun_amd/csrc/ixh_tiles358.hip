@@ -1,7 +1,9 @@
 // (3,5,8) fused decode + skinny GEMM for gfx950, tile variant: 16 weight rows x 16 activation rows per matrix
 // instruction, so that up to 16 activation rows cost what one costs.
 //
-// Work split.  A workgroup owns whole rows.  Its rows are cut into tiles of 16, 8 or 4 (one size per launch); a tile of
+// Work split.  A workgroup owns whole rows, or, where rows are few per CU, shares a taller block of rows with k - 1
+// others, each taking a run of the rows' column blocks (their fp32 sums go to a workspace as [piece][m][row] and
+// k_reduce_chunks adds them in piece order): taller blocks fill tiles of 16 and need fewer parts (below).  Its rows are cut into tiles of 16, 8 or 4 (one size per launch); a tile of
 // 16 / s rows takes s column blocks side by side in a step (slots), so that the 16 columns of the matrix instruction
 // are always 16 different (row, block) pairs, and serves up to 16 / s activation rows: row a of the other operand is
 // activation row a % (16 / s) at the columns of slot a / (16 / s), and the products whose slots agree are the sums.
