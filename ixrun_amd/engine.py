@@ -39,6 +39,13 @@ MAX_FUSED_ROWS = 16  # activation rows served by the fused decode+GEMV kernel
 # decoder in its tile mode) against 119-123 us: the pair keeps those (the any-scheme kernel took 209-260 us).
 MAX_FUSED_ROWS_WITH_BUFFER = 16
 MAX_FUSED_ROWS_WITH_BUFFER_DENSE = 16
+# 17 .. 32 rows on a large layer that is almost all level 1: two fused calls (16 rows and the rest) instead of the
+# many-row paths.  MI355X, Student-t weights with 99.4 % of the elements in level 1, hipGraph replays over distinct
+# layers: 5120 x 17408 at 17 / 24 / 32 rows 60 / 70 / 75 us in two calls against 118-120 us fused decode+GEMM and
+# 137 us decode + library GEMM; 17408 x 5120 54 / 60 / 64 us against 120-122 and 87 us.  On 5120 x 5120 the two
+# calls tie with the fused decode+GEMM (37-45 against 44-45 us) and lose to decode + library GEMM (34 us), and three
+# calls for 33 .. 48 rows gain nothing on any shape: large layers and up to 32 rows only.
+SPLIT_FUSED_MIN_WEIGHTS = 40_000_000
 # More rows than that: with a shared decode buffer the layer decodes into it and calls the library GEMM
 # (5120 x 5120 five-level on MI355X: 60 us at 32 rows, 84 us at 512); without one it runs the fused
 # decode+GEMM, which keeps the bf16 weight out of HBM altogether but is slower (84 us and 194 us): its
@@ -144,14 +151,18 @@ class StreamingLinear(nn.Module):
             fused_rows = MAX_FUSED_ROWS_WITH_BUFFER_DENSE
         else:
             fused_rows = 1
-        if (self._use_fused and x.dtype == torch.bfloat16 and x.is_cuda and 1 <= rows <= fused_rows
+        two_calls = (MAX_FUSED_ROWS < rows <= 2 * MAX_FUSED_ROWS and fused_rows == MAX_FUSED_ROWS
+                     and self.N >= SPLIT_FUSED_MIN_WEIGHTS and self.counts[0] * 100 >= self.N * 97)
+        if (self._use_fused and x.dtype == torch.bfloat16 and x.is_cuda and (1 <= rows <= fused_rows or two_calls)
                 and x.shape[-1] == self.in_features):
             x2 = x.reshape(rows, self.in_features)
             if x2.stride(1) != 1:
                 x2 = x2.contiguous()
             y = torch.empty((rows, self.out_features), dtype=torch.bfloat16, device=x.device)
-            ws = shared_workspace(x.device, self._dp.gemv_workspace_bytes(self._unit, rows))
-            self._dp.gemv(self._table, self._unit, x2, y=y, workspace=ws)
+            for r0 in range(0, rows, MAX_FUSED_ROWS):  # one call, or two on the same stream and workspace
+                n = min(MAX_FUSED_ROWS, rows - r0)
+                ws = shared_workspace(x.device, self._dp.gemv_workspace_bytes(self._unit, n))
+                self._dp.gemv(self._table, self._unit, x2[r0:r0 + n], y=y[r0:r0 + n], workspace=ws)
             y = y.view(x.shape[:-1] + (self.out_features,))
             if self._bias is not None:
                 y = y + self._bias.to(y.dtype)

@@ -168,3 +168,37 @@ def test_row_count_policy_with_a_decode_buffer(oracle, rows, dense):
         assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-3
     decoded = bool((buf != 9.0).any())  # the buffer was written iff the pair path ran
     assert decoded == (rows > 16)
+
+
+@pytest.mark.parametrize("rows", [16, 17, 24, 32, 33])
+@pytest.mark.parametrize("buffered", [False, True])
+def test_two_fused_calls_for_17_to_32_rows(oracle, monkeypatch, rows, buffered):
+    """17 .. 32 rows on a large layer that is almost all level 1 go through the fused kernel in two calls (16 rows and
+    the rest), with or without a decode buffer (which then stays untouched); 33 rows and small layers keep the
+    many-row paths.  The size limit is lowered for the test so that a small layer counts as large."""
+    from ixrun_amd import engine
+    from helpers import int8_mix, packed_from_int8
+
+    dev = torch.device("cuda:0")
+    p = packed_from_int8(int8_mix("rare_other", 128 * 2048, seed=7), 128, 2048)
+    assert p["counts"][0] * 100 >= p["N"] * 97
+    x = torch.randn(rows, 2048, generator=torch.Generator("cpu").manual_seed(rows)).bfloat16()
+    w_deq = oracle.bf16_bits_to_f32(oracle.decode_packed_bf16(p)).astype(np.float64).reshape(128, 2048)
+    want = torch.from_numpy(x.double().numpy() @ w_deq.T).bfloat16().double().numpy()
+    for limit, two_calls in ((0, 16 < rows <= 32), (engine.SPLIT_FUSED_MIN_WEIGHTS, False)):
+        monkeypatch.setattr(engine, "SPLIT_FUSED_MIN_WEIGHTS", limit)
+        layer = engine.StreamingLinear(p)
+        buf = torch.full((p["N"],), 9.0, dtype=torch.bfloat16, device=dev)
+        if buffered:
+            layer._set_shared_buf(buf)
+        calls = []
+        real = layer._dp.gemv
+        monkeypatch.setattr(layer._dp, "gemv", lambda *a, **k: (calls.append(a[2].shape[0]), real(*a, **k))[1])
+        got = layer(x.to(dev)).float().cpu().numpy()
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-3
+        if rows <= 16:
+            assert calls == [rows]
+        elif two_calls:
+            assert calls == [16, rows - 16] and not bool((buf != 9.0).any())
+        else:
+            assert calls == [] and bool((buf != 9.0).any()) == buffered
