@@ -189,6 +189,13 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     const uint32_t unit0 = row0 * n_chunks;
     const uint32_t entries = P.out_f * n_chunks + 1;
     const uint32_t n_local = rows_here * n_chunks;
+    // the ranks at the ends of the workgroup's rows (what its share of the side streams is worked out from): asked for
+    // here, so that the share's words can be asked for with the rest of the set-up
+    uint32_t q1b = 0, q2b = 0, q1e = 0, q2e = 0;
+    if (!ANY) {
+        q1b = (uint32_t)prefix[unit0], q2b = (uint32_t)prefix[entries + unit0];
+        q1e = (uint32_t)prefix[unit0 + n_local], q2e = (uint32_t)prefix[entries + unit0 + n_local];
+    }
 
     const __amdgpu_buffer_rsrc_t b1_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[0], 0, (int)(P.bm_words[0] * 4u), 0x00020000);
@@ -242,20 +249,11 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     if (c_begin < c_end) request(c_begin, T);
 
     // ---- workgroup set-up: activations, table slices, side streams, pair table, splice masks ----
-    // activation rows of the part's columns into padded strips: 16-byte piece p of row i holds columns 8p .. 8p+7
-    auto load_activations = [&]() __attribute__((always_inline)) {
-        const uint32_t pieces = part_count * (kFastChunk / 8), first_piece = part_first * (kFastChunk / 8);
-        uint32_t t0 = threadIdx.x;
-        asm volatile("" : "+v"(t0));  // worked out anew at every call: no register is held for it across the loop
-        // eight loads of a thread in flight at a time, then their stores: one piece a trip to memory (a loop of load
-        // and store) made a part of five column blocks at 16 activation rows eight trips long.  Row and piece are
-        // stepped, not divided out, for every load.
-        const uint32_t total = (uint32_t)m * pieces, stride = blockDim.x;
-        const uint32_t di = stride / pieces, dp = stride - di * pieces;
-        uint32_t i = t0 / pieces, p = t0 - i * pieces;
-        for (uint32_t tb = t0, done = 0; tb < total; tb += 8u * stride, done += 8u * stride) {
-            // (named registers, not an array: the array went to scratch memory; a slot that no thread of the workgroup
-            // needs is skipped by a scalar branch)
+    // activation rows of the part's columns into padded strips: 16-byte piece p of row i holds columns 8p .. 8p+7.
+    // Eight loads of a thread in flight at a time, then their stores: one piece a trip to memory (a loop of load and
+    // store) made a part of five column blocks at 16 activation rows eight trips long.  Row and piece are stepped, not
+    // divided out, for every load.  (Named registers, not an array: the array went to scratch memory; a slot that no
+    // thread of the workgroup needs is skipped by a scalar branch.)
 #define IXH_T_LOAD(u)                                                                                              \
     const bool any##u = done + (uint32_t)(u) * stride < total;                                                      \
     uint4 v##u = make_uint4(0, 0, 0, 0);                                                                            \
@@ -271,29 +269,56 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
             ++i;                                                                                                    \
         }                                                                                                           \
     }
-            IXH_T_LOAD(0) IXH_T_LOAD(1) IXH_T_LOAD(2) IXH_T_LOAD(3) IXH_T_LOAD(4) IXH_T_LOAD(5) IXH_T_LOAD(6) IXH_T_LOAD(7)
-#undef IXH_T_LOAD
 #define IXH_T_STORE(u) \
     if (at##u != ~0u) *reinterpret_cast<uint4 *>(smem + at##u) = v##u;
-            IXH_T_STORE(0) IXH_T_STORE(1) IXH_T_STORE(2) IXH_T_STORE(3) IXH_T_STORE(4) IXH_T_STORE(5) IXH_T_STORE(6) IXH_T_STORE(7)
-#undef IXH_T_STORE
+#define IXH_T_LOAD_ALL IXH_T_LOAD(0) IXH_T_LOAD(1) IXH_T_LOAD(2) IXH_T_LOAD(3) IXH_T_LOAD(4) IXH_T_LOAD(5) IXH_T_LOAD(6) IXH_T_LOAD(7)
+#define IXH_T_STORE_ALL IXH_T_STORE(0) IXH_T_STORE(1) IXH_T_STORE(2) IXH_T_STORE(3) IXH_T_STORE(4) IXH_T_STORE(5) IXH_T_STORE(6) IXH_T_STORE(7)
+#define IXH_T_COPY_STATE                                                                                            \
+    const uint32_t pieces = part_count * (kFastChunk / 8), first_piece = part_first * (kFastChunk / 8);             \
+    uint32_t t0 = threadIdx.x;                                                                                      \
+    asm volatile("" : "+v"(t0)); /* worked out anew at every call: no register is held for it across the loop */    \
+    const uint32_t total = (uint32_t)m * pieces, stride = blockDim.x;                                               \
+    const uint32_t di = stride / pieces, dp = stride - di * pieces;                                                 \
+    uint32_t i = t0 / pieces, p = t0 - i * pieces;                                                                  \
+    uint32_t tb = t0, done = 0;
+    auto load_activations = [&]() __attribute__((always_inline)) {
+        IXH_T_COPY_STATE
+        for (; tb < total; tb += 8u * stride, done += 8u * stride) {
+            IXH_T_LOAD_ALL
+            IXH_T_STORE_ALL
         }
     };
-    load_activations();
-    for (uint32_t t = tid; t < kTStripBytes / 4; t += blockDim.x) reinterpret_cast<uint32_t *>(smem + L.zero)[t] = 0u;
-    for (uint32_t i = tid; i <= n_local; i += blockDim.x) {
-        tq1[i] = (uint32_t)prefix[unit0 + i];
-        if (!ANY) tq2[i] = (uint32_t)prefix[entries + unit0 + i];
-    }
+    // The set-up's loads are all asked for before the first of them is stored: the first eight pieces of a thread's
+    // activations, its first table entries, its first two words of the side streams.  One phase after the other, each
+    // waiting for its own loads, the set-up was four trips to memory long.
+    IXH_T_COPY_STATE
+    IXH_T_LOAD_ALL
+    const uint32_t n_tbl = n_local + 1u;
+    const uint32_t tbl_i = min(tid, n_local);
+    const uint32_t tbl_1 = (uint32_t)prefix[unit0 + tbl_i];
+    const uint32_t tbl_2 = ANY ? 0u : (uint32_t)prefix[entries + unit0 + tbl_i];
     // this workgroup's share of bitmap 1 and of the 5-bit / 8-bit streams: small when few elements are above level 1,
     // then it is staged in LDS and resolving them touches no global memory
     SideView sv;
     sv.staged = false;
     sv.base = L.side;
     sv.b2w0 = sv.l2w0 = sv.l3w0 = 0;
+    const uint32_t *const last32 = reinterpret_cast<const uint32_t *>(P.last);
+    const uint32_t last_words = (P.last_bytes + 3u) >> 2;  // whole dwords (allocations are 256-byte granular)
+    auto side_word = [&](uint32_t t) -> uint32_t {  // word t of the staged share (past a stream's end: zero)
+        if (t < 256) {
+            const uint32_t w = sv.b2w0 + t;
+            return w < P.bm_words[1] ? P.bm[1][w] : 0u;
+        }
+        if (t < 768) {
+            const uint32_t w = sv.l2w0 + (t - 256);
+            return w < P.st_words[1] ? P.st[1][w] : 0u;
+        }
+        const uint32_t w = sv.l3w0 + (t - 768);
+        return w < last_words ? last32[w] : 0u;
+    };
+    uint32_t side_0 = 0, side_1 = 0;
     if (!ANY) {
-        const uint32_t q1b = (uint32_t)prefix[unit0], q2b = (uint32_t)prefix[entries + unit0];
-        const uint32_t q1e = (uint32_t)prefix[unit0 + n_local], q2e = (uint32_t)prefix[entries + unit0 + n_local];
         const uint32_t nl1b = row0 * P.in_f - q1b, nl1e = (row0 + rows_here) * P.in_f - q1e;
         sv.b2w0 = nl1b >> 5;
         sv.l2w0 = (uint32_t)(((uint64_t)q2b * 5u) >> 5);
@@ -304,25 +329,37 @@ k_gemv358_tiles(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
         // one word of slack each: the resolver reads the word after a code's first word unconditionally
         sv.staged = (flags & kFlagStageSide) && n_b2 < 256 && n_l2 < 511 && n_l3 <= 256;
         if (sv.staged) {
-            uint32_t *side = reinterpret_cast<uint32_t *>(smem + L.side);
-            const uint32_t *last32 = reinterpret_cast<const uint32_t *>(P.last);
-            const uint32_t last_words = (P.last_bytes + 3u) >> 2;  // whole dwords (allocations are 256-byte granular)
-            for (uint32_t t = tid; t < kRSideBytes / 4; t += blockDim.x) {
-                uint32_t v = 0;
-                if (t < 256) {
-                    const uint32_t w = sv.b2w0 + t;
-                    if (w < P.bm_words[1]) v = P.bm[1][w];
-                } else if (t < 768) {
-                    const uint32_t w = sv.l2w0 + (t - 256);
-                    if (w < P.st_words[1]) v = P.st[1][w];
-                } else {
-                    const uint32_t w = sv.l3w0 + (t - 768);
-                    if (w < last_words) v = last32[w];
-                }
-                side[t] = v;
-            }
+            if (tid < kRSideBytes / 4) side_0 = side_word(tid);
+            if (tid + blockDim.x < kRSideBytes / 4) side_1 = side_word(tid + blockDim.x);
         }
     }
+    // what needs no memory: the strip of zeros (the pair table and the splice masks follow below)
+    for (uint32_t t = tid; t < kTStripBytes / 4; t += blockDim.x) reinterpret_cast<uint32_t *>(smem + L.zero)[t] = 0u;
+    // the stores, in the order of the requests, and what one request per thread did not cover
+    IXH_T_STORE_ALL
+    for (tb += 8u * stride, done += 8u * stride; tb < total; tb += 8u * stride, done += 8u * stride) {
+        IXH_T_LOAD_ALL
+        IXH_T_STORE_ALL
+    }
+    if (tid < n_tbl) {
+        tq1[tid] = tbl_1;
+        if (!ANY) tq2[tid] = tbl_2;
+    }
+    for (uint32_t i2 = tid + blockDim.x; i2 < n_tbl; i2 += blockDim.x) {
+        tq1[i2] = (uint32_t)prefix[unit0 + i2];
+        if (!ANY) tq2[i2] = (uint32_t)prefix[entries + unit0 + i2];
+    }
+    if (!ANY && sv.staged) {
+        uint32_t *side = reinterpret_cast<uint32_t *>(smem + L.side);
+        if (tid < kRSideBytes / 4) side[tid] = side_0;
+        if (tid + blockDim.x < kRSideBytes / 4) side[tid + blockDim.x] = side_1;
+        for (uint32_t t = tid + 2u * blockDim.x; t < kRSideBytes / 4; t += blockDim.x) side[t] = side_word(t);
+    }
+#undef IXH_T_COPY_STATE
+#undef IXH_T_LOAD_ALL
+#undef IXH_T_STORE_ALL
+#undef IXH_T_LOAD
+#undef IXH_T_STORE
     const float scale = bf16_bits_to_f32(scale_bits);
     for (uint32_t i = tid; i < 64 * 32; i += blockDim.x) {
         const int c0 = (i >> 5) & 7, c1 = i >> 8;
