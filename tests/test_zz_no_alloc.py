@@ -70,6 +70,26 @@ def test_noalloc_equals_gemv_twice_in_a_row(dev, recipe, level_bits, m):
     assert used > 0  # at least one of the routes really went through the buffer
 
 
+@pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8)])
+@pytest.mark.parametrize("m", [3, 8, 16])
+def test_noalloc_with_row_blocks_shared_by_workgroups(dev, gemv_option, level_bits, m):
+    """The tile kernel with two and three workgroups to a block of rows: their partial sums meet in the built-in
+    buffer and a second launch adds them.  Twice in a row, the smaller tensor second."""
+    from ixrun_amd import _lib
+
+    big, big_t = _layer("student_t", 640, 4608, dev, level_bits)
+    small, small_t = _layer("student_t", 96, 1536, dev, level_bits)
+    gemv_option("gemv_tiles", 1)
+    gemv_option("gemv_tile_cus", 4)
+    for split in (2, 3):
+        gemv_option("gemv_tile_split", split)
+        for dp, table in ((big, big_t), (small, small_t)):
+            x = activations(m, dp.in_f, seed=5 + m).to(dev)
+            y_ref, y_new, need = _both(dp, table, x, _lib.IXH_GEMV_FORCE_358, dev)
+            assert 0 < need <= LIMIT
+            assert np.array_equal(y_ref, y_new), (level_bits, m, split, dp.out_f)
+
+
 def test_noalloc_rejects_what_does_not_fit(dev):
     """A request whose partial sums exceed the built-in buffer fails with IXH_EWORKSPACE before anything is launched
     (the table handed in is a real one for that chunk, so even a wrongly accepted call would run validly); the
