@@ -38,9 +38,15 @@ def run_chain(layers, x):
 @pytest.mark.parametrize("maker,m,level_bits", [
     (student_t_weight, 1, (3, 5, 8)), (outlier_weight, 1, (3, 5, 8)), (student_t_weight, 4, (3, 5, 8)),
     (outlier_weight, 16, (3, 5, 8)), (dense_weight, 1, (3, 4, 5, 6, 8)), (student_t_weight, 16, (3, 4, 5, 6, 8)),
-    (dense_weight, 2, (3, 5, 8)), (dense_weight, 8, (3, 5, 8)), (dense_weight, 16, (3, 5, 8)), (student_t_weight, 8, (3, 5, 8))])
-def test_graph_replay_matches_eager(maker, m, level_bits):
+    (dense_weight, 2, (3, 5, 8)), (dense_weight, 8, (3, 5, 8)), (dense_weight, 16, (3, 5, 8)), (student_t_weight, 8, (3, 5, 8)),
+    (student_t_weight, -8, (3, 5, 8)), (student_t_weight, -16, (3, 4, 5, 6, 8))])
+def test_graph_replay_matches_eager(maker, m, level_bits, gemv_option):
     dev = torch.device("cuda:0")
+    if m < 0:  # the tile kernel with two workgroups to a block of rows: two launches a layer, pieces in the shared scratch
+        m = -m
+        gemv_option("gemv_tiles", 1)
+        gemv_option("gemv_tile_cus", 8)
+        gemv_option("gemv_tile_split", 2)
     layers = build_chain(6, 1024, dev, maker, level_bits)
     x = activations(m, 1024, seed=3).to(dev)
     eager = run_chain(layers, x).clone()
