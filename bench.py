@@ -75,17 +75,17 @@ WORKLOADS = {
     "attn_proj_5120x5120_m1_student_t": (5120, 5120, 1, "student_t"),
     "down_proj_5120x17408_m4_student_t": (5120, 17408, 4, "student_t"),
     "down_proj_5120x17408_m8_student_t": (5120, 17408, 8, "student_t"),
-    "down_proj_5120x17408_m16_student_t": (27676.0 * 2.0 * 1024 + 960.0 * 1024, _TILES, "9b8732b9ed8225da"),
+    "down_proj_5120x17408_m16_student_t": (5120, 17408, 16, "student_t"),
     "down_proj_5120x17408_m2_student_t": (5120, 17408, 2, "student_t"),
     "attn_proj_5120x5120_m2_student_t": (5120, 5120, 2, "student_t"),
     "attn_proj_5120x5120_m4_student_t": (5120, 5120, 4, "student_t"),
     "attn_proj_5120x5120_m8_student_t": (5120, 5120, 8, "student_t"),
-    "attn_proj_5120x5120_m16_student_t": (8657.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "9b8732b9ed8225da"),
+    "attn_proj_5120x5120_m16_student_t": (5120, 5120, 16, "student_t"),
     "gate_up_17408x5120_m1_student_t": (17408, 5120, 1, "student_t"),
     "gate_up_17408x5120_m2_student_t": (17408, 5120, 2, "student_t"),
-    "gate_up_17408x5120_m4_student_t": (28674.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "9b8732b9ed8225da"),
+    "gate_up_17408x5120_m4_student_t": (17408, 5120, 4, "student_t"),
     "gate_up_17408x5120_m8_student_t": (17408, 5120, 8, "student_t"),
-    "gate_up_17408x5120_m16_student_t": (26631.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "9b8732b9ed8225da"),
+    "gate_up_17408x5120_m16_student_t": (17408, 5120, 16, "student_t"),
     "gate_up_17408x5120_m2_calibrated": (17408, 5120, 2, "calibrated"),
     "gate_up_17408x5120_m4_calibrated": (17408, 5120, 4, "calibrated"),
     "gate_up_17408x5120_m8_calibrated": (17408, 5120, 8, "calibrated"),

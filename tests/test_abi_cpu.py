@@ -130,3 +130,26 @@ def test_missing_library_is_loud(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libixhip.so")
     with pytest.raises(RuntimeError, match="no fallback"):
         _lib.lib()
+
+
+def test_bench_tables_are_well_formed():
+    """bench.py's workload table (shape, rows, recipe[, level scheme]) and its table of measured HBM traffic, whose
+    entries name sources that exist and workloads that the first table holds."""
+    import os
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    sys.path.insert(0, root)
+    try:
+        import bench
+    finally:
+        sys.path.remove(root)
+    for name, spec in bench.WORKLOADS.items():
+        assert len(spec) in (4, 5), name
+        out_f, in_f, m, recipe = spec[:4]
+        assert isinstance(out_f, int) and isinstance(in_f, int) and isinstance(m, int) and isinstance(recipe, str), name
+        assert out_f > 0 and in_f > 0 and 0 <= m <= 512, name  # m = 0: decode and encode workloads
+    for name, (nbytes, files, sha16) in bench.MEASURED_TRAFFIC_BYTES.items():
+        assert nbytes > 0 and isinstance(sha16, str), name
+        for f in files:
+            assert os.path.exists(os.path.join(root, "ixrun_amd", "csrc", f)), (name, f)
