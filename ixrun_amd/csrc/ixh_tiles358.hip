@@ -616,11 +616,13 @@ struct TilesPlan {
 // taking a run of its column blocks.  A tile of 16 >> k rows takes 1 << k column blocks per step and serves 16 >> k
 // activation rows, so short tiles suit workgroups whose rows are not a multiple of 16 when the rows of activations are
 // few.  A wave's time goes with the steps it decodes, and every further part costs two barriers and a copy: the plan
-// with the fewest steps per wave, a part counted as a third of a step (costs that also count the steps of all waves of
+// with the fewest steps per wave, a part counted as 0.6 of a step (costs that also count the steps of all waves of
 // a CU, or of a SIMD, chose slower plans on the shapes measured).  Sharing the rows' columns among k workgroups makes
 // the row blocks k times as tall, which fills tiles of 16 that a short block leaves mostly empty and takes k times
 // fewer parts per workgroup; it costs the second launch that adds the pieces (kSplitCost steps).
-constexpr float kSetupCost = 2.5f, kSplitCost = 1.0f;  // in steps: a round's set-up and final sums; the second launch
+// In steps: a further part (the wait at its two barriers and the loop's restart), a round's set-up and final sums,
+// the second launch.
+constexpr float kPartCost = 0.6f, kSetupCost = 2.5f, kSplitCost = 1.0f;
 static TilesPlan plan_tiles(uint32_t out_f, uint32_t n_chunks, uint32_t n_cu, int m, int lg_only, uint32_t max_split,
                             uint32_t split_only) {
     const uint32_t n_quads = (out_f + 3) / 4, max_quads = kTMaxRows / 4;
@@ -657,7 +659,7 @@ static TilesPlan plan_tiles(uint32_t out_f, uint32_t n_chunks, uint32_t n_cu, in
                     }
                     here.rows = rows, here.n_sub = subs, here.x_blocks = x_blocks, here.qcap = qcap;
                     here.waves = tiles * subs;
-                    here.cost = (float)rounds * ((float)per_wave + (float)(parts - 1) / 3.0f + kSetupCost) +
+                    here.cost = (float)rounds * ((float)per_wave + (float)(parts - 1) * kPartCost + kSetupCost) +
                                 (k_split > 1 ? kSplitCost : 0.0f);
                 }
                 if (here.waves != 0 && (best.waves == 0 || here.cost < best.cost)) best = here;

@@ -642,11 +642,11 @@ def down_proj_layer(oracle, dev):
     return StreamingLinear(p), oracle.decode_packed_bf16(p)
 
 
-@pytest.mark.parametrize("m", [3, 6, 8, 12, 16, 24])
+@pytest.mark.parametrize("m", [3, 6, 8, 9, 10, 12, 16, 24])
 def test_full_size_down_proj_many_rows(oracle, dev, down_proj_layer, m):
     """5120 x 17408 with 3..16 activation rows as the library plans them on the whole device: 20 rows to a workgroup
-    and three column parts at 3 rows; blocks of 80 and 64 rows shared by four and three workgroups, each with a run of
-    the column blocks, at 5..8 and 9..16 rows (their sums added by a second launch); 24 rows in two calls."""
+    at one or two activation rows; from three rows on blocks of 40 to 124 rows shared by two to six workgroups, each
+    with a run of the column blocks (their sums added by a second launch); 24 rows in two calls."""
     sl, w_bits = down_proj_layer
     x = activations(m, 17408, seed=m)
     y = sl(x.to(dev))
