@@ -30,9 +30,9 @@ __all__ = ["Int8XEngine", "StreamingLinear", "GraphLinear", "ResourceScheduler"]
 MAX_FUSED_ROWS = 16  # activation rows served by the fused decode+GEMV kernel
 # With a decode buffer at hand, more rows than this go through decode + library GEMM.  Tensors that are almost all
 # level 1, MI355X: the pair takes 72-75 us on 17408 x 5120 and 5120 x 17408 at any M up to 32 and 34-50 us on
-# 5120 x 5120 (five levels: 73-74 and 38-39 us); the fused kernels take 27 / 31 / 31 us (17408 x 5120), 35 / 45 / 48 us
-# (5120 x 17408) and 20 / 24 / 26 us (5120 x 5120) at M = 8 / 12 / 16 (five levels: 29 / 31 / 32, 39 / 45 / 51 and
-# 23 / 31 / 31 us): every row count the fused kernels take.  Dense mixes (55 / 40 / 5 %): the pair takes
+# 5120 x 5120 (five levels: 73-74 and 38-39 us); the fused kernels take 25 / 27 us (17408 x 5120), 27 / 30 us
+# (5120 x 17408) and 15 / 18 us (5120 x 5120) at M = 8 / 16 (five levels, measured before several workgroups could share
+# a block of rows: 29 / 32, 39 / 51 and 23 / 31 us): every row count the fused kernels take.  Dense mixes (55 / 40 / 5 %): the pair takes
 # 91-93 us on the large layers and 34-52 us on 5120 x 5120, the fused kernels 54-62 / 69-73 / 79-85 / 80-85 / 83-88 us
 # (large layers) and 21 / 26 / 29 / 29 / 31 us (5120 x 5120) at M = 1 / 2 / 4 / 8 / 16: every row count as well.  Dense
 # five-level mixes: one row 97-105 us fused against 120 us for the pair; two to sixteen rows 113-126 us fused (the
