@@ -166,7 +166,8 @@ int ixh_decode_gs(const IxhPacked *packed, const int32_t *prefix, int64_t chunk,
  * (ixh_gemv_workspace_bytes) and written to y, or, with IXH_GEMV_ATOMIC, added
  * into the caller-zeroed fp32 y32 [M, out_f] with atomics as the reference's
  * split kernel does (fused.py:294); y may then be NULL.  Kernels that own whole
- * rows add each output once (the same kernels as without the flag, up to 8 rows).
+ * rows add each output once, those whose workgroups share a block of rows once per
+ * workgroup of the block (the same kernels as without the flag).
  */
 int ixh_gemv(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, const uint16_t *x,
              int32_t m, int64_t ldx, uint16_t *y, int64_t ldy, float *y32, void *workspace,
