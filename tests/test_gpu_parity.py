@@ -398,8 +398,8 @@ def test_gemv_tile_split(oracle, dev, gemv_option, kind, shape, level_bits, spli
     """The tile kernel with several workgroups to a block of rows, each taking a run of the rows' column blocks: the
     pieces go through the workspace (filled with NaN before the call: every piece must be written) and a second launch
     that adds them, or one by one into the caller's fp32 sums; row blocks several times as tall, pieces of unequal
-    length, pieces held in LDS in several parts, a split that leaves a piece empty (the planner then takes another
-    plan), a workspace too small for pieces (chunk = in_f: no workspace, whole rows per workgroup); the same call
+    length, pieces held in LDS in several parts, a split that would leave a piece empty (the call then goes on to the
+    next kernel), a workspace too small for pieces (chunk = in_f: no workspace, whole rows per workgroup); the same call
     twice gives the same bits."""
     from ixrun_amd import _lib
 
