@@ -45,10 +45,10 @@ MEASURED_TRAFFIC_BYTES = {
     "attn_proj_5120x5120_m1_student_t": (7139.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "e45341197bdab021"),
     "down_proj_5120x17408_m1_calibrated": (33825.0 * 2.0 * 1024 + 40.0 * 1024, _DENSE, "711eef94d053feb1"),
     "down_proj_5120x17408_m1_five_level_calibrated": (49708.0 * 2.0 * 1024 + 1338.0 * 1024, _DENSE5, "aaca19573f1ed2a1"),
-    "gate_up_17408x5120_m4_student_t": (28674.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "1315b882c804111a"),
-    "gate_up_17408x5120_m16_student_t": (26631.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "1315b882c804111a"),
-    "attn_proj_5120x5120_m16_student_t": (8657.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "1315b882c804111a"),
-    "down_proj_5120x17408_m16_student_t": (27676.0 * 2.0 * 1024 + 960.0 * 1024, _TILES, "1315b882c804111a"),
+    "gate_up_17408x5120_m4_student_t": (28674.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "3287305ecb77f4e3"),
+    "gate_up_17408x5120_m16_student_t": (26631.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "3287305ecb77f4e3"),
+    "attn_proj_5120x5120_m16_student_t": (8657.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "3287305ecb77f4e3"),
+    "down_proj_5120x17408_m16_student_t": (27676.0 * 2.0 * 1024 + 960.0 * 1024, _TILES, "3287305ecb77f4e3"),
     "decode_5120x17408_five_level_calibrated": (49719.0 * 2.0 * 1024 + 174080.0 * 1024, _DENSE5, "aaca19573f1ed2a1"),
     "prefill_5120x5120_m512_five_level": (50297.9 * 2.0 * 1024 + 30720.0 * 1024,) + _OLD,
     "decode_5120x17408_student_t": (23268.0 * 2.0 * 1024 + 179524.0 * 1024,) + _OLD,

@@ -622,7 +622,7 @@ struct TilesPlan {
 // fewer parts per workgroup; it costs the second launch that adds the pieces (kSplitCost steps).
 // In steps: a further part (the wait at its two barriers and the loop's restart), a round's set-up and final sums,
 // the second launch.
-constexpr float kPartCost = 0.6f, kSetupCost = 2.5f, kSplitCost = 1.0f;
+constexpr float kPartCost = 0.6f, kSetupCost = 2.5f, kSplitCost = 0.9f;
 static TilesPlan plan_tiles(uint32_t out_f, uint32_t n_chunks, uint32_t n_cu, int m, int lg_only, uint32_t max_split,
                             uint32_t split_only) {
     const uint32_t n_quads = (out_f + 3) / 4, max_quads = kTMaxRows / 4;
