@@ -22,6 +22,8 @@ std::atomic<int> g_opt_gemv_tile_rows{0};
 std::atomic<int> g_opt_gemv_tile_cus{0};
 std::atomic<int> g_opt_gemv_tile_split{0};
 std::atomic<int> g_opt_gemv_dense_tiles{0};
+extern std::atomic<int> g_opt_gemv_slots;
+extern std::atomic<int> g_opt_gemv_slot_waves;
 
 void set_error(const char *fmt, ...) {
     va_list ap;
@@ -129,6 +131,16 @@ int ixh_set_option(const char *name, int64_t value) {
     if (strcmp(name, "gemv_dense_tiles") == 0) {
         if (value < -1 || value > 1) { set_error("gemv_dense_tiles %lld not in -1..1", (long long)value); return IXH_EINVAL; }
         g_opt_gemv_dense_tiles.store((int)value, std::memory_order_relaxed);
+        return IXH_OK;
+    }
+    if (strcmp(name, "gemv_slots") == 0) {
+        if (value < -1 || value > 1) { set_error("gemv_slots %lld not in -1..1", (long long)value); return IXH_EINVAL; }
+        g_opt_gemv_slots.store((int)value, std::memory_order_relaxed);
+        return IXH_OK;
+    }
+    if (strcmp(name, "gemv_slot_waves") == 0) {
+        if (value != 0 && (value < 8 || value > 16)) { set_error("gemv_slot_waves %lld not 0 or 8..16", (long long)value); return IXH_EINVAL; }
+        g_opt_gemv_slot_waves.store((int)value, std::memory_order_relaxed);
         return IXH_OK;
     }
     if (strcmp(name, "gemv_strips") == 0) {

@@ -16,6 +16,10 @@ int launch_gemv_358(const Dev &P, const int32_t *prefix, uint32_t chunk, const u
 // not touched
 int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
                          int64_t ldy, float *y32, hipStream_t s);
+// slot kernel (ixh_slots358.hip): the row-block decode with the products on the matrix pipe, up to four activation
+// rows, rows a multiple of four; same contract
+int launch_gemv_358_slots(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
+                          int64_t ldy, float *y32, hipStream_t s);
 // strip kernel (ixh_strips358.hip): up to four activation rows, products on the matrix pipe; same contract
 int launch_gemv_358_strips(const Dev &P, const int32_t *prefix, const uint16_t *x, int m, int64_t ldx, uint16_t *y,
                            int64_t ldy, float *y32, hipStream_t s);

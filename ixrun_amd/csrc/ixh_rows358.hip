@@ -952,6 +952,10 @@ int launch_gemv_358_rows(const Dev &P, const int32_t *prefix, const uint16_t *x,
     const bool any = !(P.n_levels == 3 && P.bits[1] == 5);  // not (3,5,8): the resolver that walks the nested bitmaps
     if (((uintptr_t)x & 15u) != 0 || (m > 1 && (ldx & 7) != 0)) return IXH_EUNSUPPORTED;
     const uint32_t n_chunks = P.in_f / kFastChunk;
+    if (m <= 4) {  // products on the matrix pipe (ixh_slots358.hip)
+        const int rc = launch_gemv_358_slots(P, prefix, x, m, ldx, y, ldy, y32, s);
+        if (rc != IXH_EUNSUPPORTED) return rc;
+    }
     // option "gemv_shared_x" (ixh_set_option): 0 = never the shared-x kernel, 1 = for one activation row only, 2 = up
     // to two rows, 4 = up to four, 8 = up to eight (default)
     const int shared_x = g_opt_gemv_shared_x.load(std::memory_order_relaxed);

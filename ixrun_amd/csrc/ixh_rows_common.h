@@ -148,7 +148,10 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
 // first column k_first); 1 = the workgroup's shared, swizzled copy of the whole x rows (xs_row bytes apart): 16-byte
 // piece p of the 64 bytes that lane l of a 16-lane row owns in a column block sits at piece p * 16 + l of the block;
 // 2 = the workgroup's shared copy, from column k_first (a multiple of 128) on, in strips of 128 columns, STRIP bytes
-// apart (xs_row bytes between rows).
+// apart (xs_row bytes between rows); 3 = as 1, with the column blocks kSkewedBlock bytes apart instead of 1024 and
+// records of 8 bytes: the bitmap word, and {level-1 elements of the unit before the word (9 bits), word of the unit
+// << 9, column block << 13, row of the workgroup << 20}; n_blocks is then the number of column blocks of a row.
+constexpr uint32_t kSkewedBlock = kFastChunk * 2 + 16;  // neighbouring column blocks start four LDS banks apart
 constexpr uint32_t kStripBytes = 264;  // 128 bf16 + 8: neighbouring strips start two LDS banks apart
 
 // POOL: the elements come from a task list that the waves of the workgroup filled together (entry = wave << 18 |
@@ -181,7 +184,9 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
                                              uint32_t rowacc_addr, uint16_t *__restrict__ tasks,
                                              uint32_t xs_addr, uint32_t xs_row, uint32_t k_first,
                                              int m, float scale, uint32_t lane,
-                                             const int32_t *__restrict__ prefix, uint32_t entries, TaskPool pool) {
+                                             const int32_t *__restrict__ prefix, uint32_t entries, TaskPool pool,
+                                             uint32_t n_blocks = 0) {
+    constexpr bool kCompact = SINK::active || XL == 3;
     const uint32_t *__restrict__ b2 = P.bm[1];
     const uint32_t b2_words = P.bm_words[1];
     // value of the element at rank r of bitmap 1's domain, unit `unit`, any scheme
@@ -228,6 +233,14 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
         uint32_t r0_lane = rec.y, unit = rec.z, k0 = rec.w & 0xFFFFu;
         uint32_t slot = rec.w >> 16;
         if (SINK::active) sink.unpack(rec.y, unit0, tq1_addr, r0_lane, unit, k0, slot);
+        if (XL == 3) {
+            const uint32_t in_unit = ((rec.y >> 9) & 15u) * 32u, col = (rec.y >> 13) & 127u;
+            slot = rec.y >> 20;
+            const uint32_t tidx = slot * n_blocks + col;
+            unit = unit0 + tidx;
+            r0_lane = unit * kFastChunk + in_unit - (lds_u32(tq1_addr + tidx * 4u) + (rec.y & 511u));
+            k0 = col * kFastChunk + in_unit;
+        }
         if (XL == 1) {  // the shared-x kernel's records: rank offset in the unit, LDS address of the unit's table
                     // entry, column block << 4 | lane
             const uint32_t in_unit = (rec.w & 15u) * 32u;
@@ -250,8 +263,8 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
         uint32_t xe[XL == 2 ? 1 : MT];  // the activations this element meets
 #pragma unroll
         for (int j = 0; j < (XL == 2 ? 0 : MT); ++j) {
-            if (XL == 1)
-                xe[j] = lds_u16(xs_addr + (uint32_t)j * xs_row + (k0 >> 9) * (kFastChunk * 2) +
+            if (XL == 1 || XL == 3)
+                xe[j] = lds_u16(xs_addr + (uint32_t)j * xs_row + (k0 >> 9) * (XL == 3 ? kSkewedBlock : kFastChunk * 2) +
                                 (((e >> 3) * 16u + ((k0 >> 5) & 15u)) * 16u) + (e & 7u) * 2u);
             else
                 xe[j] = lds_u16(xs_addr + ((uint32_t)j * xs_row + k0 - k_first + e) * 2u);
@@ -349,8 +362,8 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
     for (uint32_t base = 0; base < count; base += (kTwo ? 2 : 1) * kWave) {
         const uint32_t idx_a = base + lane, idx_b = idx_a + kWave;
         uint32_t zeros_a = 0, zeros_b = 0;
-        if (idx_a < count) zeros_a = read_record<SINK::active>(queue, idx_a).x;
-        if (kTwo && idx_b < count) zeros_b = read_record<SINK::active>(queue, idx_b).x;
+        if (idx_a < count) zeros_a = read_record<kCompact>(queue, idx_a).x;
+        if (kTwo && idx_b < count) zeros_b = read_record<kCompact>(queue, idx_b).x;
         const uint32_t mine_a = (uint32_t)__popc(zeros_a), mine_b = (uint32_t)__popc(zeros_b);
         const uint32_t incl = wave_scan(mine_a | (mine_b << 16));  // at most 64 x 32 elements each: 12 bits
         const uint32_t totals = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
@@ -373,7 +386,7 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
                 }
                 if (tb + lane < n_tasks) {
                     const uint32_t task = tasks[tb + lane];
-                    const uint4 rec = read_record<SINK::active>(queue, base + (task >> 5));
+                    const uint4 rec = read_record<kCompact>(queue, base + (task >> 5));
                     const uint32_t e = task & 31u;
                     one(rec, (uint32_t)__popc(rec.x & ((1u << e) - 1u)), e, Later{});
                 } else if (SINK::active) {
@@ -395,7 +408,7 @@ __device__ __forceinline__ void resolve_rows_to(SINK &sink, const Dev &P, const 
         for (uint32_t half = 0; half < (kTwo ? 2u : 1u); ++half) {
             const uint32_t idx = half == 0 ? idx_a : idx_b;
             uint4 rec = make_uint4(0, 0, 0, 0);
-            if (idx < count) rec = read_record<SINK::active>(queue, idx);
+            if (idx < count) rec = read_record<kCompact>(queue, idx);
             uint32_t zeros = rec.x, nth = 0;
             if (SINK::active) {
                 for (uint64_t left = __ballot(zeros != 0); left != 0; left = __ballot(zeros != 0)) {
@@ -427,10 +440,10 @@ __device__ __forceinline__ void resolve_rows(const Dev &P, const SideView &sv, u
                                              uint32_t xs_addr, uint32_t xs_row, uint32_t k_first,
                                              int m, float scale, uint32_t lane,
                                              const int32_t *__restrict__ prefix = nullptr, uint32_t entries = 0,
-                                             TaskPool pool = TaskPool{0, 0, 0, 1, 0, 0}) {
+                                             TaskPool pool = TaskPool{0, 0, 0, 1, 0, 0}, uint32_t n_blocks = 0) {
     NoSink none;
     resolve_rows_to<MT, STAGED, ANY, XL, POOL, STRIP>(none, P, sv, tq1_addr, tq2_addr, unit0, queue, count, rowacc_addr, tasks,
-                                                      xs_addr, xs_row, k_first, m, scale, lane, prefix, entries, pool);
+                                                      xs_addr, xs_row, k_first, m, scale, lane, prefix, entries, pool, n_blocks);
 }
 
 // s_setprio takes an immediate

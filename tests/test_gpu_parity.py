@@ -363,6 +363,35 @@ def test_gemv_strip_and_tile_kernels(oracle, dev, gemv_option, kind, shape, leve
 
 
 @pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("shape", [(8, 512), (64, 512), (40, 1536), (20, 17408), (68, 5120), (256, 4608), (1024, 2048), (12, 33792),
+                                   (4, 57344)])
+@pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8)])
+@pytest.mark.parametrize("waves", [0, 8, 13])
+def test_gemv_slot_kernel(oracle, dev, gemv_option, kind, shape, level_bits, waves):
+    """The row-block decode with its products on the matrix pipe (16 (row, column block) pairs per instruction),
+    forced for every mix at one to four activation rows, bf16 output and the fp32 accumulate contract: waves with
+    one, several and no groups of their own, a last group with unit-quads past the end, workgroups of 8, 13 and the
+    planner's number of waves, dense mixes that fill the record queue inside every group (and the resolver that
+    reads global memory), 66 column blocks beside the per-wave stages, 112 column blocks (no fit: the next kernel)."""
+    from ixrun_amd import _lib
+
+    out_f, in_f = shape
+    p = make_packed(kind, out_f, in_f, level_bits)
+    dp = device_packed(p, dev)
+    w_bits = oracle.decode_packed_bf16(p)
+    gemv_option("gemv_slots", 1)
+    gemv_option("gemv_slot_waves", waves)
+    gemv_option("gemv_tiles", -1)
+    gemv_option("gemv_strips", -1)
+    for m in (1, 2, 3, 4):
+        x = activations(m, in_f, seed=20 + m)
+        y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
+        for atomic in (False, True):
+            y = run_gemv(dp, 512, x, m, dev, flags=_lib.IXH_GEMV_FORCE_358, atomic=atomic)
+            check_outputs(y, y64, f"slots {kind} {shape} {level_bits} waves={waves} m={m} atomic={atomic}")
+
+
+@pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("shape", [(20, 512), (36, 1024), (68, 5120), (132, 1536), (100, 8704), (48, 17408)])
 @pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8)])
 @pytest.mark.parametrize("tile_rows", [4, 8, 16])
