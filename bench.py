@@ -546,6 +546,8 @@ def main():
                     help="with --unfused: let the library GEMM of the many-row path be chosen by measurement")
     ap.add_argument("--set-option", action="append", default=[], metavar="NAME=VALUE",
                     help="library switch for comparisons (ixh_set_option), e.g. gemv_tiles=-1 or decode_kernel=staged")
+    ap.add_argument("--gemv-flags", type=int, default=0,
+                    help="extra IXH_GEMV_* flags of every fused call, for comparisons (16 = the staged any-scheme kernel)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 256 MiB device copies (known traffic) so that counter runs can be scaled")
     args = ap.parse_args()
@@ -575,6 +577,9 @@ def main():
     if args.tune_gemm:
         from ixrun_amd import gemm_tuning
         gemm_tuning.enable()
+    for sl in layers:
+        sl._gemv_flags = args.gemv_flags
+        sl._plans = {}
     x = x_host.to(dev)
     table_bytes = layers[0]._table.numel() * 4
     # algorithmic bytes of one step: the packed layer, the activations in, the outputs out

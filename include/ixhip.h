@@ -77,34 +77,6 @@ int ixh_version(void);
 const char *ixh_last_error(void);
 
 /*
- * Testing and measurement hook; no counterpart in the reference.  Overrides, for the whole process, a choice the
- * library otherwise makes from the tensor (the defaults are what every other caller gets):
- *   "decode_kernel"  0 = by the tensor (default), 1 = the row-block decoder, 2 = the level-by-level decoder,
- *                    3 = the staged decoder, 4 = the wave-per-unit decoder; a named decoder that cannot take a
- *                    call is skipped for that call
- *   "gemv_shared_x"  most activation rows (0..8, default 8) that ixh_gemv gives to the row-block kernel that
- *                    shares the activations through on-chip memory; 0 = never
- *   "gemv_tiles"     the tile kernel (16, 8 or 4 weight rows x up to 16, 8 or 4 activation rows per matrix
- *                    instruction): -1 = never, 0 = where it pays (three activation rows or more, tiles at least half
- *                    full; default), 1 = wherever it fits
- *   "gemv_tile_rows" the tile kernel's tile shape: 0 = the planner's choice (default), 2 / 3 / 4 = tiles of 4 / 8 / 16
- *                    weight rows only (a shape that cannot serve the call's activation rows hands the call on)
- *   "gemv_tile_split" the number of workgroups of the tile kernel that share a block of rows, each taking a run of its
- *                    column blocks, their sums added by a second launch (needs the workspace of ixh_gemv): 0 = the
- *                    planner's choice (default), 1..8 = that many where the workspace allows
- *   "gemv_tile_cus"  the number of CUs over which the tile kernel's planner spreads the rows: 0 = the device's
- *                    (default), 1..4096 = that many (small tensors then get workgroups with several tiles); also the
- *                    number of workgroups of the dense-mix matrix-pipe kernel
- *   "gemv_dense_tiles" the level-by-level kernels for dense mixes that multiply on the matrix pipe (2..16
- *                    activation rows): -1 = never, 0 = (3,5,8) from four rows on, (3,4,5,6,8) from two (default),
- *                    1 = both from two rows on
- *   "gemv_strips"    the strip kernel (up to eight activation rows a pass): -1 = never, 0 = for three rows or more
- *                    where the tile kernel does not run and the shape fits (default), 1..6 = wherever it fits
- * Returns IXH_EINVAL for an unknown name or a value out of range.  Calls already running are not affected.
- */
-int ixh_set_option(const char *name, int64_t value);
-
-/*
  * Number of int32 entries per level of a prefix table with the given chunk:
  * ceil(n / chunk) + 1.
  */
@@ -180,8 +152,11 @@ size_t ixh_gemv_workspace_bytes(const IxhPacked *packed, int64_t chunk, int32_t 
  * harnesses that forbid hipMalloc); it has no counterpart in the reference.  Same arguments, kernels and results
  * as ixh_gemv without IXH_GEMV_ATOMIC, but the partial sums of the kernels that need a workspace go to a buffer
  * of IXH_NOALLOC_WORKSPACE_BYTES that is part of the library's code object (every GPU the library runs on holds
- * it until the process ends).  The call allocates and frees nothing.  A request whose partial sums need more
- * (ixh_gemv_workspace_bytes) fails with IXH_EWORKSPACE; IXH_GEMV_ATOMIC fails with IXH_EINVAL.  The device that
+ * it until the process ends).  The call allocates and frees nothing.  Where ixh_gemv_workspace_bytes asks for
+ * more than the buffer holds, the kernels that need no workspace (a workgroup owns whole rows) still run, the tile
+ * kernel divides a block of rows among as many workgroups as the buffer has room for (its sums are then added in
+ * another order than ixh_gemv's with a full workspace), and a call that only a kernel with one piece per 512
+ * columns can take fails with IXH_EWORKSPACE before anything is launched; IXH_GEMV_ATOMIC fails with IXH_EINVAL.  The device that
  * is current at the call must be the one the tensors live on; the first call on a device looks the buffer's
  * address up (make that call outside stream capture).  All calls on one GPU share the buffer: calls that may
  * overlap there (two streams, two threads) race on it and must be ordered by the caller.

@@ -1,4 +1,5 @@
-"""ctypes binding of ``libixhip.so`` (the C ABI declared in ``include/ixhip.h``).
+"""ctypes binding of ``libixhip.so`` (the C ABI declared in ``include/ixhip.h``; the testing hook in
+``include/ixhip_test.h``).
 
 The library is built in-tree by ``csrc/build.sh``.  There is no CPU fallback:
 if the shared object is missing, or a call is made without a GPU tensor,
@@ -52,15 +53,14 @@ class IxhError(RuntimeError):
 
 
 _lib = None
-# measurement switch: extra ixh_gemv flags for every call (e.g. 16 = IXH_GEMV_STAGED), to time one kernel
-# against another through the same harness
-_ENV_GEMV_FLAGS = int(os.environ.get("IXH_GEMV_FLAGS", "0"))
 
+# the product interface (include/ixhip.h) and the testing hook (include/ixhip_test.h)
 EXPORTS = (
-    "ixh_version", "ixh_last_error", "ixh_set_option", "ixh_prefix_entries", "ixh_prefix_build", "ixh_decode",
+    "ixh_version", "ixh_last_error", "ixh_prefix_entries", "ixh_prefix_build", "ixh_decode",
     "ixh_gemv", "ixh_gemv_workspace_bytes", "ixh_gemv_noalloc", "ixh_gemm", "ixh_gemm_workspace_bytes",
     "ixh_encode_workspace_bytes", "ixh_encode_scan", "ixh_encode_pack", "ixh_decode_gs",
 )
+TEST_EXPORTS = ("ixh_set_option",)
 
 
 def lib() -> C.CDLL:
@@ -127,8 +127,8 @@ DECODE_KERNELS = {"auto": 0, "rows": 1, "dense": 2, "staged": 3, "generic": 4}
 
 
 def set_option(name: str, value) -> None:
-    """Process-wide testing / measurement switch of the library (``ixh_set_option``); ``decode_kernel`` also takes
-    the decoder's name."""
+    """Process-wide testing / measurement switch of the library (``ixh_set_option``, declared in
+    ``include/ixhip_test.h``, not in the product header); ``decode_kernel`` also takes the decoder's name."""
     if name == "decode_kernel" and isinstance(value, str):
         value = DECODE_KERNELS[value]
     check(lib().ixh_set_option(name.encode(), int(value)))
@@ -233,8 +233,9 @@ class DevicePacked:
     def gemv_workspace_bytes(self, chunk: int, m: int, flags: int = 0) -> int:
         return int(lib().ixh_gemv_workspace_bytes(C.byref(self.struct), int(chunk), int(m), int(flags)))
 
-    def gemv(self, table, chunk, x, y=None, y32=None, workspace=None, flags=0) -> None:
-        """x bf16 [M, in_f] (row stride x.stride(0)); y bf16 [M, out_f] or y32 fp32 (atomic mode)."""
+    def _gemv_operands(self, table, chunk, x, y, y32, workspace):
+        """Check every buffer of a fused call on the host (device, dtype, layout, size): the kernels trust the
+        pointers they are given.  Returns (x as [M, in_f], M, ldx, ldy)."""
         if not x.is_cuda:
             raise RuntimeError(f"x must live on the GPU (got {x.device}); the HIP path has no CPU fallback")
         if x.dtype != torch.bfloat16:
@@ -244,8 +245,39 @@ class DevicePacked:
             raise ValueError("x rows must be contiguous")
         m = x2.shape[0]
         ldx = x2.stride(0) if m > 1 else self.in_f
-        ldy = y.stride(0) if (y is not None and y.dim() == 2 and m > 1) else self.out_f
-        flags = int(flags) | _ENV_GEMV_FLAGS
+        ldy = self.out_f
+        for name, t, dt in (("y", y, torch.bfloat16), ("y32", y32, torch.float32)):
+            if t is None:
+                continue
+            if not t.is_cuda or t.device != self.device:
+                raise RuntimeError(f"{name} must live on {self.device} (got {t.device})")
+            if t.dtype != dt:
+                raise ValueError(f"{name} must be {dt}")
+            if name == "y" and t.dim() == 2 and m > 1:  # rows may be strided (ldy); y32 is always dense [M, out_f]
+                if t.shape[0] < m or t.shape[1] < self.out_f or t.stride(1) != 1 or t.stride(0) < self.out_f:
+                    raise ValueError(f"y must hold {m} contiguous rows of {self.out_f} elements")
+                ldy = t.stride(0)
+            elif not t.is_contiguous() or t.numel() < m * self.out_f:
+                raise ValueError(f"{name} must be contiguous with at least {m * self.out_f} elements")
+        entries = self.prefix_entries(chunk)
+        if entries < 1:
+            raise ValueError(f"chunk {chunk} must be positive")
+        if not table.is_cuda or table.device != self.device:
+            raise RuntimeError(f"the rank table must live on {self.device} (got {table.device})")
+        if (table.dtype != torch.int32 or table.dim() != 2 or table.shape[0] < len(self.level_bits) - 1
+                or table.shape[1] != entries or table.stride(1) != 1 or table.stride(0) != entries):
+            raise ValueError(f"the rank table must be contiguous int32 [{len(self.level_bits) - 1}, {entries}] "
+                             f"for chunk {chunk}")
+        if workspace is not None:
+            if not workspace.is_cuda or workspace.device != self.device:
+                raise RuntimeError(f"the workspace must live on {self.device} (got {workspace.device})")
+            if not workspace.is_contiguous():
+                raise ValueError("the workspace must be contiguous")
+        return x2, m, ldx, ldy
+
+    def gemv(self, table, chunk, x, y=None, y32=None, workspace=None, flags=0) -> None:
+        """x bf16 [M, in_f] (row stride x.stride(0)); y bf16 [M, out_f] or y32 fp32 (atomic mode)."""
+        x2, m, ldx, ldy = self._gemv_operands(table, chunk, x, y, y32, workspace)
         check(lib().ixh_gemv(
             C.byref(self.struct), table.data_ptr(), int(chunk), x2.data_ptr(), m, ldx,
             y.data_ptr() if y is not None else None, ldy,
@@ -256,17 +288,11 @@ class DevicePacked:
 
     def gemv_noalloc(self, table, chunk, x, y, flags=0) -> None:
         """``gemv`` through the entry point that allocates nothing: partial sums go to the library's own buffer
-        (``IXH_NOALLOC_WORKSPACE_BYTES``); larger requests raise ``IxhError(IXH_EWORKSPACE)``."""
-        if not x.is_cuda:
-            raise RuntimeError(f"x must live on the GPU (got {x.device}); the HIP path has no CPU fallback")
-        if x.dtype != torch.bfloat16:
-            raise ValueError("x must be bf16")
-        x2 = x.reshape(-1, self.in_f)
-        if x2.stride(1) != 1:
-            raise ValueError("x rows must be contiguous")
-        m = x2.shape[0]
-        ldx = x2.stride(0) if m > 1 else self.in_f
-        ldy = y.stride(0) if (y.dim() == 2 and m > 1) else self.out_f
+        (``IXH_NOALLOC_WORKSPACE_BYTES``); requests whose kernel cannot fit its partial sums there raise
+        ``IxhError(IXH_EWORKSPACE)``."""
+        if y is None:
+            raise ValueError("gemv_noalloc needs the bf16 output y")
+        x2, m, ldx, ldy = self._gemv_operands(table, chunk, x, y, None, None)
         with torch.cuda.device(self.device):
             check(lib().ixh_gemv_noalloc(
                 C.byref(self.struct), table.data_ptr(), int(chunk), x2.data_ptr(), m, ldx, y.data_ptr(), ldy,

@@ -1,5 +1,5 @@
 // C boundary of the library: argument checks, kernel selection, error text.
-// Declarations and the reference interfaces they replace: include/ixhip.h.
+// Declarations and the reference interfaces they replace: include/ixhip.h; the testing hook: include/ixhip_test.h.
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -7,6 +7,7 @@
 #include <cstdlib>
 #include <mutex>
 
+#include "../../include/ixhip_test.h"
 #include "ixh_dev.h"
 #include "ixh_fast358.h"
 
@@ -234,9 +235,32 @@ size_t ixh_gemv_workspace_bytes(const IxhPacked *packed, int64_t chunk, int32_t 
     return n_chunks * (size_t)m * d.out_f * sizeof(float);
 }
 
+// Which of the kernel families for tensors that are almost all level 1 may take a call.
+struct Level1Family {
+    bool mostly_l1, fast, fast_any;
+};
+static Level1Family level1_family(const Dev &d, int64_t chunk, int32_t m, uint32_t flags) {
+    Level1Family f;
+    // The (3,5,8) kernels are built for tensors that are almost all level 1 (every other element costs
+    // them a queue record); denser mixes go to the general kernel unless the caller insists.
+    f.mostly_l1 = (uint64_t)d.st_words[0] * 32u / 3u >= (uint64_t)d.n / 100u * 97u;
+    f.fast = !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED | IXH_GEMV_DENSE)) && is_358(d) &&
+             fast358_supports(d, (uint32_t)chunk, m) &&
+             (f.mostly_l1 || (flags & (IXH_GEMV_COLUMN_KERNEL | IXH_GEMV_FORCE_358)));
+    // any other scheme whose first level has 3 bits, almost all level 1: the row-block kernel with the resolver that
+    // walks the nested bitmaps (the column-block kernel is (3,5,8) only, so 5..8 rows go on to the any-scheme kernel)
+    f.fast_any = !f.fast && !is_358(d) && d.n_levels >= 2 && d.bits[0] == 3 &&
+                 !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED | IXH_GEMV_DENSE | IXH_GEMV_COLUMN_KERNEL)) &&
+                 fast358_supports(d, (uint32_t)chunk, m) && (f.mostly_l1 || (flags & IXH_GEMV_FORCE_358));
+    return f;
+}
+
+// partial_ws: the workspace may be smaller than ixh_gemv_workspace_bytes says (the built-in buffer of
+// ixh_gemv_noalloc): kernels whose workgroups share a block of rows then share it among as many pieces as it holds,
+// kernels that need no workspace run as ever, and only a call whose kernel needs all of it fails.
 static int gemv_any(const IxhPacked *packed, const int32_t *prefix, int64_t chunk, const uint16_t *x, int32_t m,
                     int64_t ldx, uint16_t *y, int64_t ldy, float *y32, void *workspace, size_t workspace_bytes,
-                    uint32_t flags, ixh_stream_t stream) {
+                    uint32_t flags, ixh_stream_t stream, bool partial_ws = false) {
     Dev d;
     int rc = to_dev(packed, &d);
     if (rc) return rc;
@@ -253,29 +277,28 @@ static int gemv_any(const IxhPacked *packed, const int32_t *prefix, int64_t chun
     if (!prefix || !x) { set_error("prefix or x is NULL"); return IXH_EINVAL; }
     if (ldx < (int64_t)d.in_f && m > 1) { set_error("ldx %lld < in_f %u", (long long)ldx, d.in_f); return IXH_EINVAL; }
     const bool atomic = (flags & IXH_GEMV_ATOMIC) != 0;
+    size_t need = 0;
+    bool ws_full = true;
+    uint32_t ws_pieces = 0;
     if (atomic) {
         if (!y32) { set_error("IXH_GEMV_ATOMIC needs y32"); return IXH_EINVAL; }
     } else {
         if (!y) { set_error("y is NULL"); return IXH_EINVAL; }
         if (ldy < (int64_t)d.out_f && m > 1) { set_error("ldy %lld < out_f %u", (long long)ldy, d.out_f); return IXH_EINVAL; }
-        const size_t need = ixh_gemv_workspace_bytes(packed, chunk, m, flags);
-        if (need && (!workspace || workspace_bytes < need)) {
+        need = ixh_gemv_workspace_bytes(packed, chunk, m, flags);
+        ws_full = !need || (workspace && workspace_bytes >= need);
+        if (!ws_full && !partial_ws) {
             set_error("workspace of %zu bytes needed, %zu given", need, workspace ? workspace_bytes : (size_t)0);
             return IXH_EWORKSPACE;
         }
+        if (workspace) {  // pieces of m x out_f partial sums that the workspace holds
+            const size_t piece = (size_t)m * d.out_f * sizeof(float), n_chunks = d.in_f / (uint32_t)chunk;
+            ws_pieces = (uint32_t)(workspace_bytes / piece < n_chunks ? workspace_bytes / piece : n_chunks);
+        }
     }
     rc = IXH_EUNSUPPORTED;
-    // The (3,5,8) kernels are built for tensors that are almost all level 1 (every other element costs
-    // them a queue record); denser mixes go to the general kernel unless the caller insists.
-    const bool mostly_l1 = (uint64_t)d.st_words[0] * 32u / 3u >= (uint64_t)d.n / 100u * 97u;
-    const bool fast = !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED | IXH_GEMV_DENSE)) && is_358(d) &&
-                      fast358_supports(d, (uint32_t)chunk, m) &&
-                      (mostly_l1 || (flags & (IXH_GEMV_COLUMN_KERNEL | IXH_GEMV_FORCE_358)));
-    // any other scheme whose first level has 3 bits, almost all level 1: the row-block kernel with the resolver that
-    // walks the nested bitmaps (the column-block kernel is (3,5,8) only, so 5..8 rows go on to the any-scheme kernel)
-    const bool fast_any = !fast && !is_358(d) && d.n_levels >= 2 && d.bits[0] == 3 &&
-                          !(flags & (IXH_GEMV_FORCE_GENERIC | IXH_GEMV_STAGED | IXH_GEMV_DENSE | IXH_GEMV_COLUMN_KERNEL)) &&
-                          fast358_supports(d, (uint32_t)chunk, m) && (mostly_l1 || (flags & IXH_GEMV_FORCE_358));
+    const Level1Family fam = level1_family(d, chunk, m, flags);
+    const bool mostly_l1 = fam.mostly_l1, fast = fam.fast, fast_any = fam.fast_any;
     if ((fast || fast_any) && !(flags & IXH_GEMV_COLUMN_KERNEL)) {
         // The row-block kernels: a workgroup owns whole rows, so the split-K contract (add into the caller's fp32
         // vector) costs them one addition per output.  First the strip kernel (products on the matrix pipe, up to 16
@@ -285,8 +308,8 @@ static int gemv_any(const IxhPacked *packed, const int32_t *prefix, int64_t chun
         uint16_t *const yb = atomic ? nullptr : y;
         float *const yf = atomic ? y32 : nullptr;
         // (the workspace holds in_f / chunk pieces of m x out_f sums)
-        rc = launch_gemv_358_tiles(d, prefix, x, m, ldx, yb, ldy, yf, atomic ? nullptr : (float *)workspace,
-                                   workspace && !atomic ? (uint32_t)(d.in_f / (uint32_t)chunk) : 0u, (hipStream_t)stream);
+        rc = launch_gemv_358_tiles(d, prefix, x, m, ldx, yb, ldy, yf, atomic || !ws_pieces ? nullptr : (float *)workspace,
+                                   ws_pieces, (hipStream_t)stream);
         if (rc == IXH_EUNSUPPORTED) rc = launch_gemv_358_strips(d, prefix, x, m, ldx, yb, ldy, yf, (hipStream_t)stream);
         if (rc == IXH_EUNSUPPORTED && m <= 8)
             rc = launch_gemv_358_rows(d, prefix, x, m, ldx, yb, ldy, yf, (hipStream_t)stream);
@@ -303,6 +326,11 @@ static int gemv_any(const IxhPacked *packed, const int32_t *prefix, int64_t chun
                 }
             }
         }
+    }
+    if (rc == IXH_EUNSUPPORTED && !ws_full) {  // every kernel from here on keeps one piece per chunk of a row
+        set_error("gemv_noalloc: the kernel for this call needs %zu bytes of partial sums, the built-in buffer holds "
+                  "%zu; call ixh_gemv with a workspace of your own", need, workspace_bytes);
+        return IXH_EWORKSPACE;
     }
     if (fast && rc == IXH_EUNSUPPORTED)
         rc = launch_gemv_358(d, prefix, (uint32_t)chunk, x, m, ldx, y, ldy, y32, (float *)workspace, atomic,
@@ -386,18 +414,26 @@ int ixh_gemv_noalloc(const IxhPacked *packed, const int32_t *prefix, int64_t chu
         set_error("gemv_noalloc: IXH_GEMV_ATOMIC takes no workspace; call ixh_gemv");
         return IXH_EINVAL;
     }
-    const size_t need = ixh_gemv_workspace_bytes(packed, chunk, m, flags);  // 0 also for arguments gemv_any rejects
-    if (need > (size_t)IXH_NOALLOC_WORKSPACE_BYTES) {
-        set_error("gemv_noalloc: this call needs %zu bytes of partial sums, the built-in buffer holds %zu; "
-                  "call ixh_gemv with a workspace of your own", need, (size_t)IXH_NOALLOC_WORKSPACE_BYTES);
-        return IXH_EWORKSPACE;
+    Dev d;
+    if (to_dev(packed, &d) == IXH_OK && d.n != 0 && gemv_checks(d, chunk, m) == IXH_OK) {
+        // only the row-block kernels (no workspace, or as many pieces as there is room for) can take a call whose
+        // full set of partial sums is larger than the buffer
+        const size_t need = ixh_gemv_workspace_bytes(packed, chunk, m, flags);
+        const Level1Family fam = level1_family(d, chunk, m, flags);
+        if (need > (size_t)IXH_NOALLOC_WORKSPACE_BYTES && (!(fam.fast || fam.fast_any) || (flags & IXH_GEMV_COLUMN_KERNEL))) {
+            set_error("gemv_noalloc: the kernel for this call needs %zu bytes of partial sums, the built-in buffer "
+                      "holds %zu; call ixh_gemv with a workspace of your own", need, (size_t)IXH_NOALLOC_WORKSPACE_BYTES);
+            return IXH_EWORKSPACE;
+        }
     }
     void *ws = nullptr;
     const int rc = scratch_of_current_device(&ws);
     if (rc) return rc;
     // every partial sum the second kernel reads was written by the first in the same call: nothing to clear
+    // (a call whose kernel needs more partial sums than the buffer holds fails inside with IXH_EWORKSPACE, before
+    // any launch; the row-block kernels need none, the tile kernel shares the buffer among the pieces it holds)
     return gemv_any(packed, prefix, chunk, x, m, ldx, y, ldy, nullptr, ws, (size_t)IXH_NOALLOC_WORKSPACE_BYTES, flags,
-                    stream);
+                    stream, true);
 }
 
 size_t ixh_gemm_workspace_bytes(const IxhPacked *packed, int32_t m) {

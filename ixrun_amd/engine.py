@@ -21,11 +21,17 @@ import torch.nn.functional as F
 
 from . import _lib, gemm_tuning
 from .config import TRITON_BLOCK
-from .fused import FUSED_TILE, _pick_split, pick_unit, shared_workspace
+from .fused import FUSED_TILE, _pick_split, _workspaces, pick_unit, shared_workspace
 from .linear import _set_parent_child, iter_quantizable_linears
 from .quantize import int8x_quantize, portable_packed, quantize_for_deploy
 
 __all__ = ["Int8XEngine", "StreamingLinear", "GraphLinear", "ResourceScheduler"]
+
+try:  # the current stream's handle without building a Stream object (1 us less per forward)
+    _raw_stream = torch._C._cuda_getCurrentRawStream
+except AttributeError:  # pragma: no cover
+    def _raw_stream(index):
+        return torch.cuda.current_stream(index).cuda_stream
 
 MAX_FUSED_ROWS = 16  # activation rows served by the fused decode+GEMV kernel
 # With a decode buffer at hand, more rows than this go through decode + library GEMM.  Tensors that are almost all
@@ -77,6 +83,7 @@ class StreamingLinear(nn.Module):
         for i in range(n_levels):
             self.register_buffer(f"_l{i + 1}", packed["streams"][i].cuda())
         self.register_buffer("_scale", packed["scale"].reshape(()).cuda())
+        self._gemv_flags = 0  # extra IXH_GEMV_* flags of every fused call (comparisons: bench.py --gemv-flags)
         self._bind()
 
         # rank tables: the kernels' own (unit = 512 where rows allow it) and
@@ -84,6 +91,7 @@ class StreamingLinear(nn.Module):
         self._unit = pick_unit(self.in_features)
         ready = packed.get("table512") if self._unit == 512 else None  # left by the device encoder
         self.register_buffer("_table", ready.cuda() if ready is not None else self._dp.prefix_build(self._unit))
+        self._table_ptr = self._table.data_ptr()
         if self.N % TRITON_BLOCK == 0 and TRITON_BLOCK % self._unit == 0:
             blk_table = self._table[:, :: TRITON_BLOCK // self._unit][:, : self.N // TRITON_BLOCK]
         else:
@@ -123,6 +131,12 @@ class StreamingLinear(nn.Module):
             [getattr(self, f"_l{i + 1}") for i in range(n_levels)],
             self._scale.reshape(1),
         )
+        # what every fused call passes unchanged (the table follows the module when it moves: see _apply)
+        import ctypes
+        self._gemv_fn = _lib.lib().ixh_gemv
+        self._struct_ref = ctypes.byref(self._dp.struct)
+        self._table_ptr = self._table.data_ptr() if hasattr(self, "_table") else None
+        self._plans = {}
 
     def _apply(self, fn, recurse=True):
         # .to()/.cuda() may move the buffers: point the kernel arguments at the new storage
@@ -133,6 +147,7 @@ class StreamingLinear(nn.Module):
 
     def _set_shared_buf(self, w_buf):
         self._w_buf = w_buf
+        self._plans = {}
 
     def _decode(self):
         """Decode into the shared buffer and return it as ``[out_f, in_f]``
@@ -141,8 +156,11 @@ class StreamingLinear(nn.Module):
         self._dp.decode(self._table, self._unit, out_bf16=w_flat)
         return w_flat.view(self.out_features, self.in_features)
 
-    def forward(self, x):
-        rows = x.numel() // self.in_features if self.in_features else 0
+    def _fused_plan(self, rows):
+        """How a forward of `rows` activation rows is served by the fused kernel: the row count of each call (one, or
+        two for 17 .. 32 rows on a large layer that is almost all level 1) with the scratch it needs, or False where
+        the many-row paths take over.  Worked out once per row count; ``_set_shared_buf`` and ``_bind`` forget the
+        answers."""
         if self._w_buf is None:
             fused_rows = MAX_FUSED_ROWS
         elif self.counts[0] * 100 >= self.N * 97:
@@ -153,20 +171,45 @@ class StreamingLinear(nn.Module):
             fused_rows = 1
         two_calls = (MAX_FUSED_ROWS < rows <= 2 * MAX_FUSED_ROWS and fused_rows == MAX_FUSED_ROWS
                      and self.N >= SPLIT_FUSED_MIN_WEIGHTS and self.counts[0] * 100 >= self.N * 97)
-        if (self._use_fused and x.dtype == torch.bfloat16 and x.is_cuda and (1 <= rows <= fused_rows or two_calls)
-                and x.shape[-1] == self.in_features):
-            x2 = x.reshape(rows, self.in_features)
-            if x2.stride(1) != 1:
-                x2 = x2.contiguous()
-            y = torch.empty((rows, self.out_features), dtype=torch.bfloat16, device=x.device)
-            for r0 in range(0, rows, MAX_FUSED_ROWS):  # one call, or two on the same stream and workspace
+        plan = False
+        if 1 <= rows <= fused_rows or two_calls:
+            calls = []
+            for r0 in range(0, rows, MAX_FUSED_ROWS):
                 n = min(MAX_FUSED_ROWS, rows - r0)
-                ws = shared_workspace(x.device, self._dp.gemv_workspace_bytes(self._unit, n))
-                self._dp.gemv(self._table, self._unit, x2[r0:r0 + n], y=y[r0:r0 + n], workspace=ws)
-            y = y.view(x.shape[:-1] + (self.out_features,))
-            if self._bias is not None:
-                y = y + self._bias.to(y.dtype)
-            return y
+                calls.append((r0, n, self._dp.gemv_workspace_bytes(self._unit, n, self._gemv_flags)))
+            plan = tuple(calls)
+        self._plans[rows] = plan
+        return plan
+
+    def forward(self, x):
+        in_f = self.in_features
+        if self._use_fused and x.dtype is torch.bfloat16 and x.is_cuda and in_f and x.shape[-1] == in_f:
+            rows = x.numel() // in_f
+            plan = self._plans.get(rows)
+            if plan is None:
+                plan = self._fused_plan(rows)
+            if plan:
+                # the hot path of token generation: one ctypes call with the arguments that never change kept bound
+                out_f = self.out_features
+                if not x.is_contiguous():
+                    x = x.contiguous()
+                dev = x.device
+                y = torch.empty(x.shape[:-1] + (out_f,), dtype=torch.bfloat16, device=dev)
+                x_ptr, y_ptr = x.data_ptr(), y.data_ptr()
+                stream = _raw_stream(dev.index if dev.index is not None else torch.cuda.current_device())
+                for r0, n, ws_bytes in plan:  # one call, or two on the same stream and workspace
+                    ws = _workspaces.get(dev) if ws_bytes else None
+                    if ws_bytes and (ws is None or ws.numel() * 4 < ws_bytes):
+                        ws = shared_workspace(dev, ws_bytes)
+                    rc = self._gemv_fn(self._struct_ref, self._table_ptr, self._unit, x_ptr + r0 * in_f * 2, n, in_f,
+                                       y_ptr + r0 * out_f * 2, out_f, None, ws.data_ptr() if ws_bytes else None,
+                                       ws_bytes, self._gemv_flags, stream)
+                    if rc:
+                        _lib.check(rc)
+                if self._bias is not None:
+                    y = y + self._bias.to(y.dtype)
+                return y
+        rows = x.numel() // in_f if in_f else 0
         if (self._use_fused and self._gemm_ok and x.dtype == torch.bfloat16 and x.is_cuda and rows > MAX_FUSED_ROWS
                 and x.shape[-1] == self.in_features and self._unit == 512 and self._w_buf is None):
             # many rows: decode tiles on chip straight into the matrix-core GEMM, no bf16 weight in HBM

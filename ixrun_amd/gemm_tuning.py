@@ -10,7 +10,7 @@ this module switches that on for exactly the shapes the layers meet, one shape a
 and leaves tuning off otherwise, so that unrelated GEMMs of the host program are never
 held up.
 
-Off by default: ``enable()`` or ``IXRUN_TUNE_GEMM=1`` turns it on.  The first call of a
+Off by default: ``enable()`` turns it on (nothing is read from the environment).  The first call of a
 new (rows, out_f, in_f, dtype, bias) signature then takes up to ``max_ms`` longer.  Nothing
 is tuned while a graph is being captured: run one eager forward of each shape first.
 """
@@ -21,20 +21,19 @@ import os
 import torch
 import torch.nn.functional as F
 
-_state = {"on": None, "max_ms": 300, "seen": set()}
+_state = {"on": False, "max_ms": 300, "seen": set()}
 
 
 def enable(max_ms: int = 300, results_file: str | None = None) -> None:
     """Use tuned library GEMMs in ``linear`` from now on (per process).
 
-    torch keeps the winners in a csv file; ``results_file`` (or ``IXRUN_TUNE_GEMM_FILE``) names one to
+    torch keeps the winners in a csv file; ``results_file`` names one to
     read now and extend, so that a later process starts with them; without it the file is
     a per-process one in the temporary directory."""
     import tempfile
 
     import torch.cuda.tunable as tunable
 
-    results_file = results_file or os.environ.get("IXRUN_TUNE_GEMM_FILE")
     tunable.enable(True)
     tunable.tuning_enable(False)
     if results_file:
@@ -56,11 +55,6 @@ def disable() -> None:
 
 
 def enabled() -> bool:
-    if _state["on"] is None:  # first question: the environment decides
-        if os.environ.get("IXRUN_TUNE_GEMM", "0") not in ("", "0"):
-            enable()
-        else:
-            _state["on"] = False
     return bool(_state["on"])
 
 

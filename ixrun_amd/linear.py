@@ -51,7 +51,6 @@ class Int8XLinear(nn.Module):
         self.packed = packed
         self.use_triton = use_triton
         self._cache = cache
-        self._bias = None
         if bias is not None:
             self.register_buffer("_bias_buf", bias.detach().clone())
         else:

@@ -13,8 +13,8 @@ from ixrun_amd import _lib
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "ixhip.h")).read()
+def declared_symbols(header="ixhip.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(ixh_[a-z0-9_]+)\s*\(", text)))
 
@@ -27,6 +27,23 @@ def test_header_symbols_are_exported():
         assert hasattr(lib, name), f"{name} is declared in include/ixhip.h but not exported"
     assert set(_lib.EXPORTS) == set(names)
     assert lib.ixh_version() >= 100
+
+
+def test_option_setter_is_not_in_the_product_header():
+    """The process-wide kernel-selection switches are a testing hook: the product header declares no setter (nor
+    mentions one), the test header declares exactly that one symbol, and the binding reads nothing from the
+    environment but the library's path."""
+    public = open(os.path.join(ROOT, "include", "ixhip.h")).read()
+    assert "set_option" not in public and "option" not in " ".join(declared_symbols())
+    assert declared_symbols("ixhip_test.h") == ["ixh_set_option"] == list(_lib.TEST_EXPORTS)
+    assert hasattr(_lib.lib(), "ixh_set_option")
+    pkg = os.path.join(ROOT, "ixrun_amd")
+    reads = []
+    for name in sorted(os.listdir(pkg)):
+        if name.endswith(".py"):
+            text = open(os.path.join(pkg, name)).read()
+            reads += [(name, var) for var in re.findall(r"environ(?:\.get)?[\[(]\s*\"([A-Z_0-9]+)\"", text)]
+    assert reads == [("_lib.py", "IXH_LIB")], reads
 
 
 def _packed(level_bits=(3, 5, 8), out_f=4, in_f=8, bm0_words=1):

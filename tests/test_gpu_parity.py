@@ -234,6 +234,62 @@ def test_decode_config1_2048(oracle, dev):
 
 
 # ---------------------------------------------------------------- fused decode + GEMV
+def test_gemv_config1_2048(oracle, dev):
+    """BASELINE config 1 through the fused path: ixh_gemv on the 2048 x 2048 Student-t tensor, one activation row,
+    against the fp64 oracle; once with the kernel the library picks for this mix, once with the (3,5,8) row-block
+    kernels forced (IXH_GEMV_FORCE_358), bf16 output and the fp32 atomic mode."""
+    from ixrun_amd import _lib
+
+    p = quantize(student_t_weight(2048, 2048, seed=0))
+    dp = device_packed(p, dev)
+    w_bits = oracle.decode_packed_bf16(p)
+    x = activations(1, 2048, seed=0)
+    y64 = oracle.gemm_f64(w_bits, bf16_bits(x))
+    for flags in (0, _lib.IXH_GEMV_FORCE_358):
+        for atomic in (False, True):
+            y = run_gemv(dp, 512, x, 1, dev, flags=flags, atomic=atomic)
+            check_outputs(y, y64, f"config 1 flags={flags} atomic={atomic}")
+
+
+def test_gemv_binding_rejects_bad_buffers(dev):
+    """The Python binding checks every buffer of a fused call before the library sees a pointer: outputs on the host,
+    of the wrong type, too small or strided, a rank table for another chunk, a workspace on the host."""
+    p = quantize(outlier_weight(8, 1024, seed=1))
+    dp = device_packed(p, dev)
+    table = dp.prefix_build(512)
+    x = activations(2, 1024, seed=1).to(dev)
+    ok = torch.zeros((2, 8), dtype=torch.bfloat16, device=dev)
+    ws = torch.empty(dp.gemv_workspace_bytes(512, 2) // 4, dtype=torch.float32, device=dev)
+    dp.gemv(table, 512, x, y=ok, workspace=ws)
+    wide = torch.zeros((2, 16), dtype=torch.bfloat16, device=dev)
+    dp.gemv(table, 512, x, y=wide[:, :8], workspace=ws)  # rows 16 elements apart: ldy
+    torch.cuda.synchronize()
+    assert torch.equal(wide[:, :8], ok) and torch.all(wide[:, 8:] == 0)
+    bad = [
+        dict(y=ok.cpu()), dict(y=ok.float()), dict(y=ok[:1]), dict(y=torch.zeros((2, 4), dtype=torch.bfloat16, device=dev)),
+        dict(y=wide.t()[:8].t()[:, ::2]), dict(y=None, y32=torch.zeros((2, 8), dtype=torch.bfloat16, device=dev)),
+        dict(y=None, y32=torch.zeros(15, dtype=torch.float32, device=dev)),
+        dict(y=ok, table=dp.prefix_build(256)), dict(y=ok, table=table.cpu()), dict(y=ok, table=table.long()),
+        dict(y=ok, workspace=ws.cpu()), dict(y=ok, workspace=torch.empty((4, 64), device=dev)[:, ::2]),
+    ]
+    for kw in bad:
+        args = dict(table=table, y32=None, workspace=ws)
+        args.update(kw)
+        with pytest.raises((ValueError, RuntimeError)) as e:
+            dp.gemv(args["table"], 512, x, y=args["y"], y32=args["y32"], workspace=args["workspace"])
+        assert not isinstance(e.value, _lib_error())
+    with pytest.raises((ValueError, RuntimeError)):
+        dp.gemv_noalloc(table, 512, x, ok.float())
+    with pytest.raises(ValueError):
+        dp.gemv_noalloc(table, 512, x, None)
+
+
+def _lib_error():
+    from ixrun_amd import _lib
+
+    return _lib.IxhError
+
+
 def run_gemv(dp, chunk, x, m, dev, flags=0, atomic=False):
     from ixrun_amd import _lib
 
@@ -420,7 +476,7 @@ def test_gemv_tile_shapes(oracle, dev, gemv_option, kind, shape, level_bits, til
 
 
 @pytest.mark.parametrize("kind", KINDS)
-@pytest.mark.parametrize("shape", [(20, 1024), (68, 5120), (132, 1536), (100, 8704), (48, 17408)])
+@pytest.mark.parametrize("shape", [(20, 1024), (68, 5120), (132, 1536), (100, 8704), (48, 17408), (132, 512)])
 @pytest.mark.parametrize("level_bits", [(3, 5, 8), (3, 4, 5, 6, 8)])
 @pytest.mark.parametrize("split", [2, 3, 4, 7])
 def test_gemv_tile_split(oracle, dev, gemv_option, kind, shape, level_bits, split):
@@ -428,8 +484,10 @@ def test_gemv_tile_split(oracle, dev, gemv_option, kind, shape, level_bits, spli
     pieces go through the workspace (filled with NaN before the call: every piece must be written) and a second launch
     that adds them, or one by one into the caller's fp32 sums; row blocks several times as tall, pieces of unequal
     length, pieces held in LDS in several parts, a split that would leave a piece empty (the call then goes on to the
-    next kernel), a workspace too small for pieces (chunk = in_f: no workspace, whole rows per workgroup); the same call
-    twice gives the same bits."""
+    next kernel), no workspace at all (in_f = 512: a row is one column block, ixh_gemv_workspace_bytes is 0, and the tile
+    kernel runs with whole rows per workgroup whatever split is asked for); the same call twice gives the same bits.
+    The last call, with chunk = in_f, is served by the wave-per-unit kernel for every in_f but 512 (the other kernels
+    take chunk = 512 only) and checks that the options leave it alone."""
     from ixrun_amd import _lib
 
     out_f, in_f = shape

@@ -1,7 +1,8 @@
 """The entry point that allocates nothing (ixh_gemv_noalloc) against ixh_gemv, through the C ABI.
 
 Both run the same kernels; the only difference is where the partial sums of the kernels that need a workspace
-live (the library's built-in buffer instead of a caller's tensor), so the outputs must be equal bit for bit.  Each
+live (the library's built-in buffer instead of a caller's tensor), so the outputs must be equal bit for bit.  The
+calls must not change the device's free memory and must replay correctly from a hipGraph.  Each
 case calls twice in a row, the second time with a smaller tensor, so that what the first call left in the shared
 buffer would show.
 """
@@ -108,5 +109,91 @@ def test_noalloc_rejects_what_does_not_fit(dev):
     with pytest.raises(_lib.IxhError) as e:
         dp.gemv_noalloc(table, 1, x, y, flags=_lib.IXH_GEMV_ATOMIC)
     assert e.value.code == -1
+    torch.cuda.synchronize()
+    assert torch.all(y == 7.0)  # nothing ran
+
+
+def test_noalloc_allocates_nothing_and_replays_in_a_graph(dev):
+    """The device's free memory does not move over a run of calls (outputs allocated beforehand; the first call on a
+    device, which looks the buffer's address up, is made before the measurement), and a call captured into a
+    hipGraph replays correctly: three replays with new activations each time, eager work and a synchronisation
+    between them, every replay equal to the eager ixh_gemv result."""
+    from ixrun_amd import _lib
+
+    cases = []
+    for recipe, out_f, in_f, m, flags in (("student_t", 640, 4608, 1, 0), ("student_t", 640, 4608, 16, 0),
+                                          ("outlier", 96, 1536, 3, _lib.IXH_GEMV_STAGED),
+                                          ("calibrated", 640, 4608, 2, _lib.IXH_GEMV_COLUMN_KERNEL)):
+        dp, table = _layer(recipe, out_f, in_f, dev)
+        x = activations(m, in_f, seed=11 + m).to(dev)
+        y = torch.empty((m, out_f), dtype=torch.bfloat16, device=dev)
+        cases.append((dp, table, x, y, flags))
+    for dp, table, x, y, flags in cases:  # warm: code object loaded, buffer address known, plans cached
+        dp.gemv_noalloc(table, 512, x, y, flags=flags)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info(dev)
+    for _ in range(20):
+        for dp, table, x, y, flags in cases:
+            dp.gemv_noalloc(table, 512, x, y, flags=flags)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info(dev)
+    assert free_after == free_before
+
+    for dp, table, x, y, flags in cases:
+        m = x.shape[0]
+        need = dp.gemv_workspace_bytes(512, m, flags)
+        ws = torch.empty(max(need // 4, 1), dtype=torch.float32, device=dev)
+        y_ref = torch.empty_like(y)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            dp.gemv_noalloc(table, 512, x, y, flags=flags)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            dp.gemv_noalloc(table, 512, x, y, flags=flags)
+        for replay in range(3):
+            x.copy_(activations(m, dp.in_f, seed=100 + replay).to(dev))
+            y.fill_(7.0)
+            dp.gemv(table, 512, x, y=y_ref, workspace=ws, flags=flags)  # eager work between the replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert np.array_equal(bf16_bits(y), bf16_bits(y_ref)), (dp.out_f, m, flags, replay)
+
+
+def test_noalloc_takes_a_large_layer_whose_kernels_fit(dev):
+    """A layer whose full set of partial sums (one piece per 512 columns) is larger than the built-in buffer: the
+    row-block kernels need none of it and the tile kernel divides a block of rows among at most eight workgroups, so
+    the call runs and equals ixh_gemv with a full workspace; only the kernels with one piece per 512 columns are
+    refused.  Weights made and encoded on the device (normal with a few large elements: 99 % level 1)."""
+    from ixrun_amd import _lib
+
+    out_f, in_f = 8320, 16384
+    g = torch.Generator(device=dev).manual_seed(5)
+    w = (torch.randn((out_f, in_f), generator=g, device=dev) * 0.008).bfloat16()
+    w[::97, ::89] = 1.0
+    dp, table, counts = _lib.encode_device(w, (3, 5, 8))
+    del w
+    assert counts[0] * 100 >= dp.N * 97
+    for m in (1, 16):
+        need = dp.gemv_workspace_bytes(512, m)
+        x = activations(m, in_f, seed=21 + m).to(dev)
+        ws = torch.empty(need // 4, dtype=torch.float32, device=dev)
+        y_ref = torch.zeros((m, out_f), dtype=torch.bfloat16, device=dev)
+        dp.gemv(table, 512, x, y=y_ref, workspace=ws)
+        y_new = torch.full((m, out_f), 7.0, dtype=torch.bfloat16, device=dev)
+        if m == 16:
+            assert need > LIMIT
+        dp.gemv_noalloc(table, 512, x, y_new)
+        torch.cuda.synchronize()
+        assert np.array_equal(bf16_bits(y_ref), bf16_bits(y_new)), m
+    x = activations(16, in_f, seed=3).to(dev)
+    y = torch.full((16, out_f), 7.0, dtype=torch.bfloat16, device=dev)
+    for flags in (_lib.IXH_GEMV_STAGED, _lib.IXH_GEMV_COLUMN_KERNEL):
+        with pytest.raises(_lib.IxhError) as e:
+            dp.gemv_noalloc(table, 512, x, y, flags=flags)
+        assert e.value.code == -4 and "built-in buffer" in str(e.value)
     torch.cuda.synchronize()
     assert torch.all(y == 7.0)  # nothing ran
