@@ -471,30 +471,38 @@ __host__ __device__ inline RowsXLds rowsx_layout(uint32_t rows_cap, uint32_t n_c
 // unit-quad are 128 registers per lane.
 template <int MT, bool ANY>
 __global__ void __launch_bounds__((MT > 4 ? kXMaxWaves / 2 : kXMaxWaves) * kWave)
-k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, uint32_t quads_per_wg, uint32_t flags,
-                const uint16_t *__restrict__ x, int m, int64_t ldx, uint16_t *__restrict__ y, int64_t ldy,
-               float *__restrict__ y32) {
+k_gemv358_rowsx(const int32_t *__restrict__ prefix, const uint16_t *__restrict__ x, const uint16_t *__restrict__ scale_ptr,
+                int64_t ldx, const uint32_t *__restrict__ bm0, const uint32_t *__restrict__ st0, uint32_t out_f, uint32_t geometry,
+                Dev P, uint16_t *__restrict__ y, int64_t ldy, float *__restrict__ y32) {
+    // The arguments before P are what the first requests to memory need.  They fill the 14 argument registers that
+    // the hardware loads before a wave starts (the file is compiled with that many preloaded), so those requests do
+    // not wait for a read of the argument block: scale_ptr, bm0, st0 and out_f repeat fields of P for that reason,
+    // and the launch geometry (the workgroup size included, which the compiler would read from the block) is
+    // packed into one word (column blocks, row quads per workgroup, waves, activation rows, flags).
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t n_chunks = geometry & 0xFFFu, quads_per_wg = (geometry >> 12) & 0xFFu, n_waves = (geometry >> 20) & 0x1Fu;
+    const int m = (int)((geometry >> 25) & 0xFu);
+    const uint32_t flags = geometry >> 29;
+    const uint32_t in_f = n_chunks * kFastChunk, n_threads = n_waves * kWave;
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const uint32_t n_waves = blockDim.x >> 6;
     const uint32_t quarter = lane >> 4, li = lane & 15;
 
-    const uint32_t n_quads = (P.out_f + 3) >> 2;
+    const uint32_t n_quads = (out_f + 3) >> 2;
     const uint32_t quad0 = blockIdx.x * quads_per_wg;
     const uint32_t n_steps = min(quads_per_wg, n_quads - quad0);
     const uint32_t row0 = quad0 * 4;
-    const uint32_t rows_here = min(n_steps * 4, P.out_f - row0);
+    const uint32_t rows_here = min(n_steps * 4, out_f - row0);
     constexpr uint32_t qcap = kRQueue;  // records the wave's queue holds
-    const uint32_t rows_cap = min(quads_per_wg * 4, P.out_f);
+    const uint32_t rows_cap = min(quads_per_wg * 4, out_f);
     const RowsXLds L = rowsx_layout(rows_cap, n_chunks, n_waves, MT, qcap);
 
     // the pair table is addressed with (index bits | lane bits): it must sit at LDS address 0
     if ((uint32_t)(uintptr_t)(lds_ptr_t)smem != 0) {
-        for (uint32_t t = tid; t < rows_here * MT; t += blockDim.x)
+        for (uint32_t t = tid; t < rows_here * MT; t += n_threads)
             if ((int)(t % MT) < m) {
-                if (y32) y32[(size_t)(t % MT) * P.out_f + row0 + t / MT] = __uint_as_float(0x7FC00000u);  // NaN
+                if (y32) y32[(size_t)(t % MT) * out_f + row0 + t / MT] = __uint_as_float(0x7FC00000u);  // NaN
                 else y[(int64_t)(t % MT) * ldy + row0 + t / MT] = 0x7FC0;
             }
         return;
@@ -511,12 +519,12 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
     // the scale is asked for here, with the first requests: read where the pair table is built, it was a trip to memory
     // of its own between the table slices' and the barrier
-    const uint16_t scale_bits = *P.scale;
+    const uint16_t scale_bits = *scale_ptr;
     // ---- the activation row: needs nothing but the arguments, so it is requested first.  Lane (t, l) of the copy
     // fetches piece l * 4 + t of the block and the hardware puts it at piece t * 16 + l.
     {
         const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)x, 0, (int)((((int64_t)(m - 1) * ldx + P.in_f) * 2)), 0x00020000);
+            (void *)x, 0, (int)((((int64_t)(m - 1) * ldx + in_f) * 2)), 0x00020000);
         for (uint32_t t = wave; t < (uint32_t)m * n_chunks; t += n_waves) {
             const uint32_t j = t / n_chunks, col = t - j * n_chunks;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
@@ -527,13 +535,13 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
     // ---- workgroup set-up: table slices, pair table, splice masks ----
     const uint32_t unit0 = row0 * n_chunks;
-    const uint32_t entries = P.out_f * n_chunks + 1;
-    for (uint32_t i = tid; i <= rows_here * n_chunks; i += blockDim.x) {
+    const uint32_t entries = out_f * n_chunks + 1;
+    for (uint32_t i = tid; i <= rows_here * n_chunks; i += n_threads) {
         tq1[i] = (uint32_t)prefix[unit0 + i];
         if (!ANY) tq2[i] = (uint32_t)prefix[entries + unit0 + i];
     }
     const float scale = bf16_bits_to_f32(scale_bits);
-    for (uint32_t i = tid; i < 64 * 32; i += blockDim.x) {
+    for (uint32_t i = tid; i < 64 * 32; i += n_threads) {
         const int c0 = (i >> 5) & 7, c1 = i >> 8;
         const f32x2 w = {c0 < 7 ? (float)(c0 - 3) * scale : 0.0f, c1 < 7 ? (float)(c1 - 3) * scale : 0.0f};
         lut[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(w, bf16x2));  // round to nearest even
@@ -555,9 +563,9 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     __syncthreads();
 
     const __amdgpu_buffer_rsrc_t b1_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc((void *)P.bm[0], 0, (int)(P.bm_words[0] * 4u), 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc((void *)bm0, 0, (int)(out_f * (in_f >> 5) * 4u), 0x00020000);  // whole words here
     const __amdgpu_buffer_rsrc_t l1_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc((void *)P.st[0], 0, (int)(P.st_words[0] * 4u), 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc((void *)st0, 0, (int)(P.st_words[0] * 4u), 0x00020000);
 
     // ---- this workgroup's share of bitmap 1 and of the 5-bit / 8-bit streams (as in k_gemv358_rows) ----
     SideView sv;
@@ -565,7 +573,7 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
     if (!ANY) {
         const uint32_t n_local = rows_here * n_chunks;
         const uint32_t q1b = tq1[0], q2b = tq2[0], q1e = tq1[n_local], q2e = tq2[n_local];
-        const uint32_t nl1b = row0 * P.in_f - q1b, nl1e = (row0 + rows_here) * P.in_f - q1e;
+        const uint32_t nl1b = row0 * in_f - q1b, nl1e = (row0 + rows_here) * in_f - q1e;
         sv.base = L.side;
         sv.b2w0 = nl1b >> 5;
         sv.l2w0 = (uint32_t)(((uint64_t)q2b * 5u) >> 5);
@@ -803,14 +811,14 @@ k_gemv358_rowsx(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, ui
 
     // ---- add the waves' row sums in wave order, write bf16 ----
     const uint32_t first_acc = L.waves + kXStages * kRStageBytes + qcap * 16;
-    for (uint32_t t = tid; t < rows_here * MT; t += blockDim.x) {
+    for (uint32_t t = tid; t < rows_here * MT; t += n_threads) {
         const uint32_t slot = t / MT, j = t - slot * MT;
         if ((int)j >= m) continue;
         float sum = 0.0f;
         for (uint32_t w = 0; w < n_waves; ++w)
             sum += *reinterpret_cast<const float *>(smem + first_acc + w * wave_lds_bytes_x(MT, rows_cap, qcap) + t * 4);
         // a workgroup owns whole rows: the one addition per output a split-K caller's fp32 vector takes, or bf16
-        if (y32) atomicAdd(&y32[(size_t)j * P.out_f + row0 + slot], sum);
+        if (y32) atomicAdd(&y32[(size_t)j * out_f + row0 + slot], sum);
         else y[(int64_t)j * ldy + row0 + slot] = (uint16_t)f32_to_bf16_bits(sum);
     }
 }
@@ -940,8 +948,12 @@ static int launch_rowsx(const Dev &P, const int32_t *prefix, uint32_t n_chunks, 
     uint32_t flags = 0;
     if (((uintptr_t)P.last & 3u) == 0) flags |= kFlagStageSide;
     const size_t lds = rowsx_layout(min(quads * 4, P.out_f), n_chunks, waves, MT, kRQueue).total;
-    hipLaunchKernelGGL((k_gemv358_rowsx<MT, ANY>), dim3(groups), dim3(waves * kWave), lds, s, P, prefix, n_chunks, quads,
-                       flags, x, m, ldx, y, ldy, y32);
+    // the launch geometry in one word: column blocks (12 bits), row quads per workgroup (8), waves (5), activation rows
+    // (4), flags (3)
+    if (n_chunks > 0xFFFu || quads > 0xFFu || waves > 0x1Fu || m > 0xF || flags > 7u) return IXH_EUNSUPPORTED;
+    const uint32_t geometry = n_chunks | (quads << 12) | (waves << 20) | ((uint32_t)m << 25) | (flags << 29);
+    hipLaunchKernelGGL((k_gemv358_rowsx<MT, ANY>), dim3(groups), dim3(waves * kWave), lds, s, prefix, x, P.scale, ldx,
+                       P.bm[0], P.st[0], P.out_f, geometry, P, y, ldy, y32);
     return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
 }
 
