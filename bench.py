@@ -34,28 +34,48 @@ MFMA_BF16_PEAK = 2.5e15  # FLOP/s dense bf16, MI355X published
 # sources it was measured on (kernel_sources_sha16) and is reported only while the sources still hash to it;
 # workloads without a counter run, or measured on other sources, report null.
 # (bytes per launch, the sources the kernel is compiled from, their kernel_sources_sha16 at the counter run)
-_ROWS = ("ixh_rows358.hip", "ixh_rows_common.h", "ixh_dev.h")
+_ROWS = ("ixh_rows358.hip", "ixh_rows_common.h", "ixh_dev.h", "build.sh")
 _TILES = ("ixh_tiles358.hip", "ixh_rows_common.h", "ixh_dev.h")
 _DENSE = ("ixh_dense358.hip", "ixh_dense_tiles.h", "ixh_dev.h")
 _DENSE5 = ("ixh_dense5.hip", "ixh_dense_tiles.h", "ixh_dev.h")
+_PREFILL = ("ixh_prefill.hip", "ixh_staged.h", "ixh_dev.h")
+_DECODE_ROWS = ("ixh_decode_rows358.hip", "ixh_rows_common.h", "ixh_dev.h")
 _OLD = ((), "measured-on-earlier-sources")  # figures kept for the record; reported as null
 MEASURED_TRAFFIC_BYTES = {
-    "down_proj_5120x17408_m1_student_t": (23035.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "e45341197bdab021"),
-    "gate_up_17408x5120_m1_student_t": (22939.0 * 2.0 * 1024 + 40.0 * 1024, _ROWS, "e45341197bdab021"),
-    "attn_proj_5120x5120_m1_student_t": (7139.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "e45341197bdab021"),
+    "down_proj_5120x17408_m1_student_t": (23032.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "5ccd2523b03e02ca"),
+    "gate_up_17408x5120_m1_student_t": (22936.0 * 2.0 * 1024 + 40.0 * 1024, _ROWS, "5ccd2523b03e02ca"),
+    "attn_proj_5120x5120_m1_student_t": (7135.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "5ccd2523b03e02ca"),
     "down_proj_5120x17408_m1_calibrated": (33825.0 * 2.0 * 1024 + 40.0 * 1024, _DENSE, "711eef94d053feb1"),
     "down_proj_5120x17408_m1_five_level_calibrated": (49708.0 * 2.0 * 1024 + 1338.0 * 1024, _DENSE5, "aaca19573f1ed2a1"),
-    "gate_up_17408x5120_m4_student_t": (28674.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "3287305ecb77f4e3"),
-    "gate_up_17408x5120_m16_student_t": (26631.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "3287305ecb77f4e3"),
-    "attn_proj_5120x5120_m16_student_t": (8657.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "3287305ecb77f4e3"),
-    "down_proj_5120x17408_m16_student_t": (27676.0 * 2.0 * 1024 + 960.0 * 1024, _TILES, "3287305ecb77f4e3"),
+    "gate_up_17408x5120_m4_student_t": (28740.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "21f9d013a3b417ff"),
+    "gate_up_17408x5120_m16_student_t": (26687.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "21f9d013a3b417ff"),
+    "attn_proj_5120x5120_m16_student_t": (8657.0 * 2.0 * 1024 + 640.0 * 1024, _TILES, "21f9d013a3b417ff"),
+    "down_proj_5120x17408_m16_student_t": (27677.0 * 2.0 * 1024 + 960.0 * 1024, _TILES, "21f9d013a3b417ff"),
     "decode_5120x17408_five_level_calibrated": (49719.0 * 2.0 * 1024 + 174080.0 * 1024, _DENSE5, "aaca19573f1ed2a1"),
     "prefill_5120x5120_m512_five_level": (50297.9 * 2.0 * 1024 + 30720.0 * 1024,) + _OLD,
+    # both kernels of a step: k_prefill<5> + k_prefill_reduce
+    "prefill_5120x17408_m512_five_level": ((190401.0 + 15378.0) * 2.0 * 1024 + (30720.0 + 5120.0) * 1024, _PREFILL, "17fc44b7da55ae09"),
+    # k_decode358_rows<true> (x 2.0 / x 1.0 as above) + the operands and outputs of the library GEMM that
+    # torch.cuda.tunable picked (bf16 weight, X, Y: its FETCH_SIZE, 158,001, is weighted for other request sizes than
+    # our kernels' and fixes its reads only between 162 and 324 MB)
+    "prefill_5120x17408_m512_five_level_unfused": (23101.0 * 2.0 * 1024 + 179854.0 * 1024
+                                                   + 2.0 * (5120 * 17408 + 512 * 17408 + 512 * 5120),
+                                                   _DECODE_ROWS, "54f9e436740640ef"),
     "decode_5120x17408_student_t": (23268.0 * 2.0 * 1024 + 179524.0 * 1024,) + _OLD,
     "decode_5120x17408_calibrated": (36308.0 * 2.0 * 1024 + 174080.0 * 1024,) + _OLD,
     "decode_gs_5120x17408_student_t": (33559.0 * 2.0 * 1024 + 174080.0 * 1024,) + _OLD,
     # all kernels of one encode step together (absmax, count, scans, clear, pack)
     "encode_5120x17408_student_t": ((87053 + 87092 + 1402 + 15 + 92442) * 2.0 * 1024 + (32 + 2040 + 1362 + 32694 + 63405) * 1024,) + _OLD,
+}
+
+# Wave-level instruction counts per launch of the dominant kernel (SQ_INSTS_VALU, SQ_INSTS_SALU, SQ_INSTS_LDS from one
+# rocprofv3 --pmc run of this script, mean over the launches), gated by the hash of the kernel's sources like the
+# traffic figures.  Reported per weight: vector and LDS instructions x 64 lanes / weights, scalar instructions / weights.
+MEASURED_INSTRUCTIONS = {
+    "down_proj_5120x17408_m1_student_t": ((5734195.0, 4469166.0, 1360042.0), _ROWS, "5ccd2523b03e02ca"),
+    "gate_up_17408x5120_m1_student_t": ((6030194.0, 4450915.0, 1414314.0), _ROWS, "5ccd2523b03e02ca"),
+    "attn_proj_5120x5120_m1_student_t": ((3570752.0, 2281697.0, 593732.0), _ROWS, "5ccd2523b03e02ca"),
+    "down_proj_5120x17408_m1_level1_only": ((4881551.0, 4104235.0, 1254926.0), _ROWS, "5ccd2523b03e02ca"),
 }
 
 WORKLOADS = {
@@ -72,6 +92,9 @@ WORKLOADS = {
     "attn_proj_5120x5120_m1_five_level": (5120, 5120, 1, "student_t", (3, 4, 5, 6, 8)),
     "attn_proj_5120x5120_m1_calibrated": (5120, 5120, 1, "calibrated"),
     "graph64_5120x5120_m1_calibrated": (5120, 5120, 1, "calibrated"),
+    # level-1 share swept between the dense mix and the almost-all-level-1 mix (the rest 8 : 1 between levels 2 and 3):
+    # where the row-block kernels (--gemv-flags 8) and the level-by-level kernel (--gemv-flags 32) cross
+    **{f"down_proj_5120x17408_m1_l1_share_{pct}": (5120, 17408, 1, f"l1_share_{pct}") for pct in (80, 85, 90, 95, 97, 99)},
     "attn_proj_5120x5120_m1_student_t": (5120, 5120, 1, "student_t"),
     "down_proj_5120x17408_m4_student_t": (5120, 17408, 4, "student_t"),
     "down_proj_5120x17408_m8_student_t": (5120, 17408, 8, "student_t"),
@@ -125,6 +148,9 @@ def make_weight(out_f, in_f, recipe):
         return student_t_weight(out_f, in_f, seed=0)
     if recipe == "outlier":
         return outlier_weight(out_f, in_f, seed=0)
+    if recipe.startswith("l1_share_"):
+        l1 = int(recipe.rsplit("_", 1)[1]) / 100.0
+        return calibrated_weight(out_f, in_f, seed=0, fractions=(l1, (1.0 - l1) * 8 / 9, (1.0 - l1) / 9))[0]
     if recipe == "level1_only":  # every value within the first level but the one +-127 that fixes the scale
         return calibrated_weight(out_f, in_f, seed=0, fractions=(1.0, 0.0, 0.0))[0]
     return calibrated_weight(out_f, in_f, seed=0)[0]
@@ -363,6 +389,19 @@ def measured_traffic(workload):
     return nbytes if files and sha16 == kernel_sources_sha16(files) else None
 
 
+def measured_instructions(workload, n_weights):
+    """Vector / scalar / LDS instructions per weight from the committed counter run (None when the kernel's sources
+    have changed since)."""
+    hit = MEASURED_INSTRUCTIONS.get(workload)
+    if hit is None:
+        return {"valu_per_weight": None, "salu_per_weight": None, "lds_per_weight": None}
+    (valu, salu, lds), files, sha16 = hit
+    if not files or sha16 != kernel_sources_sha16(files):
+        return {"valu_per_weight": None, "salu_per_weight": None, "lds_per_weight": None}
+    return {"valu_per_weight": round(valu * 64.0 / n_weights, 3), "salu_per_weight": round(salu / n_weights, 4),
+            "lds_per_weight": round(lds * 64.0 / n_weights, 3)}
+
+
 def build_layers(workload, dev, copies=0, unfused=False):
     """The packed layer of a workload (CPU generator, CPU writer: the literal recipe), `copies` device copies of it
     as StreamingLinear modules, and its activations."""
@@ -510,6 +549,10 @@ def also_block(dev, args):
                 flops = 2.0 * m * out_f * in_f
                 r["TFLOP_per_s"] = round(flops / (ms * 1e-3) / 1e12, 1)
                 r["frac_mfma"] = round(flops / (ms * 1e-3) / MFMA_BF16_PEAK, 4)
+                # the same step against the HBM roofline: packed layer + activations in + outputs out
+                alg_bytes = packed["total_bytes"] + m * in_f * 2 + m * out_f * 2
+                r["frac_hbm"] = round(alg_bytes / (ms * 1e-3) / HBM_PEAK, 4)
+                r["traffic"] = measured_traffic(name if variant == "fused" else name + "_unfused")
                 out.setdefault(name, {})["ixh_gemm" if variant == "fused" else "decode_plus_tuned_library_gemm"] = r
             else:
                 alg_bytes = packed["total_bytes"] + m * in_f * 2 + m * out_f * 2
@@ -626,9 +669,12 @@ def main():
         "roofline": {
             "bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
             "frac": achieved / HBM_PEAK, "traffic": measured_traffic(args.workload),
+            **measured_instructions(args.workload, out_f * in_f),
             "note": "algorithmic bytes = packed layer + x + y per launch; time = HIP-event time of the timed region / "
-                    "steps; traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script "
-                    "(null when the kernel sources have changed since those runs)",
+                    "steps; traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script; "
+                    "valu / lds_per_weight = wave instructions x 64 lanes / weights, salu_per_weight = scalar "
+                    "instructions / weights, from an SQ_INSTS_* run (all null when the kernel sources have changed "
+                    "since those runs)",
         },
         "launch": "eager" if graph is None else f"hipGraph of {copies} layer launches, replayed {steps // copies}x",
         "timed_region": f"{steps} steps = {ms_per_step * steps:.1f} ms: at least --steps ({args.steps}) and at least "

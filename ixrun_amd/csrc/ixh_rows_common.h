@@ -98,14 +98,6 @@ __device__ __forceinline__ uint64_t lds_read2_raw(uint32_t addr) {  // words at 
     asm volatile("ds_read2_b32 %0, %1 offset1:1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
     return v;
 }
-// LDS stores that the compiler does not order against copies into LDS that are still in flight (it would wait for all
-// of them before a store it can see); complete after s_waitcnt lgkmcnt(0)
-__device__ __forceinline__ void lds_store_u32_raw(uint32_t addr, uint32_t v) {
-    asm volatile("ds_write_b32 %0, %1" ::"v"(addr), "v"(v) : "memory");
-}
-__device__ __forceinline__ void lds_store_u128_raw(uint32_t addr, u32x4 v) {
-    asm volatile("ds_write_b128 %0, %1" ::"v"(addr), "v"(v) : "memory");
-}
 __device__ __forceinline__ void lds_add_f32_raw(uint32_t addr, float v) {  // complete after s_waitcnt lgkmcnt(0)
     asm volatile("ds_add_f32 %0, %1" ::"v"(addr), "v"(v) : "memory");
 }
