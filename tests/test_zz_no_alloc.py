@@ -113,21 +113,27 @@ def test_noalloc_rejects_what_does_not_fit(dev):
     assert torch.all(y == 7.0)  # nothing ran
 
 
-def test_noalloc_allocates_nothing_and_replays_in_a_graph(dev):
+def test_noalloc_allocates_nothing_and_replays_in_a_graph(dev, gemv_option):
     """The device's free memory does not move over a run of calls (outputs allocated beforehand; the first call on a
     device, which looks the buffer's address up, is made before the measurement), and a call captured into a
     hipGraph replays correctly: three replays with new activations each time, eager work and a synchronisation
-    between them, every replay equal to the eager ixh_gemv result."""
+    between them, every replay equal to the eager ixh_gemv result.  The routes: row-block kernel (no workspace), the
+    tile kernel with two workgroups to a block of rows (their pieces meet in the buffer and a second launch adds them),
+    the staged and the column-block kernel (one piece per 512 columns in the buffer)."""
     from ixrun_amd import _lib
 
+    gemv_option("gemv_tiles", 1)
+    gemv_option("gemv_tile_cus", 4)
+    gemv_option("gemv_tile_split", 2)
     cases = []
-    for recipe, out_f, in_f, m, flags in (("student_t", 640, 4608, 1, 0), ("student_t", 640, 4608, 16, 0),
+    for recipe, out_f, in_f, m, flags in (("student_t", 640, 4608, 1, 0), ("student_t", 640, 4608, 16, _lib.IXH_GEMV_FORCE_358),
                                           ("outlier", 96, 1536, 3, _lib.IXH_GEMV_STAGED),
                                           ("calibrated", 640, 4608, 2, _lib.IXH_GEMV_COLUMN_KERNEL)):
         dp, table = _layer(recipe, out_f, in_f, dev)
         x = activations(m, in_f, seed=11 + m).to(dev)
         y = torch.empty((m, out_f), dtype=torch.bfloat16, device=dev)
         cases.append((dp, table, x, y, flags))
+    assert cases[1][0].gemv_workspace_bytes(512, 16, _lib.IXH_GEMV_FORCE_358) > 0
     for dp, table, x, y, flags in cases:  # warm: code object loaded, buffer address known, plans cached
         dp.gemv_noalloc(table, 512, x, y, flags=flags)
     torch.cuda.synchronize()
