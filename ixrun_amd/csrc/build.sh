@@ -4,7 +4,7 @@
 set -e
 cd "$(dirname "$0")"
 HIPCC="${HIPCC:-/opt/rocm/bin/hipcc}"
-SRCS="ixh_api.hip ixh_generic.hip ixh_fast358.hip ixh_rows358.hip ixh_slots358.hip ixh_strips358.hip ixh_tiles358.hip ixh_prefill.hip ixh_decode_staged.hip ixh_gemv_staged.hip ixh_encode.hip ixh_dense358.hip ixh_dense5.hip ixh_decode_rows358.hip"
+SRCS="ixh_api.hip ixh_generic.hip ixh_fast358.hip ixh_rows358.hip ixh_slots358.hip ixh_strips358.hip ixh_tiles358.hip ixh_prefill.hip ixh_prefill358.hip ixh_decode_staged.hip ixh_gemv_staged.hip ixh_encode.hip ixh_dense358.hip ixh_dense5.hip ixh_decode_rows358.hip"
 FLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Xclang -target-feature -Xclang -packed-fp32-ops -Wall -Wno-unused-function -Wno-pass-failed $*"
 # Kernels of these files take the arguments that their first memory requests need as their leading arguments; the
 # hardware loads up to 14 argument words into registers before a wave starts (older firmware runs the loads that the

@@ -23,6 +23,7 @@ std::atomic<int> g_opt_gemv_tile_rows{0};
 std::atomic<int> g_opt_gemv_tile_cus{0};
 std::atomic<int> g_opt_gemv_tile_split{0};
 std::atomic<int> g_opt_gemv_dense_tiles{0};
+std::atomic<int> g_opt_gemm_tiles{0};
 extern std::atomic<int> g_opt_gemv_slots;
 extern std::atomic<int> g_opt_gemv_slot_waves;
 
@@ -132,6 +133,11 @@ int ixh_set_option(const char *name, int64_t value) {
     if (strcmp(name, "gemv_dense_tiles") == 0) {
         if (value < -1 || value > 1) { set_error("gemv_dense_tiles %lld not in -1..1", (long long)value); return IXH_EINVAL; }
         g_opt_gemv_dense_tiles.store((int)value, std::memory_order_relaxed);
+        return IXH_OK;
+    }
+    if (strcmp(name, "gemm_tiles") == 0) {
+        if (value < -1 || value > 2) { set_error("gemm_tiles %lld not in -1..2", (long long)value); return IXH_EINVAL; }
+        g_opt_gemm_tiles.store((int)value, std::memory_order_relaxed);
         return IXH_OK;
     }
     if (strcmp(name, "gemv_slots") == 0) {
@@ -439,7 +445,17 @@ int ixh_gemv_noalloc(const IxhPacked *packed, const int32_t *prefix, int64_t chu
 size_t ixh_gemm_workspace_bytes(const IxhPacked *packed, int32_t m) {
     Dev d;
     if (to_dev(packed, &d) || d.n == 0 || m < 1) return 0;
-    return prefill_workspace_bytes(d, (uint32_t)m);
+    return max(prefill_workspace_bytes(d, (uint32_t)m), prefill358_workspace_bytes(d, (uint32_t)m));
+}
+
+// The kernel of ixh_prefill358.hip: tensors that are almost all level 1 (the full decode of such tensors and the
+// products of few activation rows switch at the same share), enough activation rows to fill its 64-row wave tiles.
+static bool gemm_takes_tiles(const Dev &d, const uint16_t *x, int64_t ldx, int32_t m, const void *workspace) {
+    const int want = g_opt_gemm_tiles.load(std::memory_order_relaxed);
+    if (want < 0 || !prefill358_supports(d, x, ldx) || ((uintptr_t)workspace & 15u) != 0) return false;
+    if (want > 0) return true;
+    const bool mostly_l1 = (uint64_t)d.st_words[0] * 32u / 3u >= (uint64_t)d.n / 100u * 97u;
+    return mostly_l1 && m >= 96;
 }
 
 int ixh_gemm(const IxhPacked *packed, const int32_t *prefix, const uint16_t *x, int32_t m, int64_t ldx, uint16_t *y,
@@ -457,16 +473,21 @@ int ixh_gemm(const IxhPacked *packed, const int32_t *prefix, const uint16_t *x, 
     }
     if (!prefix || !x) { set_error("prefix or x is NULL"); return IXH_EINVAL; }
     if (ldx < (int64_t)d.in_f && m > 1) { set_error("ldx %lld < in_f %u", (long long)ldx, d.in_f); return IXH_EINVAL; }
-    if (!prefill_supports(d, x, ldx)) {
+    const bool tiles = gemm_takes_tiles(d, x, ldx, m, workspace);
+    if (!tiles && !prefill_supports(d, x, ldx)) {
         set_error("gemm: needs in_f %% 512 == 0, x 16-byte aligned, ldx %% 8 == 0, last stream 4-byte aligned");
         return IXH_EUNSUPPORTED;
     }
-    const size_t need = prefill_workspace_bytes(d, (uint32_t)m);
+    const size_t need = tiles ? prefill358_workspace_bytes(d, (uint32_t)m) : prefill_workspace_bytes(d, (uint32_t)m);
     if (!workspace || workspace_bytes < need) {
         set_error("workspace of %zu bytes needed, %zu given", need, workspace ? workspace_bytes : (size_t)0);
         return IXH_EWORKSPACE;
     }
-    rc = launch_prefill(d, prefix, x, (uint32_t)m, ldx, y, ldy, (float *)workspace, (hipStream_t)stream);
+    if (tiles)
+        rc = launch_prefill358(d, prefix, x, (uint32_t)m, ldx, y, ldy, (float *)workspace,
+                               g_opt_gemm_tiles.load(std::memory_order_relaxed) == 2 ? 1u : 0u, (hipStream_t)stream);
+    else
+        rc = launch_prefill(d, prefix, x, (uint32_t)m, ldx, y, ldy, (float *)workspace, (hipStream_t)stream);
     if (rc == IXH_ELAUNCH) set_error("gemm: launch failed");
     return rc;
 }

@@ -229,6 +229,14 @@ k_prefill_reduce(const float *__restrict__ ws, uint32_t m_rows, uint32_t out_f, 
     y[(int64_t)m * ldy + n] = (uint16_t)f32_to_bf16_bits(sum);
 }
 
+int launch_prefill_reduce(const float *ws, uint32_t m_rows, uint32_t out_f, uint32_t n_slices, uint16_t *y, int64_t ldy,
+                          hipStream_t s) {
+    const size_t total = (size_t)m_rows * out_f;
+    hipLaunchKernelGGL(k_prefill_reduce, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, ws, m_rows, out_f, n_slices,
+                       y, ldy);
+    return hipGetLastError() == hipSuccess ? IXH_OK : IXH_ELAUNCH;
+}
+
 // K slices for a shape: the count that makes rounds x (columns per workgroup + a start-up share) smallest,
 // with two workgroups per CU.
 static uint32_t pick_slices(uint32_t tiles, uint32_t n_chunks) {

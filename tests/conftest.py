@@ -35,10 +35,10 @@ def force_decoder():
 
 @pytest.fixture
 def gemv_option():
-    """Set a kernel-selection switch of ixh_gemv for the duration of a test (``ixh_set_option``)."""
+    """Set a kernel-selection switch of ixh_gemv or ixh_gemm for the duration of a test (``ixh_set_option``)."""
     from ixrun_amd import _lib
 
-    defaults = {"gemv_strips": 0, "gemv_shared_x": 8, "gemv_tiles": 0, "gemv_tile_rows": 0, "gemv_tile_cus": 0, "gemv_tile_split": 0, "gemv_dense_tiles": 0, "gemv_slots": 0, "gemv_slot_waves": 0}
+    defaults = {"gemv_strips": 0, "gemv_shared_x": 8, "gemv_tiles": 0, "gemv_tile_rows": 0, "gemv_tile_cus": 0, "gemv_tile_split": 0, "gemv_dense_tiles": 0, "gemv_slots": 0, "gemv_slot_waves": 0, "gemm_tiles": 0}
     touched = []
 
     def set_(name: str, value: int) -> None:
