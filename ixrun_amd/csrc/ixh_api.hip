@@ -136,7 +136,7 @@ int ixh_set_option(const char *name, int64_t value) {
         return IXH_OK;
     }
     if (strcmp(name, "gemm_tiles") == 0) {
-        if (value < -1 || value > 2) { set_error("gemm_tiles %lld not in -1..2", (long long)value); return IXH_EINVAL; }
+        if (value < -1 || value > 4096) { set_error("gemm_tiles %lld not in -1..2", (long long)value); return IXH_EINVAL; }
         g_opt_gemm_tiles.store((int)value, std::memory_order_relaxed);
         return IXH_OK;
     }
@@ -485,7 +485,7 @@ int ixh_gemm(const IxhPacked *packed, const int32_t *prefix, const uint16_t *x, 
     }
     if (tiles)
         rc = launch_prefill358(d, prefix, x, (uint32_t)m, ldx, y, ldy, (float *)workspace,
-                               g_opt_gemm_tiles.load(std::memory_order_relaxed) == 2 ? 1u : 0u, (hipStream_t)stream);
+                               g_opt_gemm_tiles.load(std::memory_order_relaxed) == 2 ? 1u : (uint32_t)(max(0, g_opt_gemm_tiles.load(std::memory_order_relaxed)) >> 4), (hipStream_t)stream);
     else
         rc = launch_prefill(d, prefix, x, (uint32_t)m, ldx, y, ldy, (float *)workspace, (hipStream_t)stream);
     if (rc == IXH_ELAUNCH) set_error("gemm: launch failed");

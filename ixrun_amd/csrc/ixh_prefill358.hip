@@ -9,8 +9,8 @@
 //            (ixh_decode_rows358.hip): rank the lane's bitmap word, read its 96-bit code window from the staged
 //            stream, splice the elements above level 1 out, look the code pairs up in the table of dequantised pairs;
 //   multiply every wave multiplies 64 activation rows x the 128 weight rows x 512 k: the weight operand from the LDS
-//            tile (rows 1 KB apart, the 16-byte pieces of a row XOR-swizzled with the row so that the sixteen rows of
-//            an operand hit all banks), the activation operand from global memory.
+//            tile (rows 1 KB apart, the 16-byte pieces of a row swizzled so that neither the sixteen rows of an
+//            operand nor the sixteen lanes that store a row unit collide on a bank), the activation operand from global memory.
 // The 128-row tile is what makes the activations affordable: a workgroup reads its K slice of X once per 128 weight
 // rows, and an operand register loaded from X feeds eight matrix instructions.
 //
@@ -20,12 +20,15 @@
 // re-tiles X into operand order (k_prefill_xtile: the 1 KB of an operand consecutive in memory), and the main kernel
 // reads whole operands with one fully coalesced load each, two K steps ahead of their use.
 //
-// Elements above level 1 (a fraction of a percent in these tensors).  Their values do not depend on the level-1
-// decode: the e-th such element of a row unit is the element of rank (unit start - level-1 count before the unit) + e
-// in bitmap 1's domain.  At its start the workgroup computes the values of all such elements of its rows and K slice
-// (a few hundred, spread over the lanes, each a chain of a few dependent reads of the nested bitmaps) into a list in
-// LDS; the decode phase writes the level-1 part of a row with zeros in their places and then stores the list's
-// values over the zeros.  A workgroup with more such elements than the list holds computes each where it is needed.
+// Elements above level 1 (up to a few percent in these tensors).  Their values do not depend on the level-1 decode:
+// the e-th such element of a row unit is the element of rank (unit start - level-1 count before the unit) + e in
+// bitmap 1's domain.  At its start the workgroup computes the values (int8) of all such elements of its rows and K
+// slice, one element per lane and round (each a chain of a few dependent reads of the nested bitmaps), into one list
+// per unit column in global memory, rows in order; a column's list (at most 2048 values) is copied to LDS by LDS-DMA
+// during the multiply phase of the column before, together with the count of such elements before each row in that
+// column.  The decode phase writes the level-1 part of a row with zeros in their places and then stores the
+// dequantised list values over the zeros.  A column with more such elements than the list holds computes each where
+// it is needed.
 //
 // Memory pipeline of the decode phase: the bitmap words and the 3-bit stream range of a group of four row units reach
 // LDS by LDS-DMA (two stages per wave); the first two groups of a column are requested before the multiply phase of
@@ -45,25 +48,42 @@ constexpr uint32_t kQRows = 128;       // weight rows per workgroup
 constexpr uint32_t kQMaxM = 512;       // activation rows per launch
 constexpr uint32_t kQMaxCols = 7;      // unit columns per K slice at most
 constexpr uint32_t kQMaxSlices = 16;
-constexpr uint32_t kQValueCap = 1024;  // values of elements above level 1 kept in LDS
+constexpr uint32_t kQValueCap = 2048;  // values (int8) of a unit column's elements above level 1 kept in LDS
 constexpr uint32_t kQStage = 1280;     // 1024 stream + 256 bitmap
 // LDS map.  The pair table sits at address 0: it is addressed with (index bits | lane bits).
 constexpr uint32_t kQLut = 0;                                          // [64 pairs][16 copies] words
 constexpr uint32_t kQSplice = kQLut + 64 * 16 * 4;                     // [33][2] x 16 bytes
 constexpr uint32_t kQTq = kQSplice + 33 * 32;                          // [128 rows][8]: level-1 counts before the slice's columns
-constexpr uint32_t kQRowBase = kQTq + kQRows * (kQMaxCols + 1) * 4;    // [129]: elements above level 1 before a row (in the slice)
-constexpr uint32_t kQValues = kQRowBase + 132 * 4;                     // [kQValueCap] bf16
-constexpr uint32_t kQRings = kQValues + kQValueCap * 2;                // [8 waves][2 stages]
+constexpr uint32_t kQRowBase = kQTq + kQRows * (kQMaxCols + 1) * 4;    // [2][132] u16: elements above level 1 before a row in a column (saturated), for the column being decoded and the next
+constexpr uint32_t kQValues = kQRowBase + 132 * 4;                     // [kQValueCap] int8
+constexpr uint32_t kQRings = kQValues + kQValueCap;                    // [8 waves][2 stages]
 constexpr uint32_t kQTile = (kQRings + kQWaves * 2 * kQStage + 1023u) & ~1023u;  // [128][64 pieces of 16 bytes], swizzled
 constexpr uint32_t kQLdsBytes = kQTile + kQRows * 1024;
+constexpr uint32_t kQListBytes = kQMaxCols * kQValueCap;  // a workgroup's value lists in global memory, one per column
 static_assert(kQLdsBytes <= 160 * 1024, "LDS of a CU");
 static_assert(kQSplice % 16 == 0 && kQTq % 16 == 0 && kQValues % 16 == 0 && kQRings % 16 == 0, "alignment");
 
+struct QReload { static constexpr bool value = true; };
+struct QLast { static constexpr bool value = false; };
+
 __device__ __forceinline__ void q_barrier_lds() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 __device__ __forceinline__ void q_wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// "at most N vector-memory operations outstanding", as an instruction the compiler sees: it keeps its own count of
+// what is in flight and, not knowing about a wait written in assembly, would later wait again for copies that have
+// long landed, at a point where that also waits for the ones issued since.
+template <int N>
+__device__ __forceinline__ void q_wait_vmem() {
+    static_assert(N >= 0 && N < 16, "low four bits of vmcnt");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | N);  // expcnt and lgkmcnt at their maxima: no wait on them
+    asm volatile("" ::: "memory");
+}
 
-// 16-byte piece p (0..63) of row r of the weight tile
-__device__ __forceinline__ uint32_t q_tile_addr(uint32_t r, uint32_t p) { return kQTile + r * 1024u + ((p ^ (r & 15u)) << 4); }
+// 16-byte piece p (0..63) of row r of the weight tile sits at slot p ^ (p >> 4) ^ (r & 15) of the row's 1 KB: the
+// sixteen rows of a weight operand (same p) then hit sixteen different groups of four banks, and so do the sixteen
+// lanes of a row unit when each stores the j-th of its four consecutive pieces (p = 4 lane + j).
+__device__ __forceinline__ uint32_t q_tile_addr(uint32_t r, uint32_t p) {
+    return kQTile + r * 1024u + ((p ^ (p >> 4) ^ (r & 15u)) << 4);
+}
 
 // LDS stores issued outside the compiler's memory model: in front of a store it can see the compiler waits for every
 // LDS-DMA copy in flight, which here are the copies for the groups decoded next.  Complete after s_waitcnt lgkmcnt(0).
@@ -73,6 +93,50 @@ __device__ __forceinline__ void q_store128(uint32_t addr, uint32_t a, uint32_t b
 }
 __device__ __forceinline__ void q_store16(uint32_t addr, uint32_t v) {
     asm volatile("ds_write_b16 %0, %1" ::"v"(addr), "v"(v) : "memory");
+}
+
+// LDS reads issued outside the compiler's memory model, for the part of the decode phase that runs while the copies
+// for the groups decoded later are in flight: in front of a read it can see, the compiler waits for those copies.
+// Eight table look-ups in place (the address register receives the data), without the wait: the results are there
+// after q_release16 of the same registers (which the compiler must see as redefining them, or it may copy a register
+// before its read has returned).
+__device__ __forceinline__ void q_issue8(uint32_t (&r)[16], int h) {
+    asm volatile(
+        "ds_read_b32 %0, %0\n\t"
+        "ds_read_b32 %1, %1\n\t"
+        "ds_read_b32 %2, %2\n\t"
+        "ds_read_b32 %3, %3\n\t"
+        "ds_read_b32 %4, %4\n\t"
+        "ds_read_b32 %5, %5\n\t"
+        "ds_read_b32 %6, %6\n\t"
+        "ds_read_b32 %7, %7"
+        : "+v"(r[8 * h]), "+v"(r[8 * h + 1]), "+v"(r[8 * h + 2]), "+v"(r[8 * h + 3]), "+v"(r[8 * h + 4]), "+v"(r[8 * h + 5]),
+          "+v"(r[8 * h + 6]), "+v"(r[8 * h + 7])
+        :
+        : "memory");
+}
+__device__ __forceinline__ void q_release16(uint32_t (&r)[16]) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]), "+v"(r[8]),
+                   "+v"(r[9]), "+v"(r[10]), "+v"(r[11]), "+v"(r[12]), "+v"(r[13]), "+v"(r[14]), "+v"(r[15])
+                 :
+                 : "memory");
+}
+__device__ __forceinline__ void q_issue_i8(uint32_t addr, int &out) {
+    asm volatile("ds_read_i8 %0, %1" : "=&v"(out) : "v"(addr) : "memory");
+}
+__device__ __forceinline__ void q_release2(int &a, int &b) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b) : : "memory");
+}
+__device__ __forceinline__ int q_read_i8(uint32_t addr) {
+    int v;
+    asm volatile("ds_read_i8 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+}
+__device__ __forceinline__ uint32_t q_read_u32(uint32_t addr) {
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
+    return v;
 }
 
 // Value of the element of rank r in bitmap 1's domain, which lies in table unit `unit` (whose first element has rank
@@ -127,11 +191,13 @@ k_prefill_xtile(const uint16_t *__restrict__ x, int64_t ldx, uint32_t m_rows, ui
 
 __global__ void __launch_bounds__(kWave *kQWaves, 2)
 k_prefill358(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const u32x4 *__restrict__ xt, uint32_t n_mblk,
-             uint32_t m_rows, float *__restrict__ ws, uint32_t n_slices, uint32_t flags) {
+             uint32_t m_rows, float *__restrict__ ws, int8_t *__restrict__ lists, uint32_t n_slices, uint32_t flags) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const uint32_t quarter = lane >> 4, li = lane & 15;
+    // (not const: re-derived from an opaque copy of the lane number at the top of every column, so that the compiler
+    // does not carry the dozens of lane-dependent addresses of the decode phase in registers through the multiply phase)
+    uint32_t lane_v = lane, quarter = lane >> 4, li = lane & 15;
     const uint32_t slice = blockIdx.x % n_slices, tile = blockIdx.x / n_slices;
     const uint32_t n0 = tile * kQRows;
     const uint32_t c_begin = slice * n_chunks / n_slices, c_end = (slice + 1) * n_chunks / n_slices;
@@ -150,8 +216,9 @@ k_prefill358(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const
     uint32_t *const lut = reinterpret_cast<uint32_t *>(smem + kQLut);
     uint4 *const splice = reinterpret_cast<uint4 *>(smem + kQSplice);
     uint32_t *const tq = reinterpret_cast<uint32_t *>(smem + kQTq);
-    uint32_t *const rowbase = reinterpret_cast<uint32_t *>(smem + kQRowBase);
-    uint16_t *const values = reinterpret_cast<uint16_t *>(smem + kQValues);
+    uint16_t *const rowbase = reinterpret_cast<uint16_t *>(smem + kQRowBase);
+    int8_t *const values = reinterpret_cast<int8_t *>(smem + kQValues);
+    int8_t *const my_lists = lists + (size_t)blockIdx.x * kQListBytes;
     uint8_t *const ring = smem + kQRings + wave * 2 * kQStage;
     const uint32_t ring_addr = kQRings + wave * 2 * kQStage;
 
@@ -205,31 +272,64 @@ k_prefill358(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const
     issue(0, 0);
     issue(1, 0);
 
-    // ---- elements above level 1 of this workgroup's rows and slice: how many before each row, then their values ----
-    if (wave == 0) {
+    // ---- elements above level 1 of this workgroup's rows and slice ----
+    // Per column: how many before each row (a scan over the 128 rows by one wave; the counts of all columns go to
+    // the weight tile's memory, which is free until the first decode phase), and the column totals.
+    uint32_t *const offs = reinterpret_cast<uint32_t *>(smem + kQTile);  // [cols][132]
+    auto scan_column = [&](uint32_t cu, uint32_t *dst32, uint16_t *dst16) {  // one wave; either destination may be null
         const uint32_t r0 = 2 * lane, r1 = 2 * lane + 1;
-        const uint32_t v0 = cols * kFastChunk - (tq[r0 * 8 + cols] - tq[r0 * 8]);
-        const uint32_t v1 = cols * kFastChunk - (tq[r1 * 8 + cols] - tq[r1 * 8]);
+        const uint32_t v0 = kFastChunk - (tq[r0 * 8 + cu + 1] - tq[r0 * 8 + cu]);
+        const uint32_t v1 = kFastChunk - (tq[r1 * 8 + cu + 1] - tq[r1 * 8 + cu]);
         const uint32_t incl = wave_scan(v0 + v1);
-        rowbase[r0] = incl - v0 - v1;
-        rowbase[r1] = incl - v1;
-        if (lane == 63) rowbase[kQRows] = incl;
-    }
+        if (dst32) {
+            dst32[r0] = incl - v0 - v1;
+            dst32[r1] = incl - v1;
+            if (lane == 63) dst32[kQRows] = incl;
+        }
+        if (dst16) {
+            dst16[r0] = (uint16_t)min(incl - v0 - v1, 0xFFFFu);
+            dst16[r1] = (uint16_t)min(incl - v1, 0xFFFFu);
+            if (lane == 63) dst16[kQRows] = (uint16_t)min(incl, 0xFFFFu);
+        }
+    };
+    if (wave < cols) scan_column(wave, offs + wave * 132, wave == 0 ? rowbase : nullptr);
     __syncthreads();
-    const bool listed = rowbase[kQRows] <= kQValueCap && !(flags & 1u);  // flags & 1: never use the list (testing)
-    if (listed) {
-        for (uint32_t ru = tid; ru < kQRows * cols; ru += blockDim.x) {
-            const uint32_t rl = ru / cols, cu = ru - rl * cols;
-            const uint32_t q_lo = tq[rl * 8 + cu], q_hi = tq[rl * 8 + cu + 1];
-            const uint32_t n_esc = kFastChunk - (q_hi - q_lo);
-            const uint32_t off = rowbase[rl] + cu * kFastChunk - (q_lo - tq[rl * 8]);
+    // The values: one element per lane and round over all columns' lists; entry idx of column cu is the idx-th such
+    // element of the column, rows in order: its row by bisection of the rows' first indices.
+    if (!(flags & 1u)) {  // flags & 1: no lists, every element is computed where it is needed (testing)
+        uint32_t cbase[kQMaxCols + 1];  // first item of each column's list in the workgroup's run of items
+        cbase[0] = 0;
+#pragma unroll
+        for (uint32_t cu = 0; cu < kQMaxCols; ++cu) {
+            const uint32_t n = cu < cols ? offs[cu * 132 + kQRows] : 0u;
+            cbase[cu + 1] = cbase[cu] + (n <= kQValueCap ? n : 0u);  // a column that does not fit has no list
+        }
+        for (uint32_t g = tid; g < cbase[kQMaxCols]; g += blockDim.x) {
+            uint32_t cu = 0;
+#pragma unroll
+            for (uint32_t j = 1; j < kQMaxCols; ++j)
+                if (cbase[j] <= g) cu = j;
+            uint32_t idx = g;
+#pragma unroll
+            for (uint32_t j = 1; j < kQMaxCols; ++j)
+                if (cu == j) idx = g - cbase[j];
+            const uint32_t *const off = offs + cu * 132;
+            uint32_t lo = 0, hi = kQRows;
+            while (hi - lo > 1) {
+                const uint32_t mid = (lo + hi) >> 1;
+                if (off[mid] <= idx) lo = mid;
+                else hi = mid;
+            }
+            const uint32_t rl = lo, e = idx - off[rl], q_lo = tq[rl * 8 + cu];
             const uint32_t unit = min(n0 + rl, P.out_f - 1) * n_chunks + c_begin + cu;
             const uint32_t first = unit * kFastChunk - q_lo;
-            for (uint32_t e = 0; e < n_esc; ++e)
-                values[off + e] = (uint16_t)f32_to_bf16_bits((float)q_value_at(P, prefix, entries, unit, first, first + e) * scale);
+            const int8_t v = (int8_t)q_value_at(P, prefix, entries, unit, first, first + e);
+            my_lists[cu * kQValueCap + idx] = v;
+            if (cu == 0) values[idx] = v;
         }
     }
-    // (the barrier in front of the first decode phase makes the list visible)
+    // (the wait and the barrier in front of the first decode phase complete the stores and make column 0's list
+    // visible)
 
     auto splice_once = [&](uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &zrem) {
         const uint32_t e = zrem != 0 ? (uint32_t)__builtin_ctz(zrem) : 32u;
@@ -245,27 +345,42 @@ k_prefill358(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const
         w1 = (w1 & ~fm.y) | (kZeroCodes1 & fm.y);
         w2 = (w2 & ~fm.z) | (kZeroCodes2 & fm.z);
     };
-    // code window of group i of column ci (its data is in the ring), every element above level 1 spliced out;
-    // zeros: those elements; esc0: index in the list of the lane's first one
-    auto open_window = [&](uint32_t i, uint32_t ci, uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &zeros, uint32_t &esc0) {
-        const uint32_t rl = row_of(i);
-        const uint32_t stage = ring_addr + (i & 1u) * kQStage;
-        const uint32_t word = lds_u32(stage + 1024 + lane * 4);
-        const uint32_t q1u = lds_u32(kQTq + (rl * 8u + ci) * 4u);
-        const uint32_t q1r = lds_u32(kQTq + rl * 32u);
-        const uint32_t c = __popc(word);
-        const uint32_t excl = row_scan(c) - c;
-        const uint32_t off = excl * 3u + ((q1u * 3u) & 31u);  // bit offset inside the staged stream piece
-        const uint32_t wa = stage + quarter * 256 + (off >> 5) * 4;
-        const uint32_t d0 = lds_u32(wa), d1 = lds_u32(wa + 4), d2 = lds_u32(wa + 8), d3 = lds_u32(wa + 12);
-        w0 = __builtin_amdgcn_alignbit(d1, d0, off);
-        w1 = __builtin_amdgcn_alignbit(d2, d1, off);
-        w2 = __builtin_amdgcn_alignbit(d3, d2, off);
-        zeros = ~word;
-        // elements above level 1: before the row in the slice, before the column in the row, before the word in the unit
-        esc0 = lds_u32(kQRowBase + rl * 4u) + ci * kFastChunk - (q1u - q1r) + li * 32u - excl;
-        uint32_t zrem = zeros;
-        while (__ballot(zrem != 0) != 0) splice_once(w0, w1, w2, zrem);
+    // One group's decode state: the code window (every element above level 1 spliced out), those elements, and the
+    // index in the value list of the lane's first one.
+    struct Window {
+        uint32_t w0, w1, w2, zeros, esc;
+    };
+    // Windows of groups i and i + 1 of column ci (their data is in the ring), in lockstep, so that every trip to LDS
+    // serves both.
+    auto open_pair = [&](uint32_t i, uint32_t ci, Window &A, Window &B) {
+        const uint32_t rl_a = row_of(i), rl_b = row_of(i + 1);
+        const uint32_t stage_a = ring_addr + (i & 1u) * kQStage, stage_b = ring_addr + ((i + 1) & 1u) * kQStage;
+        const uint32_t word_a = lds_u32(stage_a + 1024 + lane_v * 4), word_b = lds_u32(stage_b + 1024 + lane_v * 4);
+        const uint32_t q1u_a = lds_u32(kQTq + (rl_a * 8u + ci) * 4u), q1u_b = lds_u32(kQTq + (rl_b * 8u + ci) * 4u);
+        const uint32_t rb = kQRowBase + (ci & 1u) * 264u;
+        const uint32_t rb_a = lds_u16(rb + rl_a * 2u), rb_b = lds_u16(rb + rl_b * 2u);
+        const uint32_t c_a = __popc(word_a), c_b = __popc(word_b);
+        const uint32_t excl_a = row_scan(c_a) - c_a, excl_b = row_scan(c_b) - c_b;
+        const uint32_t off_a = excl_a * 3u + ((q1u_a * 3u) & 31u), off_b = excl_b * 3u + ((q1u_b * 3u) & 31u);
+        const uint32_t wa = stage_a + quarter * 256 + (off_a >> 5) * 4, wb = stage_b + quarter * 256 + (off_b >> 5) * 4;
+        const uint32_t a0 = lds_u32(wa), a1 = lds_u32(wa + 4), a2 = lds_u32(wa + 8), a3 = lds_u32(wa + 12);
+        const uint32_t b0 = lds_u32(wb), b1 = lds_u32(wb + 4), b2 = lds_u32(wb + 8), b3 = lds_u32(wb + 12);
+        A.w0 = __builtin_amdgcn_alignbit(a1, a0, off_a);
+        A.w1 = __builtin_amdgcn_alignbit(a2, a1, off_a);
+        A.w2 = __builtin_amdgcn_alignbit(a3, a2, off_a);
+        B.w0 = __builtin_amdgcn_alignbit(b1, b0, off_b);
+        B.w1 = __builtin_amdgcn_alignbit(b2, b1, off_b);
+        B.w2 = __builtin_amdgcn_alignbit(b3, b2, off_b);
+        A.zeros = ~word_a;
+        B.zeros = ~word_b;
+        // elements above level 1 of the column: before the row, before the word in the unit
+        A.esc = rb_a + li * 32u - excl_a;
+        B.esc = rb_b + li * 32u - excl_b;
+        uint32_t zrem_a = A.zeros, zrem_b = B.zeros;
+        while (__ballot((zrem_a | zrem_b) != 0) != 0) {
+            splice_once(A.w0, A.w1, A.w2, zrem_a);
+            splice_once(B.w0, B.w1, B.w2, zrem_b);
+        }
     };
 
     q_f32x4 acc[4][8];
@@ -280,131 +395,181 @@ k_prefill358(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const
     const __amdgpu_buffer_rsrc_t x_rs =
         __builtin_amdgcn_make_buffer_rsrc((void *)xt, 0, (int)(n_kb * n_mblk * 1024u), 0x00020000);
     const bool multiplies = wave * 64u < m_rows;  // wave-uniform
-    const uint32_t lut_lane = (lane & 15u) << 2;
-    const uint32_t b_lane = kQTile + li * 1024u;  // weight operand: row 16 nb + li, piece 4 kb + quarter
+    uint32_t lut_lane, b_lane;
 
+    const __amdgpu_buffer_rsrc_t list_rs =
+        __builtin_amdgcn_make_buffer_rsrc((void *)my_lists, 0, (int)kQListBytes, 0x00020000);
     for (uint32_t ci = 0; ci < cols; ++ci) {
-        q_barrier_lds();  // the multiply phase of the column before is done with the weight tile; the value list is written
-        wait_vmem<0>();    // groups 0 and 1 of this column have landed
-        // ---- decode phase: this wave's 16 row units, four at a time ----
-        uint32_t cw0, cw1, cw2, czeros, cesc;
-        open_window(0, ci, cw0, cw1, cw2, czeros, cesc);
-#pragma unroll
-        for (uint32_t i = 0; i < 4; ++i) {
-            uint32_t wp[16];
+        // What this wave asked for has arrived (groups 0 and 1 of this column; from waves 0 and 1 the column's value
+        // list, and at the first column the stores of the lists), then: the multiply phase of the column before is
+        // done with the weight tile, and the list and the rows' counts of this column are in LDS.
+        q_wait_vmem<0>();
+        q_barrier_lds();
+        asm volatile("" : "+v"(lane_v));
+        quarter = lane_v >> 4, li = lane_v & 15u;
+        lut_lane = li << 2;
+        b_lane = kQTile + li * 1024u;  // weight operand: row 16 nb + li, piece 4 kb + quarter
+        const bool listed = lds_u16(kQRowBase + (ci & 1u) * 264u + kQRows * 2u) <= kQValueCap && !(flags & 1u);
+        // the next column's counts, while none of this wave's copies is in flight
+        if (wave == 0 && ci + 1 < cols) scan_column(ci + 1, nullptr, rowbase + ((ci + 1) & 1u) * 132u);
+        // ---- decode phase: this wave's 16 row units, four at a time, two groups of four in lockstep ----
+        Window A, B;
+        auto lut_addresses = [&](const Window &W, uint32_t (&la)[16]) {
 #pragma unroll
             for (int t = 0; t < 16; ++t) {
                 const int bit = 6 * t, ob = bit & 31, d = bit >> 5;
-                const uint32_t lo = d == 0 ? cw0 : (d == 1 ? cw1 : cw2);
-                const uint32_t hi = d == 0 ? cw1 : cw2;
+                const uint32_t lo = d == 0 ? W.w0 : (d == 1 ? W.w1 : W.w2);
+                const uint32_t hi = d == 0 ? W.w1 : W.w2;
                 uint32_t a;  // pair index at bits 11..6
                 if (ob > 26) a = __builtin_amdgcn_alignbit(hi, lo, ob - 6);
                 else if (ob >= 6) a = lo >> (ob - 6);
                 else a = lo << (6 - ob);
-                wp[t] = lds_u32((a & 0xFC0u) | lut_lane);
+                la[t] = (a & 0xFC0u) | lut_lane;
             }
-            const uint32_t zeros_now = czeros, esc_now = cesc;
-            // the stage group i was read from is free: group i + 2 goes there; then the window of group i + 1
-            if (i + 2 < 4) {
-                q_wait_lds();
-                issue(i + 2, ci);
-            }
-            if (i + 1 < 4) {
-                if (i == 1) wait_vmem<2>();       // group 2 has landed (group 3's two copies may be in flight)
-                else if (i == 2) wait_vmem<0>();  // group 3
-                open_window(i + 1, ci, cw0, cw1, cw2, czeros, cesc);
-            }
+        };
+        // the values of a lane's elements above level 1 over the zeros the lane has just written (LDS executes a wave's
+        // instructions in order); `first` is the list's value for the first of them, already read
+        auto patch = [&](uint32_t i, const Window &W, int first) {
+            if (W.zeros == 0) return;
             const uint32_t rl = row_of(i);
+            const uint32_t unit = min(n0 + rl, P.out_f - 1) * n_chunks + c_begin + ci;
+            uint32_t zr = W.zeros, nth = 0;
+            while (zr != 0) {
+                const uint32_t e = (uint32_t)__builtin_ctz(zr);
+                zr &= zr - 1;
+                int v = first;
+                if (!listed) {
+                    // rank of the lane's first such element in bitmap 1's domain: that of the unit's first, plus
+                    // those before the word in the unit
+                    const uint32_t first_rank = unit * kFastChunk - q_read_u32(kQTq + (rl * 8u + ci) * 4u);
+                    const uint32_t in_unit = W.esc - (q_read_u32(kQRowBase + (ci & 1u) * 264u + (rl & ~1u) * 2u) >> ((rl & 1u) * 16u) & 0xFFFFu);
+                    v = q_value_at(P, prefix, entries, unit, first_rank, first_rank + in_unit + nth);
+                } else if (nth != 0) {
+                    v = q_read_i8(kQValues + W.esc + nth);
+                }
+                q_store16(q_tile_addr(rl, 4 * li + (e >> 3)) + (e & 7u) * 2u, f32_to_bf16_bits((float)v * scale));
+                ++nth;
+            }
+        };
+        // groups i and i + 1 into the weight tile, in lockstep
+        auto emit_pair = [&](uint32_t i) {
+            uint32_t wa[16], wb[16];  // table addresses, then the pairs read from them
+            int va, vb;
+            lut_addresses(A, wa);
+            lut_addresses(B, wb);
+            q_issue8(wa, 0);
+            q_issue8(wa, 1);
+            q_issue8(wb, 0);
+            q_issue8(wb, 1);
+            // (a lane without such elements reads a neighbour's value, or a byte behind the list, and drops it; a
+            // column without a list has indices beyond it)
+            q_issue_i8(kQValues + min(A.esc, kQValueCap), va);
+            q_issue_i8(kQValues + min(B.esc, kQValueCap), vb);
+            q_release16(wa);
+            q_release16(wb);
+            q_release2(va, vb);
+            const uint32_t rl_a = row_of(i), rl_b = row_of(i + 1);
 #pragma unroll
             for (uint32_t j = 0; j < 4; ++j)
-                q_store128(q_tile_addr(rl, 4 * li + j), wp[4 * j], wp[4 * j + 1], wp[4 * j + 2], wp[4 * j + 3]);
-            // the values of the elements above level 1 over the zeros just written (LDS executes a wave's
-            // instructions in order)
-            if (zeros_now != 0) {
-                uint32_t zr = zeros_now, nth = 0;
-                const uint32_t unit = min(n0 + rl, P.out_f - 1) * n_chunks + c_begin + ci;
-                while (zr != 0) {
-                    const uint32_t e = (uint32_t)__builtin_ctz(zr);
-                    zr &= zr - 1;
-                    uint32_t v;
-                    if (listed) {
-                        v = lds_u16(kQValues + (esc_now + nth) * 2u);
-                    } else {
-                        // rank of the lane's first such element in bitmap 1's domain: that of the unit's first, plus
-                        // those before the word in the unit
-                        const uint32_t q1u = lds_u32(kQTq + (rl * 8u + ci) * 4u);
-                        const uint32_t first = unit * kFastChunk - q1u;
-                        const uint32_t in_unit = esc_now - (lds_u32(kQRowBase + rl * 4u) + ci * kFastChunk - (q1u - lds_u32(kQTq + rl * 32u)));
-                        v = f32_to_bf16_bits((float)q_value_at(P, prefix, entries, unit, first, first + in_unit + nth) * scale);
-                    }
-                    q_store16(q_tile_addr(rl, 4 * li + (e >> 3)) + (e & 7u) * 2u, v);
-                    ++nth;
-                }
-            }
-        }
+                q_store128(q_tile_addr(rl_a, 4 * li + j), wa[4 * j], wa[4 * j + 1], wa[4 * j + 2], wa[4 * j + 3]);
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                q_store128(q_tile_addr(rl_b, 4 * li + j), wb[4 * j], wb[4 * j + 1], wb[4 * j + 2], wb[4 * j + 3]);
+            patch(i, A, va);
+            patch(i + 1, B, vb);
+        };
+        if (!(flags & 2u)) {
+        // Groups 0 and 1 are in the ring: opening their windows frees the two stages for groups 2 and 3, whose copies
+        // then run under the table look-ups and tile stores of groups 0 and 1.
+        open_pair(0, ci, A, B);
+        q_wait_lds();
+        issue(2, ci);
+        issue(3, ci);
+        emit_pair(0);
+        q_wait_vmem<0>();  // groups 2 and 3 have landed
+        open_pair(2, ci, A, B);
         // the first two groups of the next column, to land during the multiply phase
         if (ci + 1 < cols) {
             q_wait_lds();
             issue(0, ci + 1);
             issue(1, ci + 1);
         }
-        q_barrier_lds();  // weight tile complete
+        emit_pair(2);
+        }
+        q_barrier_lds();  // weight tile complete; nobody reads this column's counts and list any more
+        if (ci + 1 < cols) {
+            // the next column's list (waves 0 and 1 copy 1 KB each), in place during the multiply phase
+            if (wave < 2)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(list_rs, (lds_ptr_t)(smem + kQValues + wave * 1024u), 16,
+                                                         (int)((ci + 1) * kQValueCap + wave * 1024u + lane * 16u), 0, 0, 0);
+        }
 
         // ---- multiply phase: 16 K steps of 32; operands of X two steps ahead, weight operands half a step ahead ----
-        if (multiplies) {
+        if (multiplies && !(flags & 16u)) {
             // scalar part of the X offsets: this column, this wave's four 16-row blocks; a K step is x_step further
             const uint32_t x_col = (((c_begin + ci) * 16u) * n_mblk + wave * 4u) * 1024u, x_step = n_mblk * 1024u;
-            const uint32_t x_lane = lane * 16u;
-            // weight operand of K step kb, rows 16 nb + li: piece (4 kb + quarter) ^ li = (quarter ^ li) ^ (kb << 2)
+            const uint32_t x_lane = lane_v * 16u;
+            // weight operand of K step kb, rows 16 nb + li: piece p = 4 kb + quarter at slot p ^ (p >> 4) ^ li, which is
+            // (quarter ^ li) ^ (kb << 2 | kb >> 2)
             const uint32_t bb = b_lane + ((quarter ^ li) << 4);
             u32x4 a[2][4], blo[4], bhi[4];
+            // (first all of step 0, then all of step 1: the order in which the loop below reloads them, so that
+            // "all but the newest four have arrived" is the wait in front of every step)
 #pragma unroll
-            for (int st = 0; st < 2; ++st)
+            for (int st = 0; st < 2; ++st) {
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
                     a[st][t] = __builtin_amdgcn_raw_buffer_load_b128(x_rs, (int)(x_lane + t * 1024), (int)(x_col + st * x_step), 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) blo[j] = lds_u128(bb + j * 16384u);
-#pragma unroll 1
-            for (uint32_t kp = 0; kp < 8; ++kp) {
+            // K step kb with the operands a[st]; `reload`: fetch the operands of step kb + 2 into a[st] afterwards
+            auto step = [&](uint32_t kb, int st, auto reload) {
+                const uint32_t kn = kb + 1u;
+                const uint32_t ba = bb ^ (((kb << 2) | (kb >> 2)) << 4), ba_next = bb ^ (((kn << 2) | ((kn >> 2) & 3u)) << 4);
 #pragma unroll
-                for (int st = 0; st < 2; ++st) {
-                    const uint32_t kb = kp * 2u + st;
-                    const uint32_t ba = bb ^ (kb << 6), ba_next = bb ^ ((kb + 1u) << 6);
+                for (int j = 0; j < 4; ++j) bhi[j] = lds_u128(ba + 65536u + j * 16384u);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) bhi[j] = lds_u128(ba + 65536u + j * 16384u);
-                    __builtin_amdgcn_sched_barrier(0);
+                for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
+                    for (int t = 0; t < 4; ++t)
+                        acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(q_bf16x8, a[st][t]),
+                                                                            __builtin_bit_cast(q_bf16x8, blo[j]), acc[t][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                // (after the last step this reads a neighbouring row's pieces, which nobody uses)
 #pragma unroll
-                        for (int t = 0; t < 4; ++t)
-                            acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(q_bf16x8, a[st][t]),
-                                                                                __builtin_bit_cast(q_bf16x8, blo[j]), acc[t][j], 0, 0, 0);
-                    __builtin_amdgcn_sched_barrier(0);
-                    // (after the last step this reads a neighbouring row's pieces, which nobody uses)
+                for (int j = 0; j < 4; ++j) blo[j] = lds_u128(ba_next + j * 16384u);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) blo[j] = lds_u128(ba_next + j * 16384u);
-                    __builtin_amdgcn_sched_barrier(0);
+                for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
+                    for (int t = 0; t < 4; ++t)
+                        acc[t][4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(q_bf16x8, a[st][t]),
+                                                                                __builtin_bit_cast(q_bf16x8, bhi[j]), acc[t][4 + j], 0, 0, 0);
+                if (decltype(reload)::value) {
 #pragma unroll
-                        for (int t = 0; t < 4; ++t)
-                            acc[t][4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(q_bf16x8, a[st][t]),
-                                                                                    __builtin_bit_cast(q_bf16x8, bhi[j]), acc[t][4 + j], 0, 0, 0);
-                    if (kp < 7) {
-#pragma unroll
-                        for (int t = 0; t < 4; ++t)
-                            a[st][t] = __builtin_amdgcn_raw_buffer_load_b128(x_rs, (int)(x_lane + t * 1024),
-                                                                             (int)(x_col + (kb + 2u) * x_step), 0);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
+                    for (int t = 0; t < 4; ++t)
+                        a[st][t] = __builtin_amdgcn_raw_buffer_load_b128(x_rs, (int)(x_lane + t * 1024),
+                                                                         (int)(x_col + (kb + 2u) * x_step), 0);
                 }
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            // no branch around the reloads inside the loop: with one, the compiler's count of what is in flight
+            // differs between the paths and it waits for everything, the operands just requested included
+#pragma unroll 1
+            for (uint32_t kp = 0; kp < 7; ++kp) {
+                step(kp * 2u, 0, QReload{});
+                step(kp * 2u + 1u, 1, QReload{});
             }
+            step(14u, 0, QLast{});
+            step(15u, 1, QLast{});
         }
     }
 
     // ---- partial sums of this K slice: ws[slice][m][n]; lane l holds rows 4 (l / 16) + r, column l % 16 of a block ----
-    if (multiplies) {
+    if (multiplies && !(flags & 8u)) {
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -443,7 +608,9 @@ static uint32_t q_mblocks(uint32_t m_rows) { return ((min(m_rows, kQMaxM) + 63u)
 
 size_t prefill358_workspace_bytes(const Dev &P, uint32_t m_rows) {
     const uint32_t mb = min(m_rows, kQMaxM);
-    return (size_t)kQMaxSlices * mb * P.out_f * sizeof(float) + (size_t)(P.in_f / 32u) * q_mblocks(mb) * 1024u;
+    const size_t tiles = (P.out_f + kQRows - 1) / kQRows;
+    return (size_t)kQMaxSlices * mb * P.out_f * sizeof(float) + (size_t)(P.in_f / 32u) * q_mblocks(mb) * 1024u +
+           tiles * kQMaxSlices * kQListBytes;
 }
 
 bool prefill358_supports(const Dev &P, const uint16_t *x, int64_t ldx) {
@@ -468,14 +635,15 @@ int launch_prefill358(const Dev &P, const int32_t *prefix, const uint16_t *x, ui
     const uint32_t tiles = (P.out_f + kQRows - 1) / kQRows;
     const uint32_t n_slices = q_pick_slices(tiles, n_chunks);
     if (n_slices == 0) return IXH_EUNSUPPORTED;
-    // workspace: the partial sums first, the re-tiled activations behind them
+    // workspace: the partial sums first, the re-tiled activations behind them, then the workgroups' value lists
     u32x4 *const xt = reinterpret_cast<u32x4 *>(ws + (size_t)kQMaxSlices * min(m_rows, kQMaxM) * P.out_f);
+    int8_t *const lists = reinterpret_cast<int8_t *>(xt) + (size_t)n_kb * q_mblocks(min(m_rows, kQMaxM)) * 1024u;
     for (uint32_t m0 = 0; m0 < m_rows; m0 += kQMaxM) {
         const uint32_t mb = min(kQMaxM, m_rows - m0), n_mblk = q_mblocks(mb);
         hipLaunchKernelGGL(k_prefill_xtile, dim3((n_kb / 2u) * (n_mblk / 2u)), dim3(256), 0, s, x + (int64_t)m0 * ldx, ldx, mb,
                            n_kb, n_mblk, xt);
         hipLaunchKernelGGL(k_prefill358, dim3(tiles * n_slices), dim3(kWave * kQWaves), kQLdsBytes, s, P, prefix, n_chunks,
-                           (const u32x4 *)xt, n_mblk, mb, ws, n_slices, flags);
+                           (const u32x4 *)xt, n_mblk, mb, ws, lists, n_slices, flags);
         if (hipGetLastError() != hipSuccess) return IXH_ELAUNCH;
         const int rc = launch_prefill_reduce(ws, mb, P.out_f, n_slices, y + (int64_t)m0 * ldy, ldy, s);
         if (rc) return rc;
