@@ -34,8 +34,8 @@
 // LDS by LDS-DMA (two stages per wave); the first two groups of a column are requested before the multiply phase of
 // the column before, the other two while the first two are decoded.
 //
-// Partial sums of the K slices go to an fp32 workspace [slice][m][n]; the reduction kernel of ixh_prefill.hip adds them
-// in slice order and rounds to bf16.
+// Partial sums of the K slices go to an fp32 workspace in accumulator order (whole 1 KB stores); a second kernel adds
+// them in slice order and rounds to bf16.
 #include "ixh_rows_common.h"
 
 namespace ixh {
@@ -207,10 +207,8 @@ k_prefill358(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const
     // The pair table is addressed with (index bits | lane bits), which needs it at LDS address 0 (the kernel has no
     // other LDS).  Should that ever not hold, say so in the output instead of computing garbage.
     if ((uint32_t)(uintptr_t)(lds_ptr_t)smem != 0) {
-        for (uint32_t i = tid; i < min(m_rows, kQMaxM) * kQRows; i += blockDim.x) {
-            const uint32_t m = i / kQRows, n = n0 + i % kQRows;
-            if (n < P.out_f) ws[((size_t)slice * m_rows + m) * P.out_f + n] = __uint_as_float(0x7FC00000u);
-        }
+        float *const mine = ws + ((size_t)slice * (gridDim.x / n_slices) + tile) * (kQMaxM * kQRows);
+        for (uint32_t i = tid; i < kQMaxM * kQRows; i += blockDim.x) mine[i] = __uint_as_float(0x7FC00000u);
         return;
     }
     uint32_t *const lut = reinterpret_cast<uint32_t *>(smem + kQLut);
@@ -568,19 +566,39 @@ k_prefill358(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const
         }
     }
 
-    // ---- partial sums of this K slice: ws[slice][m][n]; lane l holds rows 4 (l / 16) + r, column l % 16 of a block ----
-    if (multiplies && !(flags & 8u)) {
+    // ---- partial sums of this K slice, in accumulator order: [slice][tile][wave][t][j][lane] x 4 floats, so that a
+    // store instruction writes 1 KB of consecutive memory (lane l of block (t, j) holds rows 64 wave + 16 t + 4 (l / 16)
+    // + r, column 16 j + l % 16 of the tile) ----
+    if (multiplies) {
+        q_f32x4 *const dst = reinterpret_cast<q_f32x4 *>(ws) +
+                             ((((size_t)slice * (gridDim.x / n_slices) + tile) * kQWaves + wave) * 32u) * 64u + lane;
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const uint32_t m = 64 * wave + 16 * t + 4 * quarter + r;
-                    const uint32_t n = n0 + j * 16 + li;
-                    if (m < m_rows && n < P.out_f) ws[((size_t)slice * m_rows + m) * P.out_f + n] = acc[t][j][r];
-                }
+            for (int j = 0; j < 8; ++j) dst[(t * 8 + j) * 64] = acc[t][j];
     }
+}
+
+// y[m][n] = bf16(sum over the K slices, in slice order) from the partial sums in accumulator order; a thread takes one
+// lane's four floats of one block.
+__global__ void __launch_bounds__(256)
+k_prefill358_reduce(const q_f32x4 *__restrict__ ws, uint32_t m_rows, uint32_t out_f, uint32_t tiles, uint32_t n_slices,
+                    uint16_t *__restrict__ y, int64_t ldy) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;  // ((tile * 8 + wave) * 32 + t * 8 + j) * 64 + lane
+    const uint32_t lane = i & 63u, blk = (i >> 6) & 31u, wave = (i >> 11) & 7u, tile = i >> 14;
+    if (tile >= tiles) return;
+    const uint32_t m0 = 64u * wave + 16u * (blk >> 3) + 4u * (lane >> 4), n = tile * kQRows + 16u * (blk & 7u) + (lane & 15u);
+    if (m0 >= m_rows || n >= out_f) return;
+    const size_t per_slice = (size_t)tiles * kQWaves * 32u * 64u;
+    q_f32x4 sum = ws[i];
+    for (uint32_t sl = 1; sl < n_slices; ++sl) {
+        const q_f32x4 v = ws[sl * per_slice + i];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sum[r] += v[r];
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+        if (m0 + r < m_rows) y[(int64_t)(m0 + r) * ldy + n] = (uint16_t)f32_to_bf16_bits(sum[r]);
 }
 
 // K slices for a shape: one workgroup per CU; the count that makes rounds x (columns per workgroup + a start-up
@@ -604,13 +622,14 @@ static uint32_t q_pick_slices(uint32_t tiles, uint32_t n_chunks) {
     return best;
 }
 
+// partial sums of the most slices, whole tiles of 512 x 128
+static size_t q_sums_bytes(size_t tiles) { return (size_t)kQMaxSlices * tiles * kQMaxM * kQRows * sizeof(float); }
 static uint32_t q_mblocks(uint32_t m_rows) { return ((min(m_rows, kQMaxM) + 63u) / 64u) * 4u; }
 
 size_t prefill358_workspace_bytes(const Dev &P, uint32_t m_rows) {
     const uint32_t mb = min(m_rows, kQMaxM);
     const size_t tiles = (P.out_f + kQRows - 1) / kQRows;
-    return (size_t)kQMaxSlices * mb * P.out_f * sizeof(float) + (size_t)(P.in_f / 32u) * q_mblocks(mb) * 1024u +
-           tiles * kQMaxSlices * kQListBytes;
+    return q_sums_bytes(tiles) + (size_t)(P.in_f / 32u) * q_mblocks(mb) * 1024u + tiles * kQMaxSlices * kQListBytes;
 }
 
 bool prefill358_supports(const Dev &P, const uint16_t *x, int64_t ldx) {
@@ -636,7 +655,7 @@ int launch_prefill358(const Dev &P, const int32_t *prefix, const uint16_t *x, ui
     const uint32_t n_slices = q_pick_slices(tiles, n_chunks);
     if (n_slices == 0) return IXH_EUNSUPPORTED;
     // workspace: the partial sums first, the re-tiled activations behind them, then the workgroups' value lists
-    u32x4 *const xt = reinterpret_cast<u32x4 *>(ws + (size_t)kQMaxSlices * min(m_rows, kQMaxM) * P.out_f);
+    u32x4 *const xt = reinterpret_cast<u32x4 *>(reinterpret_cast<uint8_t *>(ws) + q_sums_bytes(tiles));
     int8_t *const lists = reinterpret_cast<int8_t *>(xt) + (size_t)n_kb * q_mblocks(min(m_rows, kQMaxM)) * 1024u;
     for (uint32_t m0 = 0; m0 < m_rows; m0 += kQMaxM) {
         const uint32_t mb = min(kQMaxM, m_rows - m0), n_mblk = q_mblocks(mb);
@@ -645,8 +664,9 @@ int launch_prefill358(const Dev &P, const int32_t *prefix, const uint16_t *x, ui
         hipLaunchKernelGGL(k_prefill358, dim3(tiles * n_slices), dim3(kWave * kQWaves), kQLdsBytes, s, P, prefix, n_chunks,
                            (const u32x4 *)xt, n_mblk, mb, ws, lists, n_slices, flags);
         if (hipGetLastError() != hipSuccess) return IXH_ELAUNCH;
-        const int rc = launch_prefill_reduce(ws, mb, P.out_f, n_slices, y + (int64_t)m0 * ldy, ldy, s);
-        if (rc) return rc;
+        hipLaunchKernelGGL(k_prefill358_reduce, dim3(tiles * 64u), dim3(256), 0, s, (const q_f32x4 *)ws, mb, P.out_f, tiles,
+                           n_slices, y + (int64_t)m0 * ldy, ldy);
+        if (hipGetLastError() != hipSuccess) return IXH_ELAUNCH;
     }
     return IXH_OK;
 }
