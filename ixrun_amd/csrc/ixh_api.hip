@@ -136,7 +136,7 @@ int ixh_set_option(const char *name, int64_t value) {
         return IXH_OK;
     }
     if (strcmp(name, "gemm_tiles") == 0) {
-        if (value < -1 || value > 4096) { set_error("gemm_tiles %lld not in -1..2", (long long)value); return IXH_EINVAL; }
+        if (value < -1 || value > 2) { set_error("gemm_tiles %lld not in -1..2", (long long)value); return IXH_EINVAL; }
         g_opt_gemm_tiles.store((int)value, std::memory_order_relaxed);
         return IXH_OK;
     }
@@ -449,13 +449,15 @@ size_t ixh_gemm_workspace_bytes(const IxhPacked *packed, int32_t m) {
 }
 
 // The kernel of ixh_prefill358.hip: tensors that are almost all level 1 (the full decode of such tensors and the
-// products of few activation rows switch at the same share), enough activation rows to fill its 64-row wave tiles.
+// products of few activation rows switch at the same share) and large enough to give most CUs a 128-row tile and a
+// few unit columns; measured against k_prefill on 4096 x 4096 ... 8192 x 28672, 32 ... 2048 activation rows: ahead
+// everywhere above 2^24 elements, at 2^24 from 512 rows on, behind below.
 static bool gemm_takes_tiles(const Dev &d, const uint16_t *x, int64_t ldx, int32_t m, const void *workspace) {
     const int want = g_opt_gemm_tiles.load(std::memory_order_relaxed);
     if (want < 0 || !prefill358_supports(d, x, ldx) || ((uintptr_t)workspace & 15u) != 0) return false;
     if (want > 0) return true;
     const bool mostly_l1 = (uint64_t)d.st_words[0] * 32u / 3u >= (uint64_t)d.n / 100u * 97u;
-    return mostly_l1 && m >= 96;
+    return mostly_l1 && (d.n > (1u << 24) || (d.n == (1u << 24) && m >= 512));
 }
 
 int ixh_gemm(const IxhPacked *packed, const int32_t *prefix, const uint16_t *x, int32_t m, int64_t ldx, uint16_t *y,
@@ -485,7 +487,7 @@ int ixh_gemm(const IxhPacked *packed, const int32_t *prefix, const uint16_t *x, 
     }
     if (tiles)
         rc = launch_prefill358(d, prefix, x, (uint32_t)m, ldx, y, ldy, (float *)workspace,
-                               g_opt_gemm_tiles.load(std::memory_order_relaxed) == 2 ? 1u : (uint32_t)(max(0, g_opt_gemm_tiles.load(std::memory_order_relaxed)) >> 4), (hipStream_t)stream);
+                               g_opt_gemm_tiles.load(std::memory_order_relaxed) == 2 ? 1u : 0u, (hipStream_t)stream);
     else
         rc = launch_prefill(d, prefix, x, (uint32_t)m, ldx, y, ldy, (float *)workspace, (hipStream_t)stream);
     if (rc == IXH_ELAUNCH) set_error("gemm: launch failed");

@@ -398,20 +398,19 @@ k_prefill358(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const
     const __amdgpu_buffer_rsrc_t list_rs =
         __builtin_amdgcn_make_buffer_rsrc((void *)my_lists, 0, (int)kQListBytes, 0x00020000);
     for (uint32_t ci = 0; ci < cols; ++ci) {
-        // What this wave asked for has arrived (groups 0 and 1 of this column; from waves 0 and 1 the column's value
-        // list, and at the first column the stores of the lists), then: the multiply phase of the column before is
-        // done with the weight tile, and the list and the rows' counts of this column are in LDS.
+        // What this wave asked for has arrived: groups 0 and 1 of this column; from waves 0 and 1 the column's value
+        // list; at the first column the stores of the lists.
         q_wait_vmem<0>();
-        q_barrier_lds();
         asm volatile("" : "+v"(lane_v));
         quarter = lane_v >> 4, li = lane_v & 15u;
         lut_lane = li << 2;
         b_lane = kQTile + li * 1024u;  // weight operand: row 16 nb + li, piece 4 kb + quarter
-        const bool listed = lds_u16(kQRowBase + (ci & 1u) * 264u + kQRows * 2u) <= kQValueCap && !(flags & 1u);
-        // the next column's counts, while none of this wave's copies is in flight
+        // the next column's counts, while none of this wave's copies is in flight (the buffer they go to was last read
+        // in the decode phase of the column before)
         if (wave == 0 && ci + 1 < cols) scan_column(ci + 1, nullptr, rowbase + ((ci + 1) & 1u) * 132u);
         // ---- decode phase: this wave's 16 row units, four at a time, two groups of four in lockstep ----
         Window A, B;
+        bool listed = false;  // this column has its value list in LDS (set behind the barrier)
         auto lut_addresses = [&](const Window &W, uint32_t (&la)[16]) {
 #pragma unroll
             for (int t = 0; t < 16; ++t) {
@@ -449,23 +448,24 @@ k_prefill358(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const
                 ++nth;
             }
         };
-        // groups i and i + 1 into the weight tile, in lockstep
-        auto emit_pair = [&](uint32_t i) {
-            uint32_t wa[16], wb[16];  // table addresses, then the pairs read from them
-            int va, vb;
+        // groups i and i + 1, in lockstep: the pairs of dequantised weights from the table, then into the weight tile
+        uint32_t wa[16], wb[16];  // table addresses, then the pairs read from them
+        auto look_up_pair = [&]() {
             lut_addresses(A, wa);
             lut_addresses(B, wb);
             q_issue8(wa, 0);
             q_issue8(wa, 1);
             q_issue8(wb, 0);
             q_issue8(wb, 1);
+            q_release16(wa);
+            q_release16(wb);
+        };
+        auto store_pair = [&](uint32_t i) {
+            int va, vb;
             // (a lane without such elements reads a neighbour's value, or a byte behind the list, and drops it; a
             // column without a list has indices beyond it)
             q_issue_i8(kQValues + min(A.esc, kQValueCap), va);
             q_issue_i8(kQValues + min(B.esc, kQValueCap), vb);
-            q_release16(wa);
-            q_release16(wb);
-            q_release2(va, vb);
             const uint32_t rl_a = row_of(i), rl_b = row_of(i + 1);
 #pragma unroll
             for (uint32_t j = 0; j < 4; ++j)
@@ -473,17 +473,21 @@ k_prefill358(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const
 #pragma unroll
             for (uint32_t j = 0; j < 4; ++j)
                 q_store128(q_tile_addr(rl_b, 4 * li + j), wb[4 * j], wb[4 * j + 1], wb[4 * j + 2], wb[4 * j + 3]);
+            q_release2(va, vb);
             patch(i, A, va);
             patch(i + 1, B, vb);
         };
-        if (!(flags & 2u)) {
         // Groups 0 and 1 are in the ring: opening their windows frees the two stages for groups 2 and 3, whose copies
-        // then run under the table look-ups and tile stores of groups 0 and 1.
+        // then run under the table look-ups and tile stores of groups 0 and 1.  Everything up to the first store into
+        // the weight tile is done in front of the barrier: a wave that leaves the multiply phase early uses the wait.
         open_pair(0, ci, A, B);
         q_wait_lds();
         issue(2, ci);
         issue(3, ci);
-        emit_pair(0);
+        look_up_pair();
+        q_barrier_lds();  // the multiply phase of the column before is done with the weight tile; this column's list is in LDS
+        listed = lds_u16(kQRowBase + (ci & 1u) * 264u + kQRows * 2u) <= kQValueCap && !(flags & 1u);
+        store_pair(0);
         q_wait_vmem<0>();  // groups 2 and 3 have landed
         open_pair(2, ci, A, B);
         // the first two groups of the next column, to land during the multiply phase
@@ -492,7 +496,22 @@ k_prefill358(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const
             issue(0, ci + 1);
             issue(1, ci + 1);
         }
-        emit_pair(2);
+        look_up_pair();
+        store_pair(2);
+        // the activation operands of the first two K steps, requested in front of the barrier
+        const uint32_t x_col = (((c_begin + ci) * 16u) * n_mblk + wave * 4u) * 1024u, x_step = n_mblk * 1024u;
+        const uint32_t x_lane = lane_v * 16u;
+        u32x4 a[2][4];
+        if (multiplies) {
+            // (first all of step 0, then all of step 1: the order in which the loop below reloads them, so that
+            // "all but the newest four have arrived" is the wait in front of every step)
+#pragma unroll
+            for (int st = 0; st < 2; ++st) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    a[st][t] = __builtin_amdgcn_raw_buffer_load_b128(x_rs, (int)(x_lane + t * 1024), (int)(x_col + st * x_step), 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         q_barrier_lds();  // weight tile complete; nobody reads this column's counts and list any more
         if (ci + 1 < cols) {
@@ -503,23 +522,11 @@ k_prefill358(Dev P, const int32_t *__restrict__ prefix, uint32_t n_chunks, const
         }
 
         // ---- multiply phase: 16 K steps of 32; operands of X two steps ahead, weight operands half a step ahead ----
-        if (multiplies && !(flags & 16u)) {
-            // scalar part of the X offsets: this column, this wave's four 16-row blocks; a K step is x_step further
-            const uint32_t x_col = (((c_begin + ci) * 16u) * n_mblk + wave * 4u) * 1024u, x_step = n_mblk * 1024u;
-            const uint32_t x_lane = lane_v * 16u;
+        if (multiplies) {
             // weight operand of K step kb, rows 16 nb + li: piece p = 4 kb + quarter at slot p ^ (p >> 4) ^ li, which is
             // (quarter ^ li) ^ (kb << 2 | kb >> 2)
             const uint32_t bb = b_lane + ((quarter ^ li) << 4);
-            u32x4 a[2][4], blo[4], bhi[4];
-            // (first all of step 0, then all of step 1: the order in which the loop below reloads them, so that
-            // "all but the newest four have arrived" is the wait in front of every step)
-#pragma unroll
-            for (int st = 0; st < 2; ++st) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    a[st][t] = __builtin_amdgcn_raw_buffer_load_b128(x_rs, (int)(x_lane + t * 1024), (int)(x_col + st * x_step), 0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
+            u32x4 blo[4], bhi[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) blo[j] = lds_u128(bb + j * 16384u);
             // K step kb with the operands a[st]; `reload`: fetch the operands of step kb + 2 into a[st] afterwards
