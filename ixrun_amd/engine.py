@@ -123,6 +123,18 @@ class StreamingLinear(nn.Module):
         # the shared scratch takes its final size now, not inside some later forward (or graph capture)
         shared_workspace(self._scale.device, self._dp.gemv_workspace_bytes(self._unit, MAX_FUSED_ROWS))
 
+    def _fused_gemm_wins(self, rows: int) -> bool:
+        """Whether ``ixh_gemm`` beats decode + library GEMM when a decode buffer is at hand.
+
+        Only its 128-row tile kernel does (3-bit first level, at least 97 % of the elements there, more
+        than 2**24 elements), and only up to 512 activation rows, beyond which it decodes the weight once
+        per 512 rows.  Measured on MI355X against the tuned library GEMM, 5120 x 17408: 82 / 98 / 113 us
+        against 120 / 131 / 144 us at 128 / 256 / 512 rows; 4096 x 14336: 92 / 95 / 121 against
+        105 / 113 / 142; 17408 x 5120: 82 / 95 / 142 against 80 / 96 / 126, which is why layers with more
+        outputs than inputs go back to the library from 257 rows on."""
+        return (self.level_bits[0] == 3 and self.N > (1 << 24) and self.counts[0] * 100 >= self.N * 97
+                and (rows <= 256 or (rows <= 512 and self.in_features >= self.out_features)))
+
     def _bind(self):
         n_levels = len(self.level_bits)
         self._dp = _lib.DevicePacked(
@@ -211,7 +223,8 @@ class StreamingLinear(nn.Module):
                 return y
         rows = x.numel() // in_f if in_f else 0
         if (self._use_fused and self._gemm_ok and x.dtype == torch.bfloat16 and x.is_cuda and rows > MAX_FUSED_ROWS
-                and x.shape[-1] == self.in_features and self._unit == 512 and self._w_buf is None):
+                and x.shape[-1] == self.in_features and self._unit == 512
+                and (self._w_buf is None or self._fused_gemm_wins(rows))):
             # many rows: decode tiles on chip straight into the matrix-core GEMM, no bf16 weight in HBM
             x2 = x.reshape(rows, self.in_features)
             if x2.stride(1) != 1:
