@@ -38,13 +38,13 @@ _ROWS = ("ixh_rows358.hip", "ixh_rows_common.h", "ixh_dev.h", "build.sh")
 _TILES = ("ixh_tiles358.hip", "ixh_rows_common.h", "ixh_dev.h")
 _DENSE = ("ixh_dense358.hip", "ixh_dense_tiles.h", "ixh_dev.h")
 _DENSE5 = ("ixh_dense5.hip", "ixh_dense_tiles.h", "ixh_dev.h")
-_PREFILL = ("ixh_prefill.hip", "ixh_staged.h", "ixh_dev.h")
+_PREFILL = ("ixh_prefill358.hip", "ixh_prefill358.h", "ixh_rows_common.h", "ixh_dev.h")
 _DECODE_ROWS = ("ixh_decode_rows358.hip", "ixh_rows_common.h", "ixh_dev.h")
 _OLD = ((), "measured-on-earlier-sources")  # figures kept for the record; reported as null
 MEASURED_TRAFFIC_BYTES = {
-    "down_proj_5120x17408_m1_student_t": (23032.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "5ccd2523b03e02ca"),
-    "gate_up_17408x5120_m1_student_t": (22936.0 * 2.0 * 1024 + 40.0 * 1024, _ROWS, "5ccd2523b03e02ca"),
-    "attn_proj_5120x5120_m1_student_t": (7135.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "5ccd2523b03e02ca"),
+    "down_proj_5120x17408_m1_student_t": (23032.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "3e8407b518bc293b"),
+    "gate_up_17408x5120_m1_student_t": (22936.0 * 2.0 * 1024 + 40.0 * 1024, _ROWS, "3e8407b518bc293b"),
+    "attn_proj_5120x5120_m1_student_t": (7135.0 * 2.0 * 1024 + 16.0 * 1024, _ROWS, "3e8407b518bc293b"),
     "down_proj_5120x17408_m1_calibrated": (33825.0 * 2.0 * 1024 + 40.0 * 1024, _DENSE, "711eef94d053feb1"),
     "down_proj_5120x17408_m1_five_level_calibrated": (49708.0 * 2.0 * 1024 + 1338.0 * 1024, _DENSE5, "aaca19573f1ed2a1"),
     "gate_up_17408x5120_m4_student_t": (28740.0 * 2.0 * 1024 + 160.0 * 1024, _TILES, "21f9d013a3b417ff"),
@@ -53,8 +53,9 @@ MEASURED_TRAFFIC_BYTES = {
     "down_proj_5120x17408_m16_student_t": (27677.0 * 2.0 * 1024 + 960.0 * 1024, _TILES, "21f9d013a3b417ff"),
     "decode_5120x17408_five_level_calibrated": (49719.0 * 2.0 * 1024 + 174080.0 * 1024, _DENSE5, "aaca19573f1ed2a1"),
     "prefill_5120x5120_m512_five_level": (50297.9 * 2.0 * 1024 + 30720.0 * 1024,) + _OLD,
-    # both kernels of a step: k_prefill<5> + k_prefill_reduce
-    "prefill_5120x17408_m512_five_level": ((190401.0 + 15378.0) * 2.0 * 1024 + (30720.0 + 5120.0) * 1024, _PREFILL, "17fc44b7da55ae09"),
+    # the three kernels of a step: k_prefill_xtile + k_prefill358 + k_prefill358_reduce
+    "prefill_5120x17408_m512_five_level": ((8716.0 + 68452.0 + 30734.0) * 2.0 * 1024 + (17408.0 + 61606.0 + 5120.0) * 1024,
+                                           _PREFILL, "55862ec6d8c72acd"),
     # k_decode358_rows<true> (x 2.0 / x 1.0 as above) + the operands and outputs of the library GEMM that
     # torch.cuda.tunable picked (bf16 weight, X, Y: its FETCH_SIZE, 158,001, is weighted for other request sizes than
     # our kernels' and fixes its reads only between 162 and 324 MB)
@@ -72,10 +73,10 @@ MEASURED_TRAFFIC_BYTES = {
 # rocprofv3 --pmc run of this script, mean over the launches), gated by the hash of the kernel's sources like the
 # traffic figures.  Reported per weight: vector and LDS instructions x 64 lanes / weights, scalar instructions / weights.
 MEASURED_INSTRUCTIONS = {
-    "down_proj_5120x17408_m1_student_t": ((5734195.0, 4469166.0, 1360042.0), _ROWS, "5ccd2523b03e02ca"),
-    "gate_up_17408x5120_m1_student_t": ((6030194.0, 4450915.0, 1414314.0), _ROWS, "5ccd2523b03e02ca"),
-    "attn_proj_5120x5120_m1_student_t": ((3570752.0, 2281697.0, 593732.0), _ROWS, "5ccd2523b03e02ca"),
-    "down_proj_5120x17408_m1_level1_only": ((4881551.0, 4104235.0, 1254926.0), _ROWS, "5ccd2523b03e02ca"),
+    "down_proj_5120x17408_m1_student_t": ((5734195.0, 4469166.0, 1360042.0), _ROWS, "3e8407b518bc293b"),
+    "gate_up_17408x5120_m1_student_t": ((6030194.0, 4450915.0, 1414314.0), _ROWS, "3e8407b518bc293b"),
+    "attn_proj_5120x5120_m1_student_t": ((3570752.0, 2281697.0, 593732.0), _ROWS, "3e8407b518bc293b"),
+    "down_proj_5120x17408_m1_level1_only": ((4881551.0, 4104235.0, 1254926.0), _ROWS, "3e8407b518bc293b"),
 }
 
 WORKLOADS = {

@@ -10,6 +10,7 @@
 #include "../../include/ixhip_test.h"
 #include "ixh_dev.h"
 #include "ixh_fast358.h"
+#include "ixh_prefill358.h"
 
 namespace ixh {
 

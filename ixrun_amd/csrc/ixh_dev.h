@@ -131,14 +131,6 @@ size_t prefill_workspace_bytes(const Dev &P, uint32_t m_rows);
 bool prefill_supports(const Dev &P, const uint16_t *x, int64_t ldx);
 int launch_prefill(const Dev &P, const int32_t *prefix, const uint16_t *x, uint32_t m_rows, int64_t ldx, uint16_t *y,
                    int64_t ldy, float *ws, hipStream_t s);
-int launch_prefill_reduce(const float *ws, uint32_t m_rows, uint32_t out_f, uint32_t n_slices, uint16_t *y, int64_t ldy,
-                          hipStream_t s);
-// the 128-row tile kernel for tensors that are almost all level 1 with a 3-bit first level (ixh_prefill358.hip);
-// flags & 1: compute every element above level 1 where it is needed instead of listing them first (testing)
-size_t prefill358_workspace_bytes(const Dev &P, uint32_t m_rows);
-bool prefill358_supports(const Dev &P, const uint16_t *x, int64_t ldx);
-int launch_prefill358(const Dev &P, const int32_t *prefix, const uint16_t *x, uint32_t m_rows, int64_t ldx, uint16_t *y,
-                      int64_t ldy, float *ws, uint32_t flags, hipStream_t s);
 size_t encode_workspace_bytes(uint64_t n, int n_levels);
 int launch_encode_scan(const uint16_t *w, uint32_t n, int n_levels, const int *bits, uint16_t *scale, int32_t *table,
                        void *workspace, hipStream_t s);
@@ -151,7 +143,6 @@ enum DecodeKernel : int { kDecodeAuto = 0, kDecodeRows = 1, kDecodeDense = 2, kD
 extern std::atomic<int> g_opt_decode_kernel;   // a DecodeKernel
 extern std::atomic<int> g_opt_gemv_shared_x;   // most activation rows the shared-x row-block kernel serves (0..8)
 extern std::atomic<int> g_opt_gemv_tiles;      // the tile kernel: -1 = never, 0 = where it pays, 1 = wherever it fits
-extern std::atomic<int> g_opt_gemm_tiles;       // the 128-row tile kernel of ixh_gemm: -1 = never, 0 = where it pays, 1 = wherever it fits, 2 = as 1, no value list
 extern std::atomic<int> g_opt_gemv_strips;     // the strip kernel: -1 = never, 0 = where it fits, 1..6 = with that many chains
 
 }  // namespace ixh

@@ -16,6 +16,7 @@
 // 64 k ahead of the MFMAs.  Partial sums of the K slices go to an fp32 workspace
 // [slice][m][n]; a second kernel adds them in slice order and rounds to bf16.  The number
 // of K slices is chosen per shape so that the workgroups fill the CUs in whole rounds.
+#include "ixh_prefill358.h"
 #include "ixh_staged.h"
 
 namespace ixh {

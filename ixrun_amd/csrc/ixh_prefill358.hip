@@ -36,6 +36,7 @@
 //
 // Partial sums of the K slices go to an fp32 workspace in accumulator order (whole 1 KB stores); a second kernel adds
 // them in slice order and rounds to bf16.
+#include "ixh_prefill358.h"
 #include "ixh_rows_common.h"
 
 namespace ixh {

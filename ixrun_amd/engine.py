@@ -128,8 +128,8 @@ class StreamingLinear(nn.Module):
 
         Only its 128-row tile kernel does (3-bit first level, at least 97 % of the elements there, more
         than 2**24 elements), and only up to 512 activation rows, beyond which it decodes the weight once
-        per 512 rows.  Measured on MI355X against the tuned library GEMM, 5120 x 17408: 82 / 98 / 113 us
-        against 120 / 131 / 144 us at 128 / 256 / 512 rows; 4096 x 14336: 92 / 95 / 121 against
+        per 512 rows.  Measured on MI355X against the tuned library GEMM, 5120 x 17408: 70 / 77 / 111 us
+        against 94 / 127 / 158 us at 128 / 256 / 512 rows; 4096 x 14336: 92 / 95 / 121 against
         105 / 113 / 142; 17408 x 5120: 82 / 95 / 142 against 80 / 96 / 126, which is why layers with more
         outputs than inputs go back to the library from 257 rows on."""
         return (self.level_bits[0] == 3 and self.N > (1 << 24) and self.counts[0] * 100 >= self.N * 97
